@@ -1,0 +1,131 @@
+"""Eager-PyTorch implementation of the operator primitives (host plumbing only).
+
+Each primitive states the formula of the native call it stands in for; the HIP
+backend implements the same contracts on the device.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+
+class EagerBackend:
+    name = "eager"
+
+    # y = x . W^T, dx = dy . W, dW = dy^T . x   (reference call sites:
+    # kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:571-582, 847-859, 898-909)
+    def linear_fwd(self, x: Tensor, w: Tensor) -> Tensor:
+        return x @ w.t()
+
+    def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
+        return dy @ w
+
+    def linear_wgrad(self, dy: Tensor, x: Tensor) -> Tensor:
+        return dy.t() @ x
+
+    # rs = rsqrt(mean(x^2) + eps) in fp32, y = (x * rs) * gamma
+    # (3rdparty/TransformerEngine/transformer_engine/common/normalization/rmsnorm/
+    #  rmsnorm_fwd_kernels.cuh:90-121)
+    def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+        xf = x.float()
+        rstd = torch.rsqrt(xf.pow(2).mean(dim=-1) + eps)
+        y = (xf * rstd[:, None]) * gamma.float()
+        return y.to(x.dtype), rstd
+
+    # dx = rs * (g - xhat * mean(g * xhat)), g = gamma * dy ; dgamma = sum_rows dy * xhat
+    # (rmsnorm_bwd_kernels.cuh:95-128)
+    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor) -> Tuple[Tensor, Tensor]:
+        xhat = x.float() * rstd[:, None]
+        dyf = dy.float()
+        g = dyf * gamma.float()
+        dx = rstd[:, None] * (g - xhat * (g * xhat).mean(dim=-1, keepdim=True))
+        dgamma = (dyf * xhat).sum(dim=0)
+        return dx.to(x.dtype), dgamma.to(gamma.dtype)
+
+    # y = t cos f + rotate_half(t) sin f, rotate_half([a, b]) = [-b, a]; trig in fp32
+    # (kareus/megatron/core/models/common/embedding/rope_utils.py:147-182)
+    @staticmethod
+    def _rope(t: Tensor, freqs: Tensor, sign: float) -> Tensor:
+        rot = freqs.shape[-1]
+        cos, sin = torch.cos(freqs.float()), torch.sin(freqs.float()) * sign
+        tr = t[..., :rot].float()
+        a, b = tr.chunk(2, dim=-1)
+        out = tr * cos + torch.cat((-b, a), dim=-1) * sin
+        if rot < t.shape[-1]:
+            out = torch.cat((out, t[..., rot:].float()), dim=-1)
+        return out.to(t.dtype)
+
+    def rope_fwd(self, t: Tensor, freqs: Tensor) -> Tensor:
+        return self._rope(t, freqs, 1.0)
+
+    # The gradient of a rotation is the rotation by the opposite angle (rope_utils.py:207-222).
+    def rope_bwd(self, g: Tensor, freqs: Tensor) -> Tensor:
+        return self._rope(g, freqs, -1.0)
+
+    # y = silu(x1) * x2 with x1, x2 = chunk(x, 2, -1)
+    # (kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20, 34-44)
+    def swiglu_fwd(self, x: Tensor) -> Tensor:
+        x1, x2 = x.float().chunk(2, dim=-1)
+        return (torch.nn.functional.silu(x1) * x2).to(x.dtype)
+
+    def swiglu_bwd(self, dy: Tensor, x: Tensor) -> Tensor:
+        x1, x2 = x.float().chunk(2, dim=-1)
+        g = dy.float()
+        sig = torch.sigmoid(x1)
+        d1 = g * sig * (1 + x1 * (1 - sig)) * x2
+        d2 = g * x1 * sig
+        return torch.cat((d1, d2), dim=-1).to(x.dtype)
+
+    def add(self, a: Tensor, b: Tensor) -> Tensor:
+        return a + b
+
+    # Causal GQA attention on [s, b, heads, hd] tensors; query head i reads KV head
+    # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32
+    # (kareus/flash_attn/flash_attn_interface.py:473-493).
+    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
+        s, b, nq, hd = q.shape
+        nkv = k.shape[2]
+        rep = nq // nkv
+        qf = q.float().permute(1, 2, 0, 3)
+        kf = k.float().permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+        vf = v.float().permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+        scores = (qf @ kf.transpose(-1, -2)) * scale
+        if causal:
+            mask = torch.ones(s, s, dtype=torch.bool, device=q.device).tril()
+            scores = scores.masked_fill(~mask, float("-inf"))
+        lse = torch.logsumexp(scores, dim=-1)
+        p = torch.exp(scores - lse[..., None])
+        o = (p @ vf).permute(2, 0, 1, 3).contiguous()
+        return o.to(q.dtype), lse.contiguous()
+
+    def attn_bwd(self, do, q, k, v, o, lse, scale: float, causal: bool = True):
+        s, b, nq, hd = q.shape
+        nkv = k.shape[2]
+        rep = nq // nkv
+        qf = q.float().permute(1, 2, 0, 3)
+        kf = k.float().permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+        vf = v.float().permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+        dof = do.float().reshape(s, b, nq, hd).permute(1, 2, 0, 3)
+        of = o.float().reshape(s, b, nq, hd).permute(1, 2, 0, 3)
+        scores = (qf @ kf.transpose(-1, -2)) * scale
+        if causal:
+            mask = torch.ones(s, s, dtype=torch.bool, device=q.device).tril()
+            scores = scores.masked_fill(~mask, float("-inf"))
+        p = torch.exp(scores - lse[..., None])
+        dv = p.transpose(-1, -2) @ dof
+        dp = dof @ vf.transpose(-1, -2)
+        delta = (dof * of).sum(dim=-1, keepdim=True)
+        ds = p * (dp - delta) * scale
+        dq = ds @ kf
+        dk = ds.transpose(-1, -2) @ qf
+        dk = dk.reshape(b, nkv, rep, s, hd).sum(dim=2)
+        dv = dv.reshape(b, nkv, rep, s, hd).sum(dim=2)
+        back = lambda t: t.permute(2, 0, 1, 3).contiguous()
+        return back(dq).to(q.dtype), back(dk).to(k.dtype), back(dv).to(v.dtype)
+
+    def default_scale(self, hd: int) -> float:
+        return 1.0 / math.sqrt(hd)

@@ -1,0 +1,183 @@
+"""ORACLE — test infrastructure, not product code.
+
+A plain-PyTorch restatement of one GPU's shard of a Llama-style decoder layer, not
+nanobatched, with gradients from autograd.  It restates the arithmetic the
+reference reaches through third-party CUDA libraries, function by function:
+
+  rmsnorm        3rdparty/TransformerEngine/transformer_engine/common/normalization/rmsnorm/
+                 rmsnorm_fwd_kernels.cuh:90-121 (rs = rsqrt(mean(x^2)+eps), y = x*rs*gamma);
+                 backward formula rmsnorm_bwd_kernels.cuh:95-128 — here left to autograd and
+                 stated separately in ``rmsnorm_bwd_formula`` so tests can cross-check the two
+  linear         kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:571-582 (y = x W^T)
+  split_qkv      kareus/megatron/core/extensions/ops/qkv_postprocess.py:84-109
+  rope           kareus/megatron/core/models/common/embedding/rope_utils.py:147-182 with the
+                 table of 3rdparty/Megatron-LM/megatron/core/models/common/embeddings/
+                 rotary_pos_embedding.py:76-78,129,161,167
+  attention      kareus/flash_attn/flash_attn_interface.py:473-493 (semantics of the external
+                 flash-attention call: scale, causal mask, GQA head map); the un-fused
+                 statement 3rdparty/TransformerEngine/transformer_engine/pytorch/attention/
+                 dot_product_attention/backends.py:242-251, 304-347
+  swiglu         kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20; backward formula
+                 :34-44 restated in ``swiglu_bwd_formula``
+  residual adds  kareus/megatron/core/extensions/ops/bias_dropout_add.py:24-45 with p = 0, no bias
+  layer order    kareus/megatron/core/transformer/transformer_layer.py:148-174
+
+The external pieces (flash-attention 2, Apex fused RoPE, cuBLASLt, Inductor output) are not
+in the reference tree and the reference holds no golden tensors for this path, so every
+function here is pinned by mathematics instead (tests/test_oracle.py): closed forms,
+invariants, brute-force loops on tiny inputs and PyTorch library routines
+(``F.scaled_dot_product_attention``, ``F.rms_norm``, ``F.silu``, ``torch.logsumexp``).
+
+Everything runs in the dtype of its inputs (fp32 or fp64); bf16 comparisons first round the
+inputs to bf16 and then call this in fp32.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+
+@dataclass
+class LayerDims:
+    hidden: int
+    nq: int
+    nkv: int
+    hd: int
+    ffn: int
+    eps: float = 1e-5
+    rope_base: float = 500000.0
+
+    @property
+    def qkv_width(self) -> int:
+        return (self.nq + 2 * self.nkv) * self.hd
+
+
+# --------------------------------------------------------------------------- ops
+def rmsnorm(x: Tensor, gamma: Tensor, eps: float) -> Tensor:
+    rs = torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return x * rs * gamma
+
+
+def rmsnorm_bwd_formula(dy: Tensor, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+    """dx = rs (g - xhat mean(g xhat)), g = gamma dy;  dgamma = sum over rows of dy xhat."""
+    rs = torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+    xhat = x * rs
+    g = dy * gamma
+    dx = rs * (g - xhat * (g * xhat).mean(dim=-1, keepdim=True))
+    dgamma = (dy * xhat).reshape(-1, x.shape[-1]).sum(dim=0)
+    return dx, dgamma
+
+
+def linear(x: Tensor, w: Tensor) -> Tensor:
+    return torch.matmul(x, w.t())
+
+
+def split_qkv(mixed: Tensor, nq: int, nkv: int, hd: int) -> Tuple[Tensor, Tensor, Tensor]:
+    """[..., nkv*(nq/nkv+2)*hd] -> q [..., nq, hd], k, v [..., nkv, hd]; features are laid out
+    per KV group as (its query heads, its key head, its value head)."""
+    per = nq // nkv
+    g = mixed.reshape(*mixed.shape[:-1], nkv, (per + 2) * hd)
+    q = g[..., : per * hd].reshape(*mixed.shape[:-1], nq, hd)
+    k = g[..., per * hd : (per + 1) * hd]
+    v = g[..., (per + 1) * hd :]
+    return q, k, v
+
+
+def rope_table(seq_len: int, dim: int, base: float, dtype=torch.float32) -> Tensor:
+    """[s, 1, 1, dim]: angle(pos, i) = pos * base^(-2i/dim) for i < dim/2, repeated twice."""
+    inv = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=dtype) / dim))
+    ang = torch.outer(torch.arange(seq_len, dtype=dtype), inv)
+    return torch.cat((ang, ang), dim=-1)[:, None, None, :]
+
+
+def rope(t: Tensor, freqs: Tensor) -> Tensor:
+    """t [s, b, heads, hd]; y = t cos f + rotate_half(t) sin f, rotate_half([a, b]) = [-b, a]."""
+    f = freqs.to(t.dtype)
+    a, b = t.chunk(2, dim=-1)
+    return t * torch.cos(f) + torch.cat((-b, a), dim=-1) * torch.sin(f)
+
+
+def causal_gqa_attention(q: Tensor, k: Tensor, v: Tensor, scale: Optional[float] = None,
+                         return_lse: bool = False):
+    """q [s, b, nq, hd], k/v [s, b, nkv, hd] -> [s, b, nq, hd] (and lse [b, nq, s])."""
+    s, b, nq, hd = q.shape
+    rep = nq // k.shape[2]
+    scale = 1.0 / math.sqrt(hd) if scale is None else scale
+    qh = q.permute(1, 2, 0, 3)
+    kh = k.permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+    vh = v.permute(1, 2, 0, 3).repeat_interleave(rep, dim=1)
+    scores = torch.matmul(qh, kh.transpose(-1, -2)) * scale
+    keep = torch.ones(s, s, dtype=torch.bool, device=q.device).tril()
+    scores = scores.masked_fill(~keep, float("-inf"))
+    p = torch.softmax(scores, dim=-1)
+    out = torch.matmul(p, vh).permute(2, 0, 1, 3)
+    if return_lse:
+        return out, torch.logsumexp(scores, dim=-1)
+    return out
+
+
+def swiglu(x: Tensor) -> Tensor:
+    x1, x2 = x.chunk(2, dim=-1)
+    return torch.nn.functional.silu(x1) * x2
+
+
+def swiglu_bwd_formula(dy: Tensor, x: Tensor) -> Tensor:
+    x1, x2 = x.chunk(2, dim=-1)
+    sig = torch.sigmoid(x1)
+    return torch.cat((dy * sig * (1 + x1 * (1 - sig)) * x2, dy * x1 * sig), dim=-1)
+
+
+# ------------------------------------------------------------------------- layer
+PARAM_ORDER = ("ln1", "w_qkv", "w_proj", "ln2", "w_fc1", "w_fc2")
+
+
+def init_layer_params(dims: LayerDims, generator: torch.Generator, std: float = 0.02,
+                      dtype=torch.float32) -> Dict[str, Tensor]:
+    """Weights N(0, std^2) drawn in fp32 in the order qkv, proj, fc1, fc2; norm weights one."""
+    def draw(*shape):
+        return torch.empty(*shape, dtype=torch.float32).normal_(0.0, std, generator=generator).to(dtype)
+
+    p = {
+        "ln1": torch.ones(dims.hidden, dtype=dtype),
+        "w_qkv": draw(dims.qkv_width, dims.hidden),
+        "w_proj": draw(dims.hidden, dims.nq * dims.hd),
+        "ln2": torch.ones(dims.hidden, dtype=dtype),
+        "w_fc1": draw(2 * dims.ffn, dims.hidden),
+        "w_fc2": draw(dims.hidden, dims.ffn),
+    }
+    return p
+
+
+def layer_forward(x: Tensor, p: Dict[str, Tensor], dims: LayerDims, freqs: Tensor) -> Tensor:
+    """x [s, b, h] -> [s, b, h]; pre-norm attention block then pre-norm SwiGLU MLP block."""
+    s, b, _ = x.shape
+    h1 = rmsnorm(x, p["ln1"], dims.eps)
+    q, k, v = split_qkv(linear(h1, p["w_qkv"]), dims.nq, dims.nkv, dims.hd)
+    q, k = rope(q, freqs), rope(k, freqs)
+    a = causal_gqa_attention(q, k, v).reshape(s, b, dims.nq * dims.hd)
+    x = x + linear(a, p["w_proj"])
+    h2 = rmsnorm(x, p["ln2"], dims.eps)
+    return x + linear(swiglu(linear(h2, p["w_fc1"])), p["w_fc2"])
+
+
+def stack_forward(x: Tensor, layers: List[Dict[str, Tensor]], dims: LayerDims, freqs: Tensor) -> Tensor:
+    for p in layers:
+        x = layer_forward(x, p, dims, freqs)
+    return x
+
+
+def stack_forward_backward(x: Tensor, layers: List[Dict[str, Tensor]], dims: LayerDims,
+                           grad_out: Tensor, freqs: Optional[Tensor] = None):
+    """Returns (y, dx, [per-layer dict of parameter gradients])."""
+    if freqs is None:
+        freqs = rope_table(x.shape[0], dims.hd, dims.rope_base, dtype=x.dtype)
+    x = x.detach().clone().requires_grad_(True)
+    leaves = [{k: v.detach().clone().requires_grad_(True) for k, v in p.items()} for p in layers]
+    y = stack_forward(x, leaves, dims, freqs)
+    y.backward(grad_out)
+    return y.detach(), x.grad, [{k: v.grad for k, v in p.items()} for p in leaves]
