@@ -1,0 +1,128 @@
+/*
+ * C ABI of libkareus_hip.so — hand-written gfx950 (MI355X) kernels for one GPU's shard of
+ * a Llama-style decoder layer.  This is the boundary a drop-in replacement of the
+ * reference's native calls binds to: every entry point below names the native call of the
+ * reference it stands in for.
+ *
+ * Conventions (all entry points)
+ *   - Pointers are raw device addresses; bf16 data is 2-byte brain-float, fp32 where stated.
+ *   - Leading dimensions and strides are in ELEMENTS.  Rows must start 16-byte aligned.
+ *   - The caller allocates every output and every workspace; the library never allocates
+ *     or frees device memory, keeps no mutable global state and never synchronises the
+ *     device.  Calls on different streams may be issued concurrently from different threads.
+ *   - `stream` is a hipStream_t (NULL = the default stream).
+ *   - Return value: KR_OK (0) or a negative KR_E* code.  Nothing is launched on error.
+ */
+#ifndef KAREUS_HIP_H
+#define KAREUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KR_OK 0
+#define KR_EINVAL (-1)       /* null pointer, non-positive size, misaligned pointer or stride */
+#define KR_EUNSUPPORTED (-2) /* shape outside what the kernels are built for */
+#define KR_ELAUNCH (-3)      /* the HIP runtime rejected the launch */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int kr_version(void);
+/* Static text for a return code. */
+const char* kr_error_string(int code);
+
+/* ---- GEMM ------------------------------------------------------------------------------
+ * bf16 x bf16 -> fp32 accumulate -> bf16.  Replaces tex.generic_gemm (cuBLASLt) as called
+ * by kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:
+ *   KR_GEMM_TN  :571-582  y  = x . W^T     A = x  [M,K] row-major, B = W  [N,K] row-major
+ *   KR_GEMM_NN  :847-859  dx = dy . W      A = dy [M,K] row-major, B = W  [K,N] row-major
+ *   KR_GEMM_NT  :898-909  dW = dy^T . x    A = dy [K,M] row-major, B = x  [K,N] row-major
+ * C is [M,N] row-major.  M, N, K, lda, ldb, ldc must be multiples of 8.
+ * accumulate != 0 adds the product to the existing contents of C (rounded once).          */
+#define KR_GEMM_TN 0
+#define KR_GEMM_NN 1
+#define KR_GEMM_NT 2
+int kr_gemm_bf16(int layout, int M, int N, int K,
+                 const void* A, int64_t lda, const void* B, int64_t ldb,
+                 void* C, int64_t ldc, int accumulate, void* stream);
+
+/* ---- RMSNorm ---------------------------------------------------------------------------
+ * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd
+ * (kareus/transformer_engine/pytorch/ops/basic/rmsnorm.py:210-219, 256-263).
+ * x, y, dy, dx: [rows, cols] bf16 contiguous; gamma, dgamma: [cols] bf16; rstd: [rows] fp32.
+ * cols must be a multiple of 8 and at most 8192.
+ * fwd: rstd = rsqrt(mean(x^2) + eps), y = (x * rstd) * gamma.
+ * bwd: dx = rstd * (g - xhat * mean(g * xhat)), g = gamma * dy, xhat = x * rstd;
+ *      dgamma = sum over rows of dy * xhat.  workspace: kr_rmsnorm_bwd_workspace_bytes().  */
+int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd,
+                   int rows, int cols, float eps, void* stream);
+size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols);
+int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
+                   void* dx, void* dgamma, void* workspace, int rows, int cols, void* stream);
+
+/* ---- Rotary position embedding ---------------------------------------------------------
+ * Replaces fused_rotary_positional_embedding.forward / backward (Apex), called from
+ * kareus/apex/transformer/functional/fused_rope.py:27-35, 41-46.
+ * t, out: [s, b, heads, hd] bf16 addressed as s*stride_s + b*stride_b + head*stride_h + d
+ * (hd contiguous; strides multiples of 8).  freqs: [s, hd] fp32 angles; all hd channels are
+ * rotated, halves layout: out = t*cos(f) + rotate_half(t)*sin(f), rotate_half([a,b]) = [-b,a].
+ * backward != 0 rotates by -f (the gradient of the forward).  out may alias t.
+ * hd must be a multiple of 16 and at most 256.                                             */
+int kr_rope(const void* t, void* out, const float* freqs,
+            int s, int b, int heads, int hd,
+            int64_t t_stride_s, int64_t t_stride_b, int64_t t_stride_h,
+            int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
+            int backward, void* stream);
+
+/* ---- SwiGLU ----------------------------------------------------------------------------
+ * Replaces the Inductor kernels of fused_swiglu_forward / fused_swiglu_backward
+ * (kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20, 34-44).
+ * x, dx: [rows, 2*F] bf16; y, dy: [rows, F] bf16; all contiguous; F a multiple of 8.
+ * y = silu(x[:, :F]) * x[:, F:].                                                           */
+int kr_swiglu_fwd(const void* x, void* y, int64_t rows, int F, void* stream);
+int kr_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t rows, int F, void* stream);
+
+/* ---- Residual add ----------------------------------------------------------------------
+ * out = a + b over n bf16 elements (fp32 add, one rounding).  Replaces the Inductor kernel
+ * of fused_bias_dropout_add_forward with p = 0 and no bias
+ * (kareus/megatron/core/extensions/ops/bias_dropout_add.py:15-32) and the gradient sum of
+ * ResidualForkOp (kareus/megatron/core/extensions/ops/residual_fork.py:104-106).
+ * out may alias a or b.                                                                    */
+int kr_add(const void* a, const void* b, void* out, int64_t n, void* stream);
+
+/* ---- Causal grouped-query attention ----------------------------------------------------
+ * Replaces flash_attn_2_cuda.fwd / bwd as called from
+ * kareus/flash_attn/flash_attn_interface.py:66-80, 174-194.
+ * q, o, dq, do: [s, b, nq, hd]; k, v, dk, dv: [s, b, nkv, hd]; bf16, element (si, bi, h, d) at
+ * si*stride_s + bi*stride_b + h*stride_h + d.  lse: [b, nq, s] fp32 contiguous
+ * (natural log-sum-exp of the scaled, masked scores).  Query head h reads KV head
+ * h / (nq/nkv).  Causal, query i sees keys <= i.  hd must be 128; s a multiple of 128.
+ * kr_attn_bwd also needs a workspace of kr_attn_bwd_workspace_bytes() bytes.               */
+int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                int s, int b, int nq, int nkv, int hd, float scale,
+                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_h,
+                int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
+                int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
+                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
+                void* stream);
+size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);
+int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                const void* o, const float* lse,
+                void* dq, void* dk, void* dv, void* workspace,
+                int s, int b, int nq, int nkv, int hd, float scale,
+                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_h,
+                int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
+                int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
+                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
+                int64_t do_stride_s, int64_t do_stride_b, int64_t do_stride_h,
+                int64_t dq_stride_s, int64_t dq_stride_b, int64_t dq_stride_h,
+                int64_t dk_stride_s, int64_t dk_stride_b, int64_t dk_stride_h,
+                int64_t dv_stride_s, int64_t dv_stride_b, int64_t dv_stride_h,
+                void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KAREUS_HIP_H */

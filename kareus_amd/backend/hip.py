@@ -1,0 +1,245 @@
+"""The product backend: gfx950 kernels of ``libkareus_hip.so`` called through its C ABI.
+
+PyTorch supplies device memory and the current HIP stream; every arithmetic step is a
+hand-written kernel.  There is no fallback: a missing library, a non-HIP tensor or a
+dtype other than bf16 raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Tuple
+
+import torch
+from torch import Tensor
+
+_LIB_NAME = "libkareus_hip.so"
+_c_void_p, _c_int, _c_i64, _c_float, _c_size_t = (
+    ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t,
+)
+
+# name -> (restype, argtypes); mirrors include/kareus_hip.h
+_SIGNATURES = {
+    "kr_version": (_c_int, []),
+    "kr_error_string": (ctypes.c_char_p, [_c_int]),
+    "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
+                              _c_void_p, _c_i64, _c_int, _c_void_p]),
+    "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p]),
+    "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
+    "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_void_p]),
+    "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
+                + [_c_int, _c_void_p]),
+    "kr_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
+    "kr_swiglu_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
+    "kr_add": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
+    "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 12 + [_c_void_p]),
+    "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
+    "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 24 + [_c_void_p]),
+}
+
+KR_GEMM_TN, KR_GEMM_NN, KR_GEMM_NT = 0, 1, 2
+
+
+def library_path() -> str:
+    return os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), _LIB_NAME)
+
+
+def load_library() -> ctypes.CDLL:
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{path} is missing: build it with `make -C kareus_amd/csrc` "
+            "(or __graft_entry__.build()). The hip backend has no fallback."
+        )
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in _SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+class HipBackend:
+    name = "hip"
+
+    def __init__(self) -> None:
+        self.lib = load_library()
+
+    # -- plumbing -------------------------------------------------------------------
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def _check(self, rc: int, what: str) -> None:
+        if rc != 0:
+            raise RuntimeError(f"{what} failed: {self.lib.kr_error_string(rc).decode()} (code {rc})")
+
+    @staticmethod
+    def _dev(*tensors: Tensor) -> None:
+        for t in tensors:
+            if not t.is_cuda:
+                raise RuntimeError("the hip backend needs tensors on the HIP device")
+            if t.dtype not in (torch.bfloat16, torch.float32):
+                raise RuntimeError(f"unsupported dtype {t.dtype}")
+
+    @staticmethod
+    def _bf16(*tensors: Tensor) -> None:
+        for t in tensors:
+            if t.dtype != torch.bfloat16:
+                raise RuntimeError(f"the hip backend computes in bf16, got {t.dtype}")
+
+    # -- GEMM -------------------------------------------------------------------------
+    def gemm(self, layout: int, a: Tensor, b: Tensor, m: int, n: int, k: int,
+             out: Tensor = None, accumulate: bool = False) -> Tensor:
+        self._dev(a, b)
+        self._bf16(a, b)
+        if a.stride(-1) != 1 or b.stride(-1) != 1:
+            raise RuntimeError("GEMM operands must have a contiguous last dimension")
+        if out is None:
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+        rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
+                                   out.data_ptr(), out.stride(0), int(accumulate), self._stream())
+        self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k})")
+        return out
+
+    def linear_fwd(self, x: Tensor, w: Tensor) -> Tensor:
+        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1])
+
+    def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
+        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1])
+
+    def linear_wgrad(self, dy: Tensor, x: Tensor) -> Tensor:
+        return self.gemm(KR_GEMM_NT, dy, x, dy.shape[1], x.shape[1], dy.shape[0])
+
+    # -- RMSNorm ----------------------------------------------------------------------
+    def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+        self._dev(x, gamma)
+        self._bf16(x, gamma)
+        rows, cols = x.shape
+        y = torch.empty_like(x)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rc = self.lib.kr_rmsnorm_fwd(x.data_ptr(), gamma.data_ptr(), y.data_ptr(), rstd.data_ptr(),
+                                     rows, cols, eps, self._stream())
+        self._check(rc, "kr_rmsnorm_fwd")
+        return y, rstd
+
+    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor) -> Tuple[Tensor, Tensor]:
+        self._dev(dy, x, rstd, gamma)
+        self._bf16(dy, x, gamma)
+        rows, cols = x.shape
+        dx = torch.empty_like(x)
+        dgamma = torch.empty_like(gamma)
+        ws = torch.empty(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), dtype=torch.uint8, device=x.device)
+        rc = self.lib.kr_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+                                     dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols, self._stream())
+        self._check(rc, "kr_rmsnorm_bwd")
+        return dx, dgamma
+
+    # -- RoPE -------------------------------------------------------------------------
+    def _rope(self, t: Tensor, freqs: Tensor, backward: bool, out: Tensor = None) -> Tensor:
+        self._dev(t, freqs)
+        self._bf16(t)
+        if freqs.dtype != torch.float32:
+            raise RuntimeError("the rotary table must be fp32")
+        s, b, heads, hd = t.shape
+        if t.stride(3) != 1:
+            raise RuntimeError("rotary input needs a contiguous head dimension")
+        if freqs.shape[-1] != hd:
+            raise RuntimeError("partial rotary (rot_dim < head_dim) is not supported")
+        f2d = freqs.reshape(freqs.shape[0], hd)
+        if not f2d.is_contiguous():
+            f2d = f2d.contiguous()
+        if out is None:
+            out = torch.empty((s, b, heads, hd), dtype=t.dtype, device=t.device)
+        rc = self.lib.kr_rope(t.data_ptr(), out.data_ptr(), f2d.data_ptr(), s, b, heads, hd,
+                              t.stride(0), t.stride(1), t.stride(2),
+                              out.stride(0), out.stride(1), out.stride(2), int(backward), self._stream())
+        self._check(rc, "kr_rope")
+        return out
+
+    def rope_fwd(self, t: Tensor, freqs: Tensor) -> Tensor:
+        return self._rope(t, freqs, False)
+
+    def rope_bwd(self, g: Tensor, freqs: Tensor) -> Tensor:
+        return self._rope(g, freqs, True)
+
+    def rope_inplace(self, t: Tensor, freqs: Tensor, backward: bool) -> Tensor:
+        return self._rope(t, freqs, backward, out=t)
+
+    # -- SwiGLU / add -------------------------------------------------------------------
+    def swiglu_fwd(self, x: Tensor) -> Tensor:
+        self._dev(x)
+        self._bf16(x)
+        rows, two_f = x.shape
+        y = torch.empty((rows, two_f // 2), dtype=x.dtype, device=x.device)
+        self._check(self.lib.kr_swiglu_fwd(x.data_ptr(), y.data_ptr(), rows, two_f // 2, self._stream()),
+                    "kr_swiglu_fwd")
+        return y
+
+    def swiglu_bwd(self, dy: Tensor, x: Tensor) -> Tensor:
+        self._dev(dy, x)
+        self._bf16(dy, x)
+        rows, two_f = x.shape
+        dx = torch.empty_like(x)
+        self._check(self.lib.kr_swiglu_bwd(dy.data_ptr(), x.data_ptr(), dx.data_ptr(), rows, two_f // 2,
+                                           self._stream()), "kr_swiglu_bwd")
+        return dx
+
+    def add(self, a: Tensor, b: Tensor) -> Tensor:
+        self._dev(a, b)
+        self._bf16(a, b)
+        if a.shape != b.shape:
+            raise RuntimeError(f"add: shapes differ, {tuple(a.shape)} vs {tuple(b.shape)}")
+        if not a.is_contiguous():
+            a = a.contiguous()
+        if not b.is_contiguous():
+            b = b.contiguous()
+        out = torch.empty_like(a)
+        self._check(self.lib.kr_add(a.data_ptr(), b.data_ptr(), out.data_ptr(), a.numel(), self._stream()), "kr_add")
+        return out
+
+    # -- attention ----------------------------------------------------------------------
+    @staticmethod
+    def _sbh(t: Tensor):
+        if t.stride(3) != 1:
+            raise RuntimeError("attention tensors need a contiguous head dimension")
+        return t.stride(0), t.stride(1), t.stride(2)
+
+    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
+        if not causal:
+            raise RuntimeError("only causal attention is implemented")
+        self._dev(q, k, v)
+        self._bf16(q, k, v)
+        s, b, nq, hd = q.shape
+        nkv = k.shape[2]
+        o = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
+        lse = torch.empty((b, nq, s), dtype=torch.float32, device=q.device)
+        rc = self.lib.kr_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                  s, b, nq, nkv, hd, scale, *self._sbh(q), *self._sbh(k), *self._sbh(v),
+                                  *self._sbh(o), self._stream())
+        self._check(rc, f"kr_attn_fwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
+        return o, lse
+
+    def attn_bwd(self, do: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor,
+                 scale: float, causal: bool = True):
+        if not causal:
+            raise RuntimeError("only causal attention is implemented")
+        self._dev(do, q, k, v, o, lse)
+        self._bf16(do, q, k, v, o)
+        s, b, nq, hd = q.shape
+        nkv = k.shape[2]
+        do4 = do.reshape(s, b, nq, hd)
+        o4 = o.reshape(s, b, nq, hd)
+        dq = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
+        dk = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
+        dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
+        nbytes = self.lib.kr_attn_bwd_workspace_bytes(s, b, nq, nkv, hd)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+        rc = self.lib.kr_attn_bwd(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
+                                  lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
+                                  s, b, nq, nkv, hd, scale,
+                                  *self._sbh(q), *self._sbh(k), *self._sbh(v), *self._sbh(o4), *self._sbh(do4),
+                                  *self._sbh(dq), *self._sbh(dk), *self._sbh(dv), self._stream())
+        self._check(rc, f"kr_attn_bwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
+        return dq, dk, dv

@@ -1,0 +1,639 @@
+// Causal grouped-query flash attention for head_dim 128 on the gfx950 matrix cores.
+//
+// Roofline: MFMA.  Algorithmic work: forward 2*b*nq*s^2*hd FLOP (causal half of 4*s^2*hd),
+// backward 2.5x that.
+//
+// Forward.  A workgroup of 4 waves owns 128 consecutive queries of one (batch, query head);
+// each wave owns 32 of them and never exchanges data with the others — they only share the
+// K/V tiles (64 keys at a time) that the workgroup stages in LDS, double-buffered with the
+// next tile's global loads in flight during the current tile's math.
+//   S^T = K . Q^T is computed with K rows on the MFMA A port and the wave's Q fragment (held
+//   in registers for the whole kernel) on the B port, so a lane ends up with 16 scores per
+//   32-key tile *of a single query row* (row = lane % 32; lanes l and l+32 split the keys).
+//   The online-softmax row maximum and row sum are therefore in-lane reductions plus one
+//   exchange between the two half-waves.
+//   O^T += V^T . P^T: the probabilities are already laid out as the B-port operand (the
+//   contraction index of an MFMA can be permuted freely as long as both operands agree), and
+//   V^T fragments come out of LDS through the transposing read ds_read_b64_tr_b16.  Neither
+//   P nor V is ever transposed through memory.
+// Tensors are addressed through (seq, batch, head) strides, so sequence-major [s, b, h, d]
+// views of the fused QKV projection are consumed in place.
+#include <mutex>
+
+#include "kr_common.h"
+
+namespace {
+
+constexpr int HD = 128;
+constexpr int BQ = 128;       // queries per workgroup (4 waves x 32)
+constexpr int BKV = 64;       // keys per staged tile
+constexpr int LDKT = HD + 8;  // K tile row length in LDS (elements)
+constexpr int LDVT = HD + 32; // V tile row length in LDS (elements)
+constexpr int K_ELEMS = BKV * LDKT;
+constexpr int V_ELEMS = BKV * LDVT;
+constexpr int FWD_THREADS = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr int kXcds = 8;
+
+__device__ __forceinline__ int xcd_contiguous_id(int pid, int nblocks) {
+  const int q = nblocks / kXcds, r = nblocks % kXcds;
+  const int xcd = pid % kXcds;
+  return xcd * q + (xcd < r ? xcd : r) + pid / kXcds;
+}
+
+struct KVStager {
+  bf16x8 kreg[4], vreg[4];
+  __device__ __forceinline__ void load(const bf16* __restrict__ kb, const bf16* __restrict__ vb,
+                                       int64_t k_ss, int64_t v_ss, int key0, int tid) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * FWD_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
+      kreg[i] = ldg8(kb + (int64_t)(key0 + row) * k_ss + col);
+      vreg[i] = ldg8(vb + (int64_t)(key0 + row) * v_ss + col);
+    }
+  }
+  __device__ __forceinline__ void store(bf16* kt, bf16* vt, int tid) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * FWD_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
+      *reinterpret_cast<bf16x8*>(kt + row * LDKT + col) = kreg[i];
+      *reinterpret_cast<bf16x8*>(vt + row * LDVT + col) = vreg[i];
+    }
+  }
+};
+
+// V^T fragment for one MFMA: rows-of-output d = d0 + lane%32, contraction slots
+// {key0 + 4h + 0..3, key0 + 8 + 4h + 0..3}, h = lane/32 (matches how P sits in registers).
+__device__ __forceinline__ bf16x8 read_vt_frag(const bf16* vt, int key0, int d0, int lane) {
+  const int p = lane & 15;
+  const int row = key0 + 4 * (lane >> 5) + (p >> 2);
+  const int col = d0 + ((lane >> 4) & 1) * 16 + (p & 3) * 4;
+  const bf16* a0 = vt + row * LDVT + col;
+  union {
+    struct { s16x4 lo, hi; } s;
+    bf16x8 v;
+  } u;
+  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
+  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 8 * LDVT));
+  return u.v;
+}
+
+__global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
+    int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
+    int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb, int64_t o_sh) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  constexpr int STAGE = K_ELEMS + V_ELEMS;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int nqt = s / BQ;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int qt = nqt - 1 - (lid % nqt);  // longest rows first inside each (batch, head)
+  const int head = (lid / nqt) % nq;
+  const int bi = lid / (nqt * nq);
+  const int kvh = head / (nq / nkv);
+
+  const int q0 = qt * BQ;
+  const int qw0 = q0 + wave * 32;
+  const int qrow = qw0 + (lane & 31);
+  const bf16* qp = q + (int64_t)bi * q_sb + (int64_t)head * q_sh + (int64_t)qrow * q_ss;
+  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
+  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
+
+  bf16x8 qf[HD / 16];
+#pragma unroll
+  for (int kk = 0; kk < HD / 16; ++kk) qf[kk] = ldg8(qp + kk * 16 + h * 8);
+
+  f32x16 oacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int ntiles = (q0 + BQ) / BKV;
+  KVStager st;
+  st.load(kb, vb, k_ss, v_ss, 0, tid);
+  st.store(smem, smem + K_ELEMS, tid);
+  __syncthreads();
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int cur = j & 1;
+    if (j + 1 < ntiles) st.load(kb, vb, k_ss, v_ss, (j + 1) * BKV, tid);
+    const int key0 = j * BKV;
+    if (key0 <= qw0 + 31) {  // wave-uniform: this tile has keys some of the wave's rows may see
+      const bf16* kt = smem + cur * STAGE;
+      const bf16* vt = kt + K_ELEMS;
+      f32x16 sacc[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < HD / 16; ++kk) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+              kt + (t * 32 + (lane & 31)) * LDKT + kk * 16 + h * 8);
+          sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sacc[t], 0, 0, 0);
+        }
+      }
+      // scores -> log2 domain, causal mask, online softmax
+      const bool need_mask = key0 + BKV - 1 > qw0;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          float sv = sacc[t][e] * scale_log2;
+          if (need_mask) {
+            const int key = key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+            if (key > qrow) sv = -INFINITY;
+          }
+          sacc[t][e] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      float psum = 0.f;
+      bf16x8 pb[2][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float p = __builtin_amdgcn_exp2f(sacc[t][e] - m_new);
+          psum += p;
+          pb[t][e >> 3][e & 7] = (bf16)p;
+        }
+      l_run = l_run * alpha + psum;
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; ++dt) {
+            const bf16x8 vf = read_vt_frag(vt, t * 32 + k2 * 16, dt * 32, lane);
+            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[t][k2], oacc[dt], 0, 0, 0);
+          }
+    }
+    if (j + 1 < ntiles) st.store(smem + (cur ^ 1) * STAGE, smem + (cur ^ 1) * STAGE + K_ELEMS, tid);
+    __syncthreads();
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
+  const float inv_l = 1.0f / l_tot;
+  bf16* op = o + (int64_t)bi * o_sb + (int64_t)head * o_sh + (int64_t)qrow * o_ss;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x4 ov;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ov[e] = (bf16)(oacc[dt][g * 4 + e] * inv_l);
+      *reinterpret_cast<bf16x4*>(op + dt * 32 + g * 8 + h * 4) = ov;
+    }
+  if (h == 0)
+    lse[((int64_t)bi * nq + head) * s + qrow] = (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2;
+}
+
+}  // namespace
+
+static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
+  if (s <= 0 || b <= 0 || nq <= 0 || nkv <= 0) return KR_EINVAL;
+  if (hd != HD || s % BQ || nq % nkv) return KR_EUNSUPPORTED;
+  return KR_OK;
+}
+
+extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
+                           int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
+                           int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh, int64_t v_ss,
+                           int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb, int64_t o_sh,
+                           void* stream) {
+  if (!q || !k || !v || !o || !lse) return KR_EINVAL;
+  const int rc = check_attn_common(s, b, nq, nkv, hd);
+  if (rc != KR_OK) return rc;
+  if (!kr_aligned16(q) || !kr_aligned16(k) || !kr_aligned16(v) || !kr_aligned16(o)) return KR_EINVAL;
+  if ((q_ss | q_sb | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sh) % 8)
+    return KR_EINVAL;
+  constexpr size_t lds_bytes = 2 * (K_ELEMS + V_ELEMS) * sizeof(bf16);
+  static std::once_flag once;
+  static hipError_t attr_status = hipSuccess;
+  std::call_once(once, [&] {
+    attr_status = hipFuncSetAttribute((const void*)attn_fwd_kernel,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  });
+  if (attr_status != hipSuccess) return KR_ELAUNCH;
+  const int blocks = (s / BQ) * nq * b;
+  hipLaunchKernelGGL(attn_fwd_kernel, dim3(blocks), dim3(FWD_THREADS), lds_bytes,
+                     (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
+                     lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sh, k_ss, k_sb, k_sh, v_ss, v_sb,
+                     v_sh, o_ss, o_sb, o_sh);
+  return kr_launch_status();
+}
+
+// =============================================================================================
+// Backward.  Three launches, no atomics, deterministic:
+//   1. delta[b, h, i] = sum_d dO[i, d] * O[i, d]                      (HBM-bound pre-pass)
+//   2. dK, dV: a workgroup owns 128 keys of one (batch, KV head) — 32 per wave, their K and V
+//      fragments in registers — and streams every query tile at or below the diagonal, for
+//      every query head of the group, through LDS.  Per 32x32 block:
+//        S = Q.K^T, dP = dO.V^T (rows = queries on the MFMA A port, so a lane holds one key
+//        column), P = exp2(S*c - lse), dS = P*(dP - delta), then dV^T += dO^T.P and
+//        dK^T += Q^T.dS with the Q / dO tiles read back transposed (ds_read_b64_tr_b16).
+//   3. dQ: a workgroup owns 128 queries of one (batch, head) and streams the key tiles up to
+//      the diagonal: S^T = K.Q^T, dP^T = V.dO^T (a lane holds one query row), dS^T, then
+//      dQ^T += K^T.dS^T with the K tile read back transposed.
+//   Recomputing S and dP in both passes costs 7 instead of 5 tile products but keeps every
+//   accumulator in registers and every output written exactly once.
+// LDS tiles that are read both ways ([rows][128] bf16, 256-byte rows, no padding) use an XOR
+// swizzle of the 16-byte chunk index, chunk ^= ((row & 7) << 1) | ((row >> 3) & 1): 8
+// consecutive rows land in 8 different 32-byte bank groups for the vector reads, and the 4x64-
+// byte footprint of a transposing read spreads over all banks as well.
+// =============================================================================================
+namespace {
+
+constexpr int TILE_ELEMS = 64 * HD;  // one swizzled [64][128] tile
+
+__device__ __forceinline__ int swz_off(int row, int col) {
+  const int f = ((row & 7) << 1) | ((row >> 3) & 1);
+  return row * HD + ((((col >> 3) ^ f)) << 3) + (col & 7);
+}
+
+// [64][128] tile, global rows row0.. -> swizzled LDS; 256 threads, 4 chunks each
+struct TileStager {
+  bf16x8 r[4];
+  __device__ __forceinline__ void load(const bf16* __restrict__ base, int64_t ss, int row0, int tid) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256;
+      r[i] = ldg8(base + (int64_t)(row0 + (c >> 4)) * ss + (c & 15) * 8);
+    }
+  }
+  __device__ __forceinline__ void store(bf16* tile, int tid) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256;
+      *reinterpret_cast<bf16x8*>(tile + swz_off(c >> 4, (c & 15) * 8)) = r[i];
+    }
+  }
+};
+
+// row-major fragment: lane gets tile row (row0 + lane%32), columns 16*kk + 8*(lane/32) + 0..7
+__device__ __forceinline__ bf16x8 read_rows_swz(const bf16* tile, int row0, int kk, int lane) {
+  return *reinterpret_cast<const bf16x8*>(tile + swz_off(row0 + (lane & 31), kk * 16 + (lane >> 5) * 8));
+}
+
+// transposed fragment: lane gets tile column (d0 + lane%32), rows {r0+4h+0..3, r0+8+4h+0..3}
+__device__ __forceinline__ bf16x8 read_cols_swz(const bf16* tile, int r0, int d0, int lane) {
+  const int p = lane & 15;
+  const int row = r0 + 4 * (lane >> 5) + (p >> 2);
+  const int col = d0 + ((lane >> 4) & 1) * 16 + (p & 3) * 4;
+  union {
+    struct { s16x4 lo, hi; } s;
+    bf16x8 v;
+  } u;
+  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row, col)));
+  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row + 8, col)));
+  return u.v;
+}
+
+__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ dout,
+                                                         const bf16* __restrict__ o,
+                                                         float* __restrict__ delta, int s, int nq,
+                                                         int64_t total_rows, int64_t do_ss,
+                                                         int64_t do_sb, int64_t do_sh, int64_t o_ss,
+                                                         int64_t o_sb, int64_t o_sh) {
+  // 16 lanes per (batch, head, position) row of 128 channels
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int sub = threadIdx.x & 15;
+  if (row >= total_rows) return;
+  const int si = (int)(row % s);
+  const int head = (int)((row / s) % nq);
+  const int bi = (int)(row / ((int64_t)s * nq));
+  const bf16x8 a = ldg8(dout + bi * do_sb + head * do_sh + (int64_t)si * do_ss + sub * 8);
+  const bf16x8 b = ldg8(o + bi * o_sb + head * o_sh + (int64_t)si * o_ss + sub * 8);
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, KR_WAVE);
+  if (sub == 0) delta[row] = acc;
+}
+
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16* __restrict__ dk, bf16* __restrict__ dv, int s, int nq, int nkv, float scale,
+    float scale_log2, int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t do_ss, int64_t do_sb,
+    int64_t do_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh, int64_t dv_ss, int64_t dv_sb,
+    int64_t dv_sh) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  // stage layout: Q tile | dO tile | lse[64] fp32 | delta[64] fp32
+  constexpr int STAGE = 2 * TILE_ELEMS + 256;  // in bf16 units (256 bf16 = 128 floats)
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int nkt = s / 128;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int kt = lid % nkt;  // low key tiles see the most queries: they come first
+  const int kvh = (lid / nkt) % nkv;
+  const int bi = lid / (nkt * nkv);
+  const int rep = nq / nkv;
+  const int key0 = kt * 128;
+  const int kw0 = key0 + wave * 32;
+  const int krow = kw0 + (lane & 31);
+
+  const bf16* kp = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh + (int64_t)krow * k_ss;
+  const bf16* vp = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh + (int64_t)krow * v_ss;
+  bf16x8 kf[HD / 16], vf[HD / 16];
+#pragma unroll
+  for (int kk = 0; kk < HD / 16; ++kk) {
+    kf[kk] = ldg8(kp + kk * 16 + h * 8);
+    vf[kk] = ldg8(vp + kk * 16 + h * 8);
+  }
+  f32x16 dkacc[HD / 32], dvacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      dkacc[dt][e] = 0.f;
+      dvacc[dt][e] = 0.f;
+    }
+
+  const int qt_first = key0 / 64;
+  const int nqt = s / 64 - qt_first;  // query tiles of 64 at or below the diagonal
+  const int niter = nqt * rep;
+  TileStager sq, sdo;
+  float st_lse = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
+
+  auto stage_load = [&](int it) {
+    const int hq = it / nqt, qt = qt_first + it % nqt;
+    const int head = kvh * rep + hq;
+    const bf16* qb = q + (int64_t)bi * q_sb + (int64_t)head * q_sh;
+    const bf16* dob = dout + (int64_t)bi * do_sb + (int64_t)head * do_sh;
+    sq.load(qb, q_ss, qt * 64, tid);
+    sdo.load(dob, do_ss, qt * 64, tid);
+    const int64_t stat = ((int64_t)bi * nq + head) * s + qt * 64;
+    if (tid < 64) st_lse = lse[stat + tid] * kLog2e;
+    else if (tid < 128) st_lse = delta[stat + tid - 64];
+  };
+  auto stage_store = [&](int buf) {
+    bf16* base = smem + buf * STAGE;
+    sq.store(base, tid);
+    sdo.store(base + TILE_ELEMS, tid);
+    float* stats = reinterpret_cast<float*>(base + 2 * TILE_ELEMS);
+    if (tid < 128) stats[tid] = st_lse;
+  };
+
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+
+  for (int it = 0; it < niter; ++it) {
+    const int cur = it & 1;
+    if (it + 1 < niter) stage_load(it + 1);
+    const int q0 = (qt_first + it % nqt) * 64;
+    const bf16* qtile = smem + cur * STAGE;
+    const bf16* dotile = qtile + TILE_ELEMS;
+    const float* stats = reinterpret_cast<const float*>(qtile + 2 * TILE_ELEMS);
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      const int qs0 = q0 + sub * 32;
+      if (qs0 + 31 < kw0) continue;  // wave-uniform: every query of the block precedes the keys
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        sacc[e] = 0.f;
+        dpacc[e] = 0.f;
+      }
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk) {
+        const bf16x8 qfr = read_rows_swz(qtile, sub * 32, kk, lane);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr, kf[kk], sacc, 0, 0, 0);
+        const bf16x8 dof = read_rows_swz(dotile, sub * 32, kk, lane);
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dof, vf[kk], dpacc, 0, 0, 0);
+      }
+      // lane: key column krow, query rows qs0 + 8g + 4h + e
+      const bool need_mask = qs0 < kw0 + 31;
+      bf16x8 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float p = __builtin_amdgcn_exp2f(sacc[g * 4 + e] * scale_log2 - l4[e]);
+          if (need_mask && (qs0 + 8 * g + 4 * h + e < krow)) p = 0.f;
+          const float ds = p * (dpacc[g * 4 + e] - d4[e]);
+          pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
+          dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
+        }
+      }
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+          const bf16x8 dot = read_cols_swz(dotile, sub * 32 + k2 * 16, dt * 32, lane);
+          dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot, pb[k2], dvacc[dt], 0, 0, 0);
+          const bf16x8 qtr = read_cols_swz(qtile, sub * 32 + k2 * 16, dt * 32, lane);
+          dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb[k2], dkacc[dt], 0, 0, 0);
+        }
+    }
+    if (it + 1 < niter) stage_store(cur ^ 1);
+    __syncthreads();
+  }
+
+  bf16* dkp = dk + (int64_t)bi * dk_sb + (int64_t)kvh * dk_sh + (int64_t)krow * dk_ss;
+  bf16* dvp = dv + (int64_t)bi * dv_sb + (int64_t)kvh * dv_sh + (int64_t)krow * dv_ss;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x4 a, b;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        a[e] = (bf16)(dkacc[dt][g * 4 + e] * scale);
+        b[e] = (bf16)dvacc[dt][g * 4 + e];
+      }
+      *reinterpret_cast<bf16x4*>(dkp + dt * 32 + g * 8 + h * 4) = a;
+      *reinterpret_cast<bf16x4*>(dvp + dt * 32 + g * 8 + h * 4) = b;
+    }
+}
+
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, int64_t q_ss,
+    int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh, int64_t v_ss,
+    int64_t v_sb, int64_t v_sh, int64_t do_ss, int64_t do_sb, int64_t do_sh, int64_t dq_ss,
+    int64_t dq_sb, int64_t dq_sh) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  constexpr int STAGE = 2 * TILE_ELEMS;  // K tile | V tile, both swizzled [64][128]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int nqt = s / BQ;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int qt = nqt - 1 - (lid % nqt);
+  const int head = (lid / nqt) % nq;
+  const int bi = lid / (nqt * nq);
+  const int kvh = head / (nq / nkv);
+  const int q0 = qt * BQ;
+  const int qw0 = q0 + wave * 32;
+  const int qrow = qw0 + (lane & 31);
+
+  const bf16* qp = q + (int64_t)bi * q_sb + (int64_t)head * q_sh + (int64_t)qrow * q_ss;
+  const bf16* dop = dout + (int64_t)bi * do_sb + (int64_t)head * do_sh + (int64_t)qrow * do_ss;
+  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
+  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
+  bf16x8 qf[HD / 16], dof[HD / 16];
+#pragma unroll
+  for (int kk = 0; kk < HD / 16; ++kk) {
+    qf[kk] = ldg8(qp + kk * 16 + h * 8);
+    dof[kk] = ldg8(dop + kk * 16 + h * 8);
+  }
+  const int64_t stat = ((int64_t)bi * nq + head) * s + qrow;
+  const float my_lse = lse[stat] * kLog2e;
+  const float my_delta = delta[stat];
+
+  f32x16 dqacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dqacc[dt][e] = 0.f;
+
+  const int ntiles = (q0 + BQ) / BKV;
+  TileStager sk, sv;
+  sk.load(kb, k_ss, 0, tid);
+  sv.load(vb, v_ss, 0, tid);
+  sk.store(smem, tid);
+  sv.store(smem + TILE_ELEMS, tid);
+  __syncthreads();
+
+  for (int j = 0; j < ntiles; ++j) {
+    const int cur = j & 1;
+    if (j + 1 < ntiles) {
+      sk.load(kb, k_ss, (j + 1) * BKV, tid);
+      sv.load(vb, v_ss, (j + 1) * BKV, tid);
+    }
+    const int key0 = j * BKV;
+    if (key0 <= qw0 + 31) {
+      const bf16* ktile = smem + cur * STAGE;
+      const bf16* vtile = ktile + TILE_ELEMS;
+      const bool need_mask = key0 + BKV - 1 > qw0;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        f32x16 sacc, dpacc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          sacc[e] = 0.f;
+          dpacc[e] = 0.f;
+        }
+#pragma unroll
+        for (int kk = 0; kk < HD / 16; ++kk) {
+          const bf16x8 kfr = read_rows_swz(ktile, t * 32, kk, lane);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[kk], sacc, 0, 0, 0);
+          const bf16x8 vfr = read_rows_swz(vtile, t * 32, kk, lane);
+          dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dpacc, 0, 0, 0);
+        }
+        // lane: query row qrow, keys key0 + 32t + 8g + 4h + e
+        bf16x8 dsb[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          float p = __builtin_amdgcn_exp2f(sacc[e] * scale_log2 - my_lse);
+          if (need_mask && (key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3) > qrow)) p = 0.f;
+          dsb[e >> 3][e & 7] = (bf16)(p * (dpacc[e] - my_delta));
+        }
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; ++dt) {
+            const bf16x8 ktr = read_cols_swz(ktile, t * 32 + k2 * 16, dt * 32, lane);
+            dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsb[k2], dqacc[dt], 0, 0, 0);
+          }
+      }
+    }
+    if (j + 1 < ntiles) {
+      sk.store(smem + (cur ^ 1) * STAGE, tid);
+      sv.store(smem + (cur ^ 1) * STAGE + TILE_ELEMS, tid);
+    }
+    __syncthreads();
+  }
+
+  bf16* dqp = dq + (int64_t)bi * dq_sb + (int64_t)head * dq_sh + (int64_t)qrow * dq_ss;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x4 a;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) a[e] = (bf16)(dqacc[dt][g * 4 + e] * scale);
+      *reinterpret_cast<bf16x4*>(dqp + dt * 32 + g * 8 + h * 4) = a;
+    }
+}
+
+}  // namespace
+
+extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
+  if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
+  return (size_t)b * nq * s * sizeof(float);
+}
+
+extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                           const void* o, const float* lse, void* dq, void* dk, void* dv,
+                           void* workspace, int s, int b, int nq, int nkv, int hd, float scale,
+                           int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+                           int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss,
+                           int64_t o_sb, int64_t o_sh, int64_t do_ss, int64_t do_sb, int64_t do_sh,
+                           int64_t dq_ss, int64_t dq_sb, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb,
+                           int64_t dk_sh, int64_t dv_ss, int64_t dv_sb, int64_t dv_sh,
+                           void* stream) {
+  if (!dout || !q || !k || !v || !o || !lse || !dq || !dk || !dv || !workspace) return KR_EINVAL;
+  const int rc = check_attn_common(s, b, nq, nkv, hd);
+  if (rc != KR_OK) return rc;
+  const void* ptrs[] = {dout, q, k, v, o, dq, dk, dv, workspace};
+  for (const void* p : ptrs)
+    if (!kr_aligned16(p)) return KR_EINVAL;
+  if ((q_ss | q_sb | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sh | do_ss |
+       do_sb | do_sh | dq_ss | dq_sb | dq_sh | dk_ss | dk_sb | dk_sh | dv_ss | dv_sb | dv_sh) % 8)
+    return KR_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  float* delta = (float*)workspace;
+  constexpr size_t lds_dkdv = 2 * (2 * TILE_ELEMS + 256) * sizeof(bf16);
+  constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
+  static std::once_flag once;
+  static hipError_t attr_status = hipSuccess;
+  std::call_once(once, [&] {
+    attr_status = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+    if (attr_status == hipSuccess)
+      attr_status = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel,
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+  });
+  if (attr_status != hipSuccess) return KR_ELAUNCH;
+
+  const int64_t rows = (int64_t)b * nq * s;
+  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
+                     (const bf16*)dout, (const bf16*)o, delta, s, nq, rows, do_ss, do_sb, do_sh,
+                     o_ss, o_sb, o_sh);
+  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+  const float scale_log2 = scale * kLog2e;
+  hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3((s / 128) * nkv * b), dim3(256), lds_dkdv, st,
+                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
+                     (const float*)delta, (bf16*)dk, (bf16*)dv, s, nq, nkv, scale, scale_log2, q_ss,
+                     q_sb, q_sh, k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, do_ss, do_sb, do_sh, dk_ss,
+                     dk_sb, dk_sh, dv_ss, dv_sb, dv_sh);
+  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+  hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3((s / BQ) * nq * b), dim3(256), lds_dq, st,
+                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
+                     (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, q_ss, q_sb, q_sh,
+                     k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, do_ss, do_sb, do_sh, dq_ss, dq_sb, dq_sh);
+  return kr_launch_status();
+}

@@ -1,0 +1,53 @@
+// Shared device helpers for the gfx950 kernels: vector types, bf16 packing, wave reductions,
+// argument checks.  CDNA4 only: 64-wide wavefronts, MFMA builtins, no portability layer.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/kareus_hip.h"
+
+typedef __bf16 bf16;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+#define KR_WAVE 64
+#define KR_LDS __attribute__((address_space(3)))
+
+// One 16-byte global access = 8 bf16.
+struct __attribute__((aligned(16))) Pack8 {
+  bf16x8 v;
+};
+
+__device__ __forceinline__ bf16x8 ldg8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ void stg8(bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)0.0f;
+  return z;
+}
+
+// Sum / max across the 64 lanes of a wave; every lane gets the result.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, KR_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, KR_WAVE));
+  return v;
+}
+
+static inline bool kr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static inline int kr_launch_status() {
+  return hipGetLastError() == hipSuccess ? KR_OK : KR_ELAUNCH;
+}

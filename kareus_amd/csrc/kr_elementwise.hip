@@ -1,0 +1,163 @@
+// HBM-bound passes: residual add, SwiGLU forward/backward, rotary embedding.
+// Each thread moves 16-byte vectors (8 bf16); the math is fp32 with one rounding on store.
+// Roofline for all of them is HBM bandwidth: bytes moved = inputs read once + outputs
+// written once.
+#include "kr_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__global__ __launch_bounds__(kThreads) void add_kernel(const bf16* a, const bf16* b, bf16* out,
+                                                       int64_t nvec,
+                                                       int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+    bf16x8 x = ldg8(a + i * 8), y = ldg8(b + i * 8), r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (bf16)((float)x[e] + (float)y[e]);
+    stg8(out + i * 8, r);
+  }
+  // tail (n not a multiple of 8)
+  if (blockIdx.x == 0) {
+    for (int64_t i = nvec * 8 + threadIdx.x; i < n; i += kThreads)
+      out[i] = (bf16)((float)a[i] + (float)b[i]);
+  }
+}
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// x [rows, 2F] -> y [rows, F]; one thread per 8 output columns.
+__global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const bf16* __restrict__ x,
+                                                              bf16* __restrict__ y, int64_t rows,
+                                                              int F) {
+  const int fv = F / 8;
+  const int64_t total = rows * fv;
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / fv;
+    const int c = (int)(i - r * fv) * 8;
+    const bf16* xr = x + r * 2 * F;
+    bf16x8 g = ldg8(xr + c), u = ldg8(xr + F + c), o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x1 = (float)g[e], x2 = (float)u[e];
+      o[e] = (bf16)(x1 * sigmoidf_(x1) * x2);
+    }
+    stg8(y + r * F + c, o);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16* __restrict__ dy,
+                                                              const bf16* __restrict__ x,
+                                                              bf16* __restrict__ dx, int64_t rows,
+                                                              int F) {
+  const int fv = F / 8;
+  const int64_t total = rows * fv;
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / fv;
+    const int c = (int)(i - r * fv) * 8;
+    const bf16* xr = x + r * 2 * F;
+    bf16x8 g = ldg8(xr + c), u = ldg8(xr + F + c), d = ldg8(dy + r * F + c), d1, d2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x1 = (float)g[e], x2 = (float)u[e], gy = (float)d[e];
+      float sg = sigmoidf_(x1);
+      d1[e] = (bf16)(gy * sg * (1.0f + x1 * (1.0f - sg)) * x2);
+      d2[e] = (bf16)(gy * x1 * sg);
+    }
+    stg8(dx + r * 2 * F + c, d1);
+    stg8(dx + r * 2 * F + F + c, d2);
+  }
+}
+
+// One block per sequence position: the hd/2 (cos, sin) pairs of that position are computed
+// once into LDS, then the block streams all (batch, head) rows of the position.
+// A thread owns 8 consecutive channels of the first half and the matching 8 of the second.
+__global__ __launch_bounds__(kThreads) void rope_kernel(
+    const bf16* t, bf16* out, const float* __restrict__ freqs, int b,
+    int heads, int hd, int64_t ts, int64_t tb, int64_t th, int64_t os, int64_t ob, int64_t oh,
+    float sin_sign) {
+  __shared__ float cs[128], sn[128];
+  const int pos = blockIdx.x;
+  const int half = hd / 2;
+  for (int i = threadIdx.x; i < half; i += kThreads) {
+    float s_, c_;
+    sincosf(freqs[(int64_t)pos * hd + i], &s_, &c_);
+    cs[i] = c_;
+    sn[i] = s_ * sin_sign;
+  }
+  __syncthreads();
+  const int vec_per_row = half / 8;
+  const int rows = b * heads;
+  const int total = rows * vec_per_row;
+  for (int i = threadIdx.x; i < total; i += kThreads) {
+    const int row = i / vec_per_row;
+    const int c = (i - row * vec_per_row) * 8;
+    const int bi = row / heads, h = row - bi * heads;
+    const bf16* src = t + pos * ts + bi * tb + h * th;
+    bf16* dst = out + pos * os + bi * ob + h * oh;
+    bf16x8 lo = ldg8(src + c), hi = ldg8(src + half + c), olo, ohi;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float a = (float)lo[e], bb = (float)hi[e];
+      float co = cs[c + e], si = sn[c + e];
+      olo[e] = (bf16)(a * co - bb * si);
+      ohi[e] = (bf16)(bb * co + a * si);
+    }
+    stg8(dst + c, olo);
+    stg8(dst + half + c, ohi);
+  }
+}
+
+inline int grid_for(int64_t work_items, int per_block) {
+  int64_t blocks = (work_items + per_block - 1) / per_block;
+  const int64_t cap = 256 * 16;  // 256 CUs, enough resident blocks to cover HBM latency
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+}  // namespace
+
+extern "C" int kr_add(const void* a, const void* b, void* out, int64_t n, void* stream) {
+  if (!a || !b || !out || n <= 0) return KR_EINVAL;
+  if (!kr_aligned16(a) || !kr_aligned16(b) || !kr_aligned16(out)) return KR_EINVAL;
+  const int64_t nvec = n / 8;
+  hipLaunchKernelGGL(add_kernel, dim3(grid_for(nvec, kThreads)), dim3(kThreads), 0,
+                     (hipStream_t)stream, (const bf16*)a, (const bf16*)b, (bf16*)out, nvec, n);
+  return kr_launch_status();
+}
+
+extern "C" int kr_swiglu_fwd(const void* x, void* y, int64_t rows, int F, void* stream) {
+  if (!x || !y || rows <= 0 || F <= 0) return KR_EINVAL;
+  if (F % 8) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(x) || !kr_aligned16(y)) return KR_EINVAL;
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid_for(rows * (F / 8), kThreads)), dim3(kThreads),
+                     0, (hipStream_t)stream, (const bf16*)x, (bf16*)y, rows, F);
+  return kr_launch_status();
+}
+
+extern "C" int kr_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t rows, int F,
+                             void* stream) {
+  if (!dy || !x || !dx || rows <= 0 || F <= 0) return KR_EINVAL;
+  if (F % 8) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(x) || !kr_aligned16(dy) || !kr_aligned16(dx)) return KR_EINVAL;
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid_for(rows * (F / 8), kThreads)), dim3(kThreads),
+                     0, (hipStream_t)stream, (const bf16*)dy, (const bf16*)x, (bf16*)dx, rows, F);
+  return kr_launch_status();
+}
+
+extern "C" int kr_rope(const void* t, void* out, const float* freqs, int s, int b, int heads,
+                       int hd, int64_t ts, int64_t tb, int64_t th, int64_t os, int64_t ob,
+                       int64_t oh, int backward, void* stream) {
+  if (!t || !out || !freqs || s <= 0 || b <= 0 || heads <= 0 || hd <= 0) return KR_EINVAL;
+  if (hd % 16 || hd > 256) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(t) || !kr_aligned16(out)) return KR_EINVAL;
+  if ((ts | tb | th | os | ob | oh) % 8) return KR_EINVAL;
+  hipLaunchKernelGGL(rope_kernel, dim3(s), dim3(kThreads), 0, (hipStream_t)stream,
+                     (const bf16*)t, (bf16*)out, freqs, b, heads, hd, ts, tb, th, os, ob, oh,
+                     backward ? -1.0f : 1.0f);
+  return kr_launch_status();
+}

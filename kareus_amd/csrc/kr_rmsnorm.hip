@@ -1,0 +1,215 @@
+// RMSNorm forward and backward.  HBM-bound: forward reads x and writes y (+4 B/row of rstd),
+// backward reads dy and x and writes dx; gamma stays in cache.  One wavefront owns one row at
+// a time and keeps it in registers (NCHUNK 16-byte vectors per lane), so each element is read
+// from HBM exactly once.  Row statistics are wave shuffle reductions in fp32.
+//
+// The weight gradient is a column sum over all rows: every wave accumulates its rows' dy*xhat
+// in registers (a lane always owns the same columns), the waves of a block combine through
+// LDS, each block writes one fp32 partial row into the workspace, and a second small kernel
+// sums the partial rows and rounds to bf16.
+#include "kr_common.h"
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * KR_WAVE;
+constexpr int kMaxBwdBlocks = 1024;
+
+template <int NCHUNK>
+__global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __restrict__ x,
+                                                               const bf16* __restrict__ gamma,
+                                                               bf16* __restrict__ y,
+                                                               float* __restrict__ rstd, int rows,
+                                                               int cols, float eps) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nvec = cols / 8;
+  const float inv_cols = 1.0f / (float)cols;
+  bf16x8 g[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int v = lane + c * 64;
+    g[c] = v < nvec ? ldg8(gamma + v * 8) : zero8();
+  }
+  for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
+    const bf16* xr = x + (int64_t)row * cols;
+    bf16x8 xv[NCHUNK];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int v = lane + c * 64;
+      xv[c] = v < nvec ? ldg8(xr + v * 8) : zero8();
+    }
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float f = (float)xv[c][e];
+        ss += f * f;
+      }
+    ss = wave_sum(ss);
+    const float rs = rsqrtf(ss * inv_cols + eps);
+    if (lane == 0) rstd[row] = rs;
+    bf16* yr = y + (int64_t)row * cols;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int v = lane + c * 64;
+      if (v < nvec) {
+        bf16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (bf16)(((float)xv[c][e] * rs) * (float)g[c][e]);
+        stg8(yr + v * 8, o);
+      }
+    }
+  }
+}
+
+template <int NCHUNK>
+__global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
+    const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
+    const bf16* __restrict__ gamma, bf16* __restrict__ dx, float* __restrict__ partial, int rows,
+    int cols) {
+  __shared__ float red[kWaves - 1][64 * 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nvec = cols / 8;
+  const float inv_cols = 1.0f / (float)cols;
+  bf16x8 g[NCHUNK];
+  float dg[NCHUNK][8];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int v = lane + c * 64;
+    g[c] = v < nvec ? ldg8(gamma + v * 8) : zero8();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dg[c][e] = 0.f;
+  }
+  for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
+    const bf16* xr = x + (int64_t)row * cols;
+    const bf16* dr = dy + (int64_t)row * cols;
+    const float rs = rstd[row];
+    bf16x8 xv[NCHUNK], dv[NCHUNK];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int v = lane + c * 64;
+      xv[c] = v < nvec ? ldg8(xr + v * 8) : zero8();
+      dv[c] = v < nvec ? ldg8(dr + v * 8) : zero8();
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xh = (float)xv[c][e] * rs;
+        const float d = (float)dv[c][e];
+        dot += d * (float)g[c][e] * xh;
+        dg[c][e] += d * xh;
+      }
+    dot = wave_sum(dot) * inv_cols;
+    bf16* oxr = dx + (int64_t)row * cols;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int v = lane + c * 64;
+      if (v < nvec) {
+        bf16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xh = (float)xv[c][e] * rs;
+          o[e] = (bf16)(rs * ((float)dv[c][e] * (float)g[c][e] - xh * dot));
+        }
+        stg8(oxr + v * 8, o);
+      }
+    }
+  }
+  // combine the block's waves chunk by chunk, then publish the block's partial row
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    if (wave > 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[wave - 1][e * 64 + lane] = dg[c][e];
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const int v = lane + c * 64;
+      if (v < nvec) {
+        float* pr = partial + (int64_t)blockIdx.x * cols + v * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float sum = dg[c][e];
+#pragma unroll
+          for (int w = 0; w < kWaves - 1; ++w) sum += red[w][e * 64 + lane];
+          pr[e] = sum;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// dgamma[col] = sum over partial rows; one thread per column, coalesced across columns.
+__global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* __restrict__ partial,
+                                                             bf16* __restrict__ dgamma,
+                                                             int nparts, int cols) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= cols) return;
+  float acc = 0.f;
+  for (int p = 0; p < nparts; ++p) acc += partial[(int64_t)p * cols + col];
+  dgamma[col] = (bf16)acc;
+}
+
+inline int bwd_blocks(int rows) {
+  int blocks = (rows + kWaves - 1) / kWaves;
+  return blocks > kMaxBwdBlocks ? kMaxBwdBlocks : blocks;
+}
+
+inline int chunks_for(int cols) { return (cols / 8 + 63) / 64; }
+
+}  // namespace
+
+#define KR_DISPATCH_CHUNKS(NC, CALL) \
+  switch (NC) {                      \
+    case 1: { constexpr int C_ = 1; CALL; } break;   \
+    case 2: { constexpr int C_ = 2; CALL; } break;   \
+    case 3: { constexpr int C_ = 3; CALL; } break;   \
+    case 4: { constexpr int C_ = 4; CALL; } break;   \
+    case 5: case 6: { constexpr int C_ = 6; CALL; } break;   \
+    case 7: case 8: { constexpr int C_ = 8; CALL; } break;   \
+    default: { constexpr int C_ = 16; CALL; } break; \
+  }
+
+extern "C" int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd, int rows,
+                              int cols, float eps, void* stream) {
+  if (!x || !gamma || !y || !rstd || rows <= 0 || cols <= 0) return KR_EINVAL;
+  if (cols % 8 || cols > 8192) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(x) || !kr_aligned16(y) || !kr_aligned16(gamma)) return KR_EINVAL;
+  int blocks = (rows + kWaves - 1) / kWaves;
+  if (blocks > 256 * 8) blocks = 256 * 8;
+  const int nc = chunks_for(cols);
+  KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_fwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
+                                           (hipStream_t)stream, (const bf16*)x, (const bf16*)gamma,
+                                           (bf16*)y, rstd, rows, cols, eps));
+  return kr_launch_status();
+}
+
+extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return (size_t)bwd_blocks(rows) * (size_t)cols * sizeof(float);
+}
+
+extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
+                              void* dx, void* dgamma, void* workspace, int rows, int cols,
+                              void* stream) {
+  if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0)
+    return KR_EINVAL;
+  if (cols % 8 || cols > 8192) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(x) || !kr_aligned16(dy) || !kr_aligned16(dx) || !kr_aligned16(gamma) ||
+      !kr_aligned16(workspace))
+    return KR_EINVAL;
+  const int blocks = bwd_blocks(rows);
+  const int nc = chunks_for(cols);
+  KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_bwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
+                                           (hipStream_t)stream, (const bf16*)dy, (const bf16*)x,
+                                           rstd, (const bf16*)gamma, (bf16*)dx, (float*)workspace,
+                                           rows, cols));
+  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 255) / 256), dim3(256), 0,
+                     (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
+  return kr_launch_status();
+}

@@ -5,9 +5,6 @@ The projection's output features are grouped per KV group ``g`` as
 ``[s, b, ng, (nq/ng + 2) * hd]`` and cut along the last axis.  Forward only makes
 views; backward reassembles the three gradients into one tensor
 (kareus/megatron/core/extensions/ops/qkv_postprocess.py:84-127, 164-184).
-
-If the three gradients already are the matching views of one fused buffer (the
-attention backward here writes them that way), that buffer is returned as is.
 """
 
 from __future__ import annotations
@@ -49,10 +46,6 @@ class QKVPostProcessOp(BasicOperation, PartitionableOperator):
 
     def merge(self, gq: torch.Tensor, gk: torch.Tensor, gv: torch.Tensor) -> torch.Tensor:
         ng, hd, per = self.ng, self.hd, self.nq // self.ng
-        fused = getattr(gq, "_kr_fused_qkv", None)
-        if (fused is not None and getattr(gk, "_kr_fused_qkv", None) is fused
-                and getattr(gv, "_kr_fused_qkv", None) is fused):
-            return fused
         gq = gq.reshape(*gq.shape[:-2], ng, per * hd)
         merged = torch.cat([gq, gk, gv], dim=-1)
         return merged.view(*merged.shape[:-2], ng * (per + 2) * hd)
