@@ -27,7 +27,7 @@ class BackwardPartition(PartitionBase):
         pre_ctx: NanoBatchContext,
         protected_tensor_ids: Optional[set] = None,
     ) -> Dict[int, List]:
-        with self._on_stream(ctx):
+        with self._on_stream(ctx), self._timed():
             return self._execute(ctx, pre_ctx, protected_tensor_ids or set())
 
     def _execute(self, ctx, pre_ctx, protected: set) -> Dict[int, List]:

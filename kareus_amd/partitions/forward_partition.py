@@ -19,7 +19,7 @@ from .partition_base import PartitionBase, _current_stream
 @dataclass
 class ForwardPartition(PartitionBase):
     def execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext) -> None:
-        with self._on_stream(ctx):
+        with self._on_stream(ctx), self._timed():
             self._execute(ctx, pre_ctx)
 
     def _execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext) -> None:

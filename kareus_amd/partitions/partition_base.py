@@ -85,6 +85,18 @@ def _current_stream():
     return torch.cuda.current_stream() if torch.cuda.is_available() else None
 
 
+class _TimerScope:
+    def __init__(self, timer, partition) -> None:
+        self.timer, self.partition = timer, partition
+
+    def __enter__(self):
+        self.timer.begin(self.partition)
+
+    def __exit__(self, *exc):
+        self.timer.end(self.partition)
+        return False
+
+
 @dataclass
 class PartitionBase:
     partition_id: int
@@ -184,6 +196,17 @@ class PartitionBase:
                 extra = comm_extra_outputs[0][k]
                 if extra is not None:
                     store.set(port.tensor_id, extra, store.needs_grad(src[k + 1].tensor_id))
+
+    # -- optional per-partition timing ---------------------------------------------
+    # Set ``PartitionBase.timer`` to an object with ``begin(partition)`` / ``end(partition)``
+    # (e.g. recording HIP events) to time partitions; None costs nothing.
+    timer = None
+
+    def _timed(self):
+        t = PartitionBase.timer
+        if t is None:
+            return contextlib.nullcontext()
+        return _TimerScope(t, self)
 
     # -- stream scoping -----------------------------------------------------------
     @staticmethod
