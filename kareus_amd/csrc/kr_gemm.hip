@@ -3,117 +3,157 @@
 // Roofline: MFMA (v_mfma_f32_32x32x16_bf16, 32768 FLOP per wave instruction).  Algorithmic
 // work per launch is 2*M*N*K FLOP.
 //
-// Structure
-//   * A workgroup owns a BM x BN tile of C and walks K in steps of 64.  Waves form a WM x WN
-//     grid; each wave owns TM x TN MFMA tiles of 32x32 and keeps them in accumulator
-//     registers for the whole K loop.
-//   * Operand tiles are staged in LDS, double-buffered: while the matrix cores work on
-//     K-step i from one buffer, the global loads of step i+1 are in flight into registers
-//     and are written to the other buffer afterwards — one barrier per K-step.
-//   * Global loads are 16-byte vectors along whichever dimension is contiguous in memory, so
-//     every layout reads full cache lines.  An operand whose contraction dimension is the
-//     contiguous one ("K-major") is fetched from LDS with ds_read_b128; an operand whose
-//     contraction dimension is the row index ("transposed", the weight in dgrad and both
-//     operands in wgrad) is fetched with the gfx950 transposing LDS read ds_read_b64_tr_b16,
-//     which returns, per lane, four consecutive contraction elements of one output row from
-//     a tile stored row-per-contraction-index.  No transposed copy of any operand is made.
+// Structure ("8-wave ping-pong")
+//   * A workgroup of 8 waves owns a 256 x 256 tile of C and walks K in steps of 64.  Each wave
+//     owns 128 x 64 of the tile as 4 x 2 MFMA tiles of 32x32 held in registers for the whole
+//     K loop.
+//   * The waves form two groups of four, one wave of each group per SIMD.  Time is cut into
+//     half-periods by workgroup barriers.  In every half-period one group only issues MFMAs
+//     (all 32 of a K-step, operands already in registers) while the other group only moves
+//     data: it reads its operand fragments for the same K-step out of LDS and (group 0) issues
+//     the global loads of a later K-step.  Then the roles swap.  The matrix pipe of every SIMD
+//     always has exactly one wave feeding it, and no wave ever waits on memory in the middle
+//     of its MFMA burst.
+//   * Global memory goes straight into LDS (global_load_lds_dwordx4): no staging registers, no
+//     LDS store instructions.  The hardware places the 64 lanes of such a load contiguously in
+//     LDS, so bank conflicts are avoided by an XOR swizzle applied on the *global* side — each
+//     lane fetches the 16-byte chunk that belongs at its LDS slot.  Two LDS stages; the tile
+//     of K-step k+2 is requested while step k is being consumed.
+//   * Loads are 16-byte vectors along whichever dimension is contiguous in memory.  An operand
+//     whose contraction dimension is contiguous ("K-major") is fetched from LDS with
+//     ds_read_b128; an operand whose contraction dimension is the row index ("transposed": the
+//     weight in dgrad, both operands in wgrad) with the transposing LDS read
+//     ds_read_b64_tr_b16.  No transposed copy of any operand is ever made.
 //   * The MFMA is issued with the operands swapped (the B tile feeds the instruction's A
-//     port), so a lane ends up with four consecutive N-columns of one C row: the epilogue
+//     port), so a lane ends up with four consecutive N-columns of one C row and the epilogue
 //     stores 8-byte bf16 quads contiguous along the row.
-//   * LDS rows are padded (K-major: 64 -> 72 elements; transposed: +32 elements) so that the
-//     16 lanes served together hit distinct banks for both the vector stores and the
-//     fragment reads.
-//   * Workgroup ids are remapped so that the 32 tiles resident on one XCD (ids congruent
-//     mod 8) form a compact GROUP_M x n rectangle of C and share A/B panels in that XCD's L2.
-#include <mutex>
-
+//   * Rows beyond the matrix edge are clamped to the last valid row instead of predicated: an
+//     output element depends only on its own A row and B row, and out-of-range outputs are
+//     never stored.  A contraction tail (K not a multiple of 64) is zeroed in LDS after its
+//     tile has landed.
+//   * Workgroup ids are remapped so that the tiles resident on one XCD (ids congruent mod 8)
+//     form a compact band of C and share A/B panels in that XCD's L2.
 #include "kr_common.h"
 
 namespace {
 
 constexpr int BK = 64;
-constexpr int LDK = BK + 8;  // padded row length (elements) of a K-major LDS tile
+constexpr int BM = 256, BN = 256;
+constexpr int TM = 4, TN = 2;  // 32x32 MFMA tiles per wave: 128 rows x 64 columns
+constexpr int NTHREADS = 512;
+constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
+constexpr int STAGE = 2 * TILE;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;
 
-template <int ROWS>
-struct TileGeom {
-  // K-major:    [ROWS][LDK]
-  // transposed: [BK][ROWS + 32]
-  static constexpr int LDT = ROWS + 32;
-  static constexpr int ELEMS = ROWS * LDK;  // == BK * LDT when ROWS == 256; take the max
-  static constexpr int ELEMS_T = BK * LDT;
-  static constexpr int SIZE = ELEMS > ELEMS_T ? ELEMS : ELEMS_T;
-};
-
-// ---- global -> registers -> LDS staging of one operand tile -------------------------------
-template <int ROWS, bool TRANSPOSED, int NT>
-struct Stager {
-  static constexpr int CHUNKS = ROWS * BK / 8;
-  static constexpr int PER_THREAD = CHUNKS / NT;
-  static_assert(CHUNKS % NT == 0, "tile must divide evenly over the threads");
-  bf16x8 regs[PER_THREAD];
-
-  // rows_total: extent of the non-contraction dimension; k_total: contraction extent
-  __device__ __forceinline__ void load(const bf16* __restrict__ base, int64_t ld, int row0, int k0,
-                                       int rows_total, int k_total, int tid) {
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + i * NT;
-      if (!TRANSPOSED) {
-        const int r = c >> 3, kc = (c & 7) * 8;
-        const bool ok = (row0 + r < rows_total) && (k0 + kc < k_total);
-        regs[i] = ok ? ldg8(base + (int64_t)(row0 + r) * ld + k0 + kc) : zero8();
-      } else {
-        constexpr int CPR = ROWS / 8;  // chunks per contraction row
-        const int kr = c / CPR, rc = (c % CPR) * 8;
-        const bool ok = (k0 + kr < k_total) && (row0 + rc < rows_total);
-        regs[i] = ok ? ldg8(base + (int64_t)(k0 + kr) * ld + row0 + rc) : zero8();
-      }
-    }
-  }
-  __device__ __forceinline__ void store(bf16* tile, int tid) const {
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int c = tid + i * NT;
-      if (!TRANSPOSED) {
-        const int r = c >> 3, kc = (c & 7) * 8;
-        *reinterpret_cast<bf16x8*>(tile + r * LDK + kc) = regs[i];
-      } else {
-        constexpr int CPR = ROWS / 8;
-        const int kr = c / CPR, rc = (c % CPR) * 8;
-        *reinterpret_cast<bf16x8*>(tile + kr * TileGeom<ROWS>::LDT + rc) = regs[i];
-      }
-    }
-  }
-};
-
-// ---- LDS -> MFMA operand fragment: lane gets row (row0 + lane%32), k = 16*kk + 8*(lane/32)+0..7
-template <int ROWS, bool TRANSPOSED>
-__device__ __forceinline__ bf16x8 read_frag(const bf16* tile, int row0, int kk, int lane) {
-  if (!TRANSPOSED) {
-    return *reinterpret_cast<const bf16x8*>(tile + (row0 + (lane & 31)) * LDK + kk * 16 +
-                                            (lane >> 5) * 8);
-  } else {
-    // Transposing read: within each group of 16 lanes, lane p supplies the address of 4
-    // consecutive rows-of-C elements in contraction row (p/4); lane p receives element p of
-    // the 16 covered rows-of-C for the group's 4 contraction rows.
-    constexpr int LDT = TileGeom<ROWS>::LDT;
-    const int p = lane & 15;
-    const int krow = kk * 16 + (lane >> 5) * 8 + (p >> 2);
-    const int col = row0 + ((lane >> 4) & 1) * 16 + (p & 3) * 4;
-    const bf16* a0 = tile + krow * LDT + col;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 4 * LDT));
-    union {
-      struct { s16x4 lo, hi; } s;
-      bf16x8 v;
-    } u;
-    u.s.lo = lo;
-    u.s.hi = hi;
-    return u.v;
-  }
+// ---- LDS layouts (element offsets inside one operand tile) ----------------------------------
+// K-major tile [256 rows][64]: 128-byte rows, 16-byte chunk index XORed with (row>>1)&7.
+__device__ __forceinline__ int kmajor_off(int row, int chunk) {
+  return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
 }
+// transposed tile [64 k-rows][256]: 512-byte rows, chunk index XORed with 4*(krow&3).
+__device__ __forceinline__ int transp_off(int krow, int col) {
+  return krow * 256 + ((((col >> 3) ^ ((krow & 3) << 2))) << 3) + (col & 7);
+}
+
+// ---- direct global -> LDS tile loads, issued by the 4 waves of the loading group -----------
+// One wave-level load moves 1 KiB into LDS at [base + lane*16].  Block b of a K-major tile
+// holds rows 8b..8b+7; block b of a transposed tile holds contraction rows 2b, 2b+1.
+template <bool TRANSPOSED>
+struct TileLoader {
+  // K-major:    load i covers tile row r0 + 32*i (clamped to rmax), 16-byte chunk `chunk`
+  // transposed: load i covers contraction row k0 + 8*i, column offset `chunk` (clamped)
+  int r0, rmax, chunk;
+  int64_t ld;
+  __device__ __forceinline__ void init(int64_t ld_, int row0, int rows_total, int wave4, int lane) {
+    ld = ld_;
+    if (!TRANSPOSED) {
+      const int row = 8 * wave4 + (lane >> 3);  // + 32*i; (row >> 1) & 7 does not depend on i
+      chunk = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+      r0 = row0 + row;
+      rmax = rows_total - 1;
+    } else {
+      const int krow = 2 * wave4 + (lane >> 5);  // + 8*i; krow & 3 does not depend on i
+      int c = row0 + ((lane & 31) ^ ((krow & 3) << 2)) * 8;
+      chunk = c + 8 <= rows_total ? c : rows_total - 8;
+      r0 = krow;
+      rmax = 0;
+    }
+  }
+  __device__ __forceinline__ uint32_t goff(int i) const {
+    if (!TRANSPOSED) {
+      int r = r0 + 32 * i;
+      r = r < rmax ? r : rmax;
+      return (uint32_t)(r * (int)ld + chunk);
+    }
+    return (uint32_t)((r0 + 8 * i) * (int)ld + chunk);
+  }
+  // contraction index (relative to the K-step) covered by load i of this lane
+  __device__ __forceinline__ int k_of(int i, int wave4, int lane) const {
+    if (!TRANSPOSED) {
+      const int row = 8 * wave4 + (lane >> 3);
+      return ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+    }
+    return 2 * (wave4 + 4 * i) + (lane >> 5);
+  }
+  __device__ __forceinline__ void issue(const bf16* __restrict__ kbase, bf16* tile, int wave4) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int b = wave4 + 4 * i;
+      __builtin_amdgcn_global_load_lds(kbase + goff(i), (KR_LDS void*)(tile + b * 512), 16, 0, 0);
+    }
+  }
+  // zero this lane's chunks whose contraction index is >= k_valid (tile already landed)
+  __device__ __forceinline__ void zero_tail(bf16* tile, int k_valid, int wave4, int lane) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int b = wave4 + 4 * i;
+      if (k_of(i, wave4, lane) >= k_valid)
+        *reinterpret_cast<bf16x8*>(tile + b * 512 + lane * 8) = zero8();
+    }
+  }
+};
+
+// ---- LDS -> MFMA operand fragments ----------------------------------------------------------
+// Fragment (t, kk): lane gets tile row (row0 + 32*t + lane%32), k = 16*kk + 8*(lane/32) + 0..7.
+// Per-lane base offsets are computed once; everything that varies inside the K loop is an
+// instruction immediate.
+template <bool TRANSPOSED, int NTILES>
+struct FragReader {
+  // K-major: one base per kk (the swizzle XOR depends on kk), tile index t is an immediate
+  // transposed: one base per t (the XOR depends on the column), kk / half are immediates
+  int base[TRANSPOSED ? NTILES : BK / 16];
+  __device__ __forceinline__ void init(int row0, int lane) {
+    if (!TRANSPOSED) {
+      const int row = row0 + (lane & 31);
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) base[kk] = kmajor_off(row, 2 * kk + (lane >> 5));
+    } else {
+      const int p = lane & 15;
+      const int krow = (lane >> 5) * 8 + (p >> 2);
+#pragma unroll
+      for (int t = 0; t < NTILES; ++t)
+        base[t] = transp_off(krow, row0 + 32 * t + ((lane >> 4) & 1) * 16 + (p & 3) * 4);
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const bf16* tile, int t, int kk) const {
+    if (!TRANSPOSED) {
+      return *reinterpret_cast<const bf16x8*>(tile + base[kk] + t * 32 * BK);
+    } else {
+      // Transposing read: within each group of 16 lanes, lane p supplies the address of 4
+      // consecutive row-of-C elements in contraction row (p/4); it receives, for its own
+      // row-of-C, the elements of the group's 4 contraction rows.
+      const bf16* a0 = tile + base[t] + kk * 16 * 256;
+      union {
+        struct { s16x4 lo, hi; } s;
+        bf16x8 v;
+      } u;
+      u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
+      u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 4 * 256));
+      return u.v;
+    }
+  }
+};
 
 __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, int tiles_n,
                                             int& tm, int& tn) {
@@ -131,23 +171,26 @@ __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, i
   tn = in_band / band_rows;
 }
 
-template <bool A_T, bool B_T, int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(const bf16* __restrict__ A, int64_t lda,
-                                                          const bf16* __restrict__ B, int64_t ldb,
-                                                          bf16* __restrict__ C, int64_t ldc, int M,
-                                                          int N, int K, int accumulate) {
-  constexpr int NT = WM * WN * 64;
-  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr int A_SIZE = TileGeom<BM>::SIZE, B_SIZE = TileGeom<BN>::SIZE;
+template <bool A_T, bool B_T>
+__global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int64_t lda,
+                                                        const bf16* __restrict__ B, int64_t ldb,
+                                                        bf16* __restrict__ C, int64_t ldc, int M,
+                                                        int N, int K, int accumulate) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  constexpr int STAGE = A_SIZE + B_SIZE;  // buffer s: A tile at s*STAGE, B tile right after it
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / WN, wn = wave % WN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int group = wave >> 2;  // 0: loads + computes first, 1: computes second
+  const int wave4 = wave & 3;
+  const int wm = group, wn = wave4;  // wave tile: rows wm*128.., columns wn*64..
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   int tile_m, tile_n;
   remap_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int nk = (K + BK - 1) / BK;
+  const int k_tail = K - (nk - 1) * BK;  // valid contraction rows of the last K-step (1..64)
+  const int64_t a_step = A_T ? (int64_t)BK * lda : BK;
+  const int64_t b_step = B_T ? (int64_t)BK * ldb : BK;
 
   f32x16 acc[TN][TM];
 #pragma unroll
@@ -157,42 +200,81 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(const bf16* __restric
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
 
-  Stager<BM, A_T, NT> sa;
-  Stager<BN, B_T, NT> sb;
-  const int nk = (K + BK - 1) / BK;
+  bf16x8 af[BK / 16][TM], bfr[BK / 16][TN];
 
-  sa.load(A, lda, m0, 0, M, K, tid);
-  sb.load(B, ldb, n0, 0, N, K, tid);
-  sa.store(smem, tid);
-  sb.store(smem + A_SIZE, tid);
-  __syncthreads();
-
-  for (int ks = 0; ks < nk; ++ks) {
-    const int cur = ks & 1;
-    if (ks + 1 < nk) {
-      sa.load(A, lda, m0, (ks + 1) * BK, M, K, tid);
-      sb.load(B, ldb, n0, (ks + 1) * BK, N, K, tid);
-    }
-    const bf16* at = smem + cur * STAGE;
-    const bf16* bt = at + A_SIZE;
+  FragReader<A_T, TM> fa;
+  FragReader<B_T, TN> fb;
+  fa.init(wm * TM * 32, lane);
+  fb.init(wn * TN * 32, lane);
+  auto read_frags = [&](int stage) {
+    const bf16* at = smem + stage * STAGE;
+    const bf16* bt = at + TILE;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[TM], bfr[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = read_frag<BM, A_T>(at, (wm * TM + i) * 32, kk, lane);
+      for (int i = 0; i < TM; ++i) af[kk][i] = fa.read(at, i, kk);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bfr[j] = read_frag<BN, B_T>(bt, (wn * TN + j) * 32, kk, lane);
+      for (int j = 0; j < TN; ++j) bfr[kk][j] = fb.read(bt, j, kk);
+    }
+  };
+  auto compute = [&]() {
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[j][i], 0, 0, 0);
+          acc[j][i] =
+              __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[kk][j], af[kk][i], acc[j][i], 0, 0, 0);
+    __builtin_amdgcn_s_setprio(0);
+  };
+
+  if (group == 0) {
+    TileLoader<A_T> la;
+    TileLoader<B_T> lb;
+    la.init(lda, m0, M, wave4, lane);
+    lb.init(ldb, n0, N, wave4, lane);
+    auto issue_tile = [&](int t) {
+      // The per-lane load coordinates are recomputed here from an opaque copy of the lane id:
+      // keeping them alive across the MFMA phases would push the wave over its register budget.
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));
+      la.init(lda, m0, M, wave4, l2);
+      lb.init(ldb, n0, N, wave4, l2);
+      bf16* st = smem + (t & 1) * STAGE;
+      la.issue(A + t * a_step, st, wave4);
+      lb.issue(B + t * b_step, st + TILE, wave4);
+    };
+    auto land_tile = [&](int t) {  // all of this wave's outstanding loads are done; fix a K tail
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
+      if (t == nk - 1 && k_tail < BK) {
+        bf16* st = smem + (t & 1) * STAGE;
+        la.zero_tail(st, k_tail, wave4, lane);
+        lb.zero_tail(st + TILE, k_tail, wave4, lane);
+      }
+    };
+    issue_tile(0);
+    land_tile(0);
+    if (nk > 1) issue_tile(1);
+    __syncthreads();  // tile 0 visible to everyone
+    read_frags(0);
+    for (int ks = 0; ks < nk; ++ks) {
+      __syncthreads();  // half-period 2ks: this group computes, the other reads fragments
+      compute();
+      if (ks + 1 < nk) land_tile(ks + 1);
+      __syncthreads();  // half-period 2ks+1: this group moves data, the other computes
+      if (ks + 2 < nk) issue_tile(ks + 2);  // stage ks&1 is free: both groups hold step ks in registers
+      if (ks + 1 < nk) read_frags((ks + 1) & 1);
     }
-    if (ks + 1 < nk) {
-      sa.store(smem + (cur ^ 1) * STAGE, tid);
-      sb.store(smem + (cur ^ 1) * STAGE + A_SIZE, tid);
-    }
+  } else {
     __syncthreads();
+    for (int ks = 0; ks < nk; ++ks) {
+      __syncthreads();
+      read_frags(ks & 1);
+      __syncthreads();
+      compute();
+    }
   }
 
   // epilogue: lane holds C[m][n..n+3] for m = tile row (lane%32), n = 8g + 4*(lane/32)
@@ -223,22 +305,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_kernel(const bf16* __restric
   }
 }
 
-template <bool A_T, bool B_T, int WM, int WN, int TM, int TN>
+// the three layouts the library serves
+template __global__ void gemm_kernel<false, false>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
+                                                   int64_t, int, int, int, int);
+template __global__ void gemm_kernel<false, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
+                                                  int64_t, int, int, int, int);
+template __global__ void gemm_kernel<true, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
+                                                 int64_t, int, int, int, int);
+
+template <bool A_T, bool B_T>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, hipStream_t stream) {
-  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr size_t lds_bytes = 2 * (TileGeom<BM>::SIZE + TileGeom<BN>::SIZE) * sizeof(bf16);
-  auto kernel = gemm_kernel<A_T, B_T, WM, WN, TM, TN>;
-  static std::once_flag once;
-  static hipError_t attr_status = hipSuccess;
-  std::call_once(once, [&] {
-    attr_status = hipFuncSetAttribute((const void*)kernel,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  });
+  constexpr size_t lds_bytes = 2 * STAGE * sizeof(bf16);
+  // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
+  static const hipError_t attr_status =
+      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(WM * WN * 64), lds_bytes, stream, A, lda, B, ldb, C,
-                     ldc, M, N, K, accumulate);
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles), dim3(NTHREADS), lds_bytes, stream, A, lda,
+                     B, ldb, C, ldc, M, N, K, accumulate);
   return kr_launch_status();
 }
 
@@ -250,6 +336,9 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return KR_EINVAL;
   if (!kr_aligned16(A) || !kr_aligned16(B) || !kr_aligned16(C)) return KR_EINVAL;
   if ((M | N | K) % 8 || (lda | ldb | ldc) % 8) return KR_EUNSUPPORTED;
+  // chunk offsets inside an operand are kept in 32 bits
+  const int64_t a_rows = layout == KR_GEMM_NT ? 64 : M, b_rows = layout == KR_GEMM_TN ? N : 64;
+  if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31) return KR_EUNSUPPORTED;
   const bf16* a = (const bf16*)A;
   const bf16* b = (const bf16*)B;
   bf16* c = (bf16*)C;
@@ -257,13 +346,13 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   switch (layout) {
     case KR_GEMM_TN:  // A [M,K], B [N,K]
       if (lda < K || ldb < K || ldc < N) return KR_EINVAL;
-      return launch<false, false, 2, 4, 4, 2>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<false, false>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
     case KR_GEMM_NN:  // A [M,K], B [K,N]
       if (lda < K || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<false, true, 2, 4, 4, 2>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<false, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
     case KR_GEMM_NT:  // A [K,M], B [K,N]
       if (lda < M || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<true, true, 2, 4, 4, 2>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<true, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
     default:
       return KR_EINVAL;
   }
