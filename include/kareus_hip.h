@@ -69,12 +69,16 @@ int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void*
  * (hd contiguous; strides multiples of 8).  freqs: [s, hd] fp32 angles; all hd channels are
  * rotated, halves layout: out = t*cos(f) + rotate_half(t)*sin(f), rotate_half([a,b]) = [-b,a].
  * backward != 0 rotates by -f (the gradient of the forward).  out may alias t.
+ * Heads are taken in groups of group_size; only the first group_rotate heads of each group are
+ * rotated, the others are copied (or left alone when out aliases t).  (1, 1) rotates every
+ * head; (nq/nkv + 2, nq/nkv + 1) rotates the query and key heads of a fused QKV projection
+ * output in place and leaves its value heads untouched.
  * hd must be a multiple of 16 and at most 256.                                             */
 int kr_rope(const void* t, void* out, const float* freqs,
             int s, int b, int heads, int hd,
             int64_t t_stride_s, int64_t t_stride_b, int64_t t_stride_h,
             int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
-            int backward, void* stream);
+            int backward, int group_size, int group_rotate, void* stream);
 
 /* ---- SwiGLU ----------------------------------------------------------------------------
  * Replaces the Inductor kernels of fused_swiglu_forward / fused_swiglu_backward
@@ -95,29 +99,37 @@ int kr_add(const void* a, const void* b, void* out, int64_t n, void* stream);
 /* ---- Causal grouped-query attention ----------------------------------------------------
  * Replaces flash_attn_2_cuda.fwd / bwd as called from
  * kareus/flash_attn/flash_attn_interface.py:66-80, 174-194.
- * q, o, dq, do: [s, b, nq, hd]; k, v, dk, dv: [s, b, nkv, hd]; bf16, element (si, bi, h, d) at
- * si*stride_s + bi*stride_b + h*stride_h + d.  lse: [b, nq, s] fp32 contiguous
- * (natural log-sum-exp of the scaled, masked scores).  Query head h reads KV head
- * h / (nq/nkv).  Causal, query i sees keys <= i.  hd must be 128; s a multiple of 128.
- * kr_attn_bwd also needs a workspace of kr_attn_bwd_workspace_bytes() bytes.               */
+ * bf16 tensors, head dimension contiguous.  Key-like tensors (k, v, dk, dv), nkv heads:
+ *   element (si, bi, kvh, d) at si*stride_s + bi*stride_b + kvh*stride_h + d.
+ * Query-like tensors (q, o, dout, dq), nq heads in nkv groups of per = nq/nkv:
+ *   element (si, bi, h, d) at si*stride_s + bi*stride_b + (h/per)*stride_g + (h%per)*stride_h + d.
+ * A dense [s, b, nq, hd] tensor has stride_g = per*stride_h; the grouped form lets the kernels
+ * read q, k, v straight out of the fused QKV projection output, whose features are laid out
+ * per KV group as (its query heads, its key head, its value head)
+ * (kareus/megatron/core/extensions/ops/qkv_postprocess.py:84-109), and write dq, dk, dv
+ * straight into a buffer of that layout.
+ * lse: [b, nq, s] fp32 contiguous (natural log-sum-exp of the scaled, masked scores).
+ * Query head h reads KV head h/per.  Causal, query i sees keys <= i.
+ * hd must be 128; s a multiple of 128.  All strides multiples of 8.
+ * kr_attn_bwd needs a workspace of kr_attn_bwd_workspace_bytes() bytes (16-byte aligned).   */
 int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                 int s, int b, int nq, int nkv, int hd, float scale,
-                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_h,
+                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
                 int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
                 int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
-                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
+                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
                 void* stream);
 size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);
 int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                 const void* o, const float* lse,
                 void* dq, void* dk, void* dv, void* workspace,
                 int s, int b, int nq, int nkv, int hd, float scale,
-                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_h,
+                int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
                 int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
                 int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
-                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_h,
-                int64_t do_stride_s, int64_t do_stride_b, int64_t do_stride_h,
-                int64_t dq_stride_s, int64_t dq_stride_b, int64_t dq_stride_h,
+                int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
+                int64_t do_stride_s, int64_t do_stride_b, int64_t do_stride_g, int64_t do_stride_h,
+                int64_t dq_stride_s, int64_t dq_stride_b, int64_t dq_stride_g, int64_t dq_stride_h,
                 int64_t dk_stride_s, int64_t dk_stride_b, int64_t dk_stride_h,
                 int64_t dv_stride_s, int64_t dv_stride_b, int64_t dv_stride_h,
                 void* stream);

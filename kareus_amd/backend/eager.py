@@ -60,10 +60,14 @@ class EagerBackend:
         return out.to(t.dtype)
 
     def rope_fwd(self, t: Tensor, freqs: Tensor) -> Tensor:
+        if t.dim() == 5:  # grouped [s, b, ng, per, hd] query view
+            t = t.flatten(2, 3)
         return self._rope(t, freqs, 1.0)
 
     # The gradient of a rotation is the rotation by the opposite angle (rope_utils.py:207-222).
     def rope_bwd(self, g: Tensor, freqs: Tensor) -> Tensor:
+        if g.dim() == 5:
+            g = g.flatten(2, 3)
         return self._rope(g, freqs, -1.0)
 
     # y = silu(x1) * x2 with x1, x2 = chunk(x, 2, -1)
@@ -87,6 +91,8 @@ class EagerBackend:
     # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32
     # (kareus/flash_attn/flash_attn_interface.py:473-493).
     def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
+        if q.dim() == 5:
+            q = q.flatten(2, 3)
         s, b, nq, hd = q.shape
         nkv = k.shape[2]
         rep = nq // nkv
@@ -103,6 +109,8 @@ class EagerBackend:
         return o.to(q.dtype), lse.contiguous()
 
     def attn_bwd(self, do, q, k, v, o, lse, scale: float, causal: bool = True):
+        if q.dim() == 5:
+            q = q.flatten(2, 3)
         s, b, nq, hd = q.shape
         nkv = k.shape[2]
         rep = nq // nkv

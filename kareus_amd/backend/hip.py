@@ -29,13 +29,13 @@ _SIGNATURES = {
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_void_p]),
     "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
-                + [_c_int, _c_void_p]),
+                + [_c_int, _c_int, _c_int, _c_void_p]),
     "kr_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_swiglu_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_add": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
-    "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 12 + [_c_void_p]),
+    "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_void_p]),
     "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
-    "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 24 + [_c_void_p]),
+    "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_void_p]),
 }
 
 KR_GEMM_TN, KR_GEMM_NN, KR_GEMM_NT = 0, 1, 2
@@ -137,35 +137,49 @@ class HipBackend:
         return dx, dgamma
 
     # -- RoPE -------------------------------------------------------------------------
-    def _rope(self, t: Tensor, freqs: Tensor, backward: bool, out: Tensor = None) -> Tensor:
-        self._dev(t, freqs)
-        self._bf16(t)
+    def _freqs2d(self, freqs: Tensor, hd: int) -> Tensor:
         if freqs.dtype != torch.float32:
             raise RuntimeError("the rotary table must be fp32")
-        s, b, heads, hd = t.shape
-        if t.stride(3) != 1:
-            raise RuntimeError("rotary input needs a contiguous head dimension")
         if freqs.shape[-1] != hd:
             raise RuntimeError("partial rotary (rot_dim < head_dim) is not supported")
         f2d = freqs.reshape(freqs.shape[0], hd)
-        if not f2d.is_contiguous():
-            f2d = f2d.contiguous()
+        return f2d if f2d.is_contiguous() else f2d.contiguous()
+
+    def _rope(self, t: Tensor, freqs: Tensor, backward: bool, out: Tensor = None,
+              group_size: int = 1, group_rotate: int = 1) -> Tensor:
+        self._dev(t, freqs)
+        self._bf16(t)
+        s, b, heads, hd = t.shape
+        if t.stride(3) != 1:
+            raise RuntimeError("rotary input needs a contiguous head dimension")
+        f2d = self._freqs2d(freqs, hd)
         if out is None:
             out = torch.empty((s, b, heads, hd), dtype=t.dtype, device=t.device)
         rc = self.lib.kr_rope(t.data_ptr(), out.data_ptr(), f2d.data_ptr(), s, b, heads, hd,
                               t.stride(0), t.stride(1), t.stride(2),
-                              out.stride(0), out.stride(1), out.stride(2), int(backward), self._stream())
+                              out.stride(0), out.stride(1), out.stride(2), int(backward),
+                              group_size, group_rotate, self._stream())
         self._check(rc, "kr_rope")
         return out
 
     def rope_fwd(self, t: Tensor, freqs: Tensor) -> Tensor:
+        if t.dim() == 5:
+            t = t.flatten(2, 3)
         return self._rope(t, freqs, False)
 
     def rope_bwd(self, g: Tensor, freqs: Tensor) -> Tensor:
+        if g.dim() == 5:
+            g = g.flatten(2, 3)
         return self._rope(g, freqs, True)
 
-    def rope_inplace(self, t: Tensor, freqs: Tensor, backward: bool) -> Tensor:
-        return self._rope(t, freqs, backward, out=t)
+    def rope_fused_inplace(self, fused: Tensor, per: int, freqs: Tensor, backward: bool) -> None:
+        """Rotate the query and key heads of a fused QKV buffer [s, b, ng, per+2, hd] in place
+        (one launch); the value heads are left untouched."""
+        s, b, ng, slots, hd = fused.shape
+        if slots != per + 2 or not fused.is_contiguous():
+            raise RuntimeError("fused QKV buffer must be contiguous [s, b, ng, per+2, hd]")
+        flat = fused.view(s, b, ng * slots, hd)
+        self._rope(flat, freqs, backward, out=flat, group_size=slots, group_rotate=per + 1)
 
     # -- SwiGLU / add -------------------------------------------------------------------
     def swiglu_fwd(self, x: Tensor) -> Tensor:
@@ -201,45 +215,79 @@ class HipBackend:
 
     # -- attention ----------------------------------------------------------------------
     @staticmethod
-    def _sbh(t: Tensor):
-        if t.stride(3) != 1:
+    def _k_strides(t: Tensor):
+        if t.stride(-1) != 1:
             raise RuntimeError("attention tensors need a contiguous head dimension")
         return t.stride(0), t.stride(1), t.stride(2)
+
+    @staticmethod
+    def _q_strides(t: Tensor, per: int):
+        """(seq, batch, group, head-in-group) strides of a dense [s, b, nq, hd] or a grouped
+        [s, b, ng, per, hd] query-like tensor."""
+        if t.stride(-1) != 1:
+            raise RuntimeError("attention tensors need a contiguous head dimension")
+        if t.dim() == 5:
+            return t.stride(0), t.stride(1), t.stride(2), t.stride(3)
+        return t.stride(0), t.stride(1), per * t.stride(2), t.stride(2)
+
+    @staticmethod
+    def _q_dims(q: Tensor, k: Tensor):
+        s, b = q.shape[0], q.shape[1]
+        nkv, hd = k.shape[2], k.shape[3]
+        nq = q.shape[2] * q.shape[3] if q.dim() == 5 else q.shape[2]
+        if q.dim() == 5 and q.shape[2] != nkv:
+            raise RuntimeError("grouped query tensor must have one group per KV head")
+        return s, b, nq, nkv, hd
 
     def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
         if not causal:
             raise RuntimeError("only causal attention is implemented")
         self._dev(q, k, v)
         self._bf16(q, k, v)
-        s, b, nq, hd = q.shape
-        nkv = k.shape[2]
+        s, b, nq, nkv, hd = self._q_dims(q, k)
+        per = nq // nkv
         o = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
         lse = torch.empty((b, nq, s), dtype=torch.float32, device=q.device)
         rc = self.lib.kr_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-                                  s, b, nq, nkv, hd, scale, *self._sbh(q), *self._sbh(k), *self._sbh(v),
-                                  *self._sbh(o), self._stream())
+                                  s, b, nq, nkv, hd, scale, *self._q_strides(q, per), *self._k_strides(k),
+                                  *self._k_strides(v), *self._q_strides(o, per), self._stream())
         self._check(rc, f"kr_attn_fwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
         return o, lse
 
     def attn_bwd(self, do: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor,
                  scale: float, causal: bool = True):
+        """Returns (dq, dk, dv).  If ``q`` is a grouped [s, b, ng, per, hd] view, the three
+        gradients are views of one buffer laid out like the fused QKV projection output and
+        carry it as ``_kr_mixed`` so the QKV-split backward can hand it on without a copy."""
         if not causal:
             raise RuntimeError("only causal attention is implemented")
         self._dev(do, q, k, v, o, lse)
         self._bf16(do, q, k, v, o)
-        s, b, nq, hd = q.shape
-        nkv = k.shape[2]
+        s, b, nq, nkv, hd = self._q_dims(q, k)
+        per = nq // nkv
         do4 = do.reshape(s, b, nq, hd)
         o4 = o.reshape(s, b, nq, hd)
-        dq = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
-        dk = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
-        dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
+        mixed = None
+        if q.dim() == 5:
+            fused = torch.empty((s, b, nkv, per + 2, hd), dtype=q.dtype, device=q.device)
+            dq, dk, dv = fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1]
+            mixed = fused.view(s, b, nkv * (per + 2) * hd)
+        else:
+            dq = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
+            dk = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
+            dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
         nbytes = self.lib.kr_attn_bwd_workspace_bytes(s, b, nq, nkv, hd)
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
         rc = self.lib.kr_attn_bwd(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
                                   lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
                                   s, b, nq, nkv, hd, scale,
-                                  *self._sbh(q), *self._sbh(k), *self._sbh(v), *self._sbh(o4), *self._sbh(do4),
-                                  *self._sbh(dq), *self._sbh(dk), *self._sbh(dv), self._stream())
+                                  *self._q_strides(q, per), *self._k_strides(k), *self._k_strides(v),
+                                  *self._q_strides(o4, per), *self._q_strides(do4, per),
+                                  *self._q_strides(dq, per), *self._k_strides(dk), *self._k_strides(dv),
+                                  self._stream())
         self._check(rc, f"kr_attn_bwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
+        if mixed is not None:
+            for t in (dq, dk, dv):
+                t._kr_mixed = mixed
+                t._kr_fused5 = fused
         return dq, dk, dv

@@ -18,8 +18,6 @@
 //   P nor V is ever transposed through memory.
 // Tensors are addressed through (seq, batch, head) strides, so sequence-major [s, b, h, d]
 // views of the fused QKV projection are consumed in place.
-#include <mutex>
-
 #include "kr_common.h"
 
 namespace {
@@ -84,8 +82,9 @@ __device__ __forceinline__ bf16x8 read_vt_frag(const bf16* vt, int key0, int d0,
 __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
-    int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
-    int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb, int64_t o_sh) {
+    int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+    int64_t o_sg, int64_t o_sh) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   constexpr int STAGE = K_ELEMS + V_ELEMS;
 
@@ -95,12 +94,13 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
   const int qt = nqt - 1 - (lid % nqt);  // longest rows first inside each (batch, head)
   const int head = (lid / nqt) % nq;
   const int bi = lid / (nqt * nq);
-  const int kvh = head / (nq / nkv);
+  const int per = nq / nkv;
+  const int kvh = head / per, hj = head % per;  // KV group and position inside the group
 
   const int q0 = qt * BQ;
   const int qw0 = q0 + wave * 32;
   const int qrow = qw0 + (lane & 31);
-  const bf16* qp = q + (int64_t)bi * q_sb + (int64_t)head * q_sh + (int64_t)qrow * q_ss;
+  const bf16* qp = q + (int64_t)bi * q_sb + kvh * q_sg + hj * q_sh + (int64_t)qrow * q_ss;
   const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
   const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
 
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
   const float inv_l = 1.0f / l_tot;
-  bf16* op = o + (int64_t)bi * o_sb + (int64_t)head * o_sh + (int64_t)qrow * o_ss;
+  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qrow * o_ss;
 #pragma unroll
   for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
@@ -214,40 +214,43 @@ static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
 
 extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
                            int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
-                           int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh, int64_t v_ss,
-                           int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb, int64_t o_sh,
-                           void* stream) {
+                           int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
+                           int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+                           int64_t o_sg, int64_t o_sh, void* stream) {
   if (!q || !k || !v || !o || !lse) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
   if (!kr_aligned16(q) || !kr_aligned16(k) || !kr_aligned16(v) || !kr_aligned16(o)) return KR_EINVAL;
-  if ((q_ss | q_sb | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sh) % 8)
+  if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
+       o_sh) % 8)
     return KR_EINVAL;
   constexpr size_t lds_bytes = 2 * (K_ELEMS + V_ELEMS) * sizeof(bf16);
-  static std::once_flag once;
-  static hipError_t attr_status = hipSuccess;
-  std::call_once(once, [&] {
-    attr_status = hipFuncSetAttribute((const void*)attn_fwd_kernel,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  });
+  static const hipError_t attr_status = hipFuncSetAttribute(
+      (const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int blocks = (s / BQ) * nq * b;
   hipLaunchKernelGGL(attn_fwd_kernel, dim3(blocks), dim3(FWD_THREADS), lds_bytes,
                      (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
-                     lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sh, k_ss, k_sb, k_sh, v_ss, v_sb,
-                     v_sh, o_ss, o_sb, o_sh);
+                     lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                     v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
   return kr_launch_status();
 }
 
 // =============================================================================================
-// Backward.  Three launches, no atomics, deterministic:
+// Backward.  Launches: delta pre-pass, dK/dV pass, (group reduction), dQ pass.  No atomics,
+// deterministic.
 //   1. delta[b, h, i] = sum_d dO[i, d] * O[i, d]                      (HBM-bound pre-pass)
-//   2. dK, dV: a workgroup owns 128 keys of one (batch, KV head) — 32 per wave, their K and V
-//      fragments in registers — and streams every query tile at or below the diagonal, for
-//      every query head of the group, through LDS.  Per 32x32 block:
+//   2. dK, dV: a workgroup owns 128 keys of one (batch, QUERY head) — 32 per wave, their K and
+//      V fragments in registers — and streams every query tile at or below the diagonal
+//      through LDS.  Per 32x32 block:
 //        S = Q.K^T, dP = dO.V^T (rows = queries on the MFMA A port, so a lane holds one key
 //        column), P = exp2(S*c - lse), dS = P*(dP - delta), then dV^T += dO^T.P and
 //        dK^T += Q^T.dS with the Q / dO tiles read back transposed (ds_read_b64_tr_b16).
+//      With grouped-query attention several query heads share a KV head: each workgroup
+//      writes an fp32 partial for its query head and a small HBM-bound kernel sums the
+//      partials of a group (one query head per KV head: bf16 results are written directly).
+//      Splitting by query head rather than looping over the group keeps enough workgroups in
+//      flight when one GPU holds only a few KV heads (a tensor-parallel shard).
 //   3. dQ: a workgroup owns 128 queries of one (batch, head) and streams the key tiles up to
 //      the diagonal: S^T = K.Q^T, dP^T = V.dO^T (a lane holds one query row), dS^T, then
 //      dQ^T += K^T.dS^T with the K tile read back transposed.
@@ -261,6 +264,18 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
 namespace {
 
 constexpr int TILE_ELEMS = 64 * HD;  // one swizzled [64][128] tile
+
+// query-like tensors: head h of KV group g = h / per sits at g*g_ + (h % per)*h_
+struct QLayout {
+  int64_t s_, b_, g_, h_;
+  __device__ __forceinline__ int64_t at(int bi, int head, int per) const {
+    return (int64_t)bi * b_ + (head / per) * g_ + (head % per) * h_;
+  }
+};
+struct KLayout {
+  int64_t s_, b_, h_;
+  __device__ __forceinline__ int64_t at(int bi, int kvh) const { return (int64_t)bi * b_ + kvh * h_; }
+};
 
 __device__ __forceinline__ int swz_off(int row, int col) {
   const int f = ((row & 7) << 1) | ((row >> 3) & 1);
@@ -308,9 +323,8 @@ __device__ __forceinline__ bf16x8 read_cols_swz(const bf16* tile, int r0, int d0
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ dout,
                                                          const bf16* __restrict__ o,
                                                          float* __restrict__ delta, int s, int nq,
-                                                         int64_t total_rows, int64_t do_ss,
-                                                         int64_t do_sb, int64_t do_sh, int64_t o_ss,
-                                                         int64_t o_sb, int64_t o_sh) {
+                                                         int per, int64_t total_rows, QLayout dol,
+                                                         QLayout ol) {
   // 16 lanes per (batch, head, position) row of 128 channels
   const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
   const int sub = threadIdx.x & 15;
@@ -318,8 +332,8 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
   const int si = (int)(row % s);
   const int head = (int)((row / s) % nq);
   const int bi = (int)(row / ((int64_t)s * nq));
-  const bf16x8 a = ldg8(dout + bi * do_sb + head * do_sh + (int64_t)si * do_ss + sub * 8);
-  const bf16x8 b = ldg8(o + bi * o_sb + head * o_sh + (int64_t)si * o_ss + sub * 8);
+  const bf16x8 a = ldg8(dout + dol.at(bi, head, per) + (int64_t)si * dol.s_ + sub * 8);
+  const bf16x8 b = ldg8(o + ol.at(bi, head, per) + (int64_t)si * ol.s_ + sub * 8);
   float acc = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
@@ -328,14 +342,14 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
   if (sub == 0) delta[row] = acc;
 }
 
+// PARTIAL = true: fp32 results for this query head go to part_k / part_v [b, nq, s, 128]
+template <bool PARTIAL>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16* __restrict__ dk, bf16* __restrict__ dv, int s, int nq, int nkv, float scale,
-    float scale_log2, int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb,
-    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t do_ss, int64_t do_sb,
-    int64_t do_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh, int64_t dv_ss, int64_t dv_sb,
-    int64_t dv_sh) {
+    bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
+    float* __restrict__ part_v, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
+    KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   // stage layout: Q tile | dO tile | lse[64] fp32 | delta[64] fp32
   constexpr int STAGE = 2 * TILE_ELEMS + 256;  // in bf16 units (256 bf16 = 128 floats)
@@ -344,15 +358,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   const int nkt = s / 128;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int kt = lid % nkt;  // low key tiles see the most queries: they come first
-  const int kvh = (lid / nkt) % nkv;
-  const int bi = lid / (nkt * nkv);
-  const int rep = nq / nkv;
+  const int head = (lid / nkt) % nq;
+  const int bi = lid / (nkt * nq);
+  const int per = nq / nkv;
+  const int kvh = head / per;
   const int key0 = kt * 128;
   const int kw0 = key0 + wave * 32;
   const int krow = kw0 + (lane & 31);
 
-  const bf16* kp = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh + (int64_t)krow * k_ss;
-  const bf16* vp = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh + (int64_t)krow * v_ss;
+  const bf16* kp = k + kl.at(bi, kvh) + (int64_t)krow * kl.s_;
+  const bf16* vp = v + vl.at(bi, kvh) + (int64_t)krow * vl.s_;
   bf16x8 kf[HD / 16], vf[HD / 16];
 #pragma unroll
   for (int kk = 0; kk < HD / 16; ++kk) {
@@ -369,28 +384,26 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     }
 
   const int qt_first = key0 / 64;
-  const int nqt = s / 64 - qt_first;  // query tiles of 64 at or below the diagonal
-  const int niter = nqt * rep;
+  const int niter = s / 64 - qt_first;  // query tiles of 64 at or below the diagonal
+  const bf16* qb = q + ql.at(bi, head, per);
+  const bf16* dob = dout + dol.at(bi, head, per);
+  const int64_t stat0 = ((int64_t)bi * nq + head) * s;
   TileStager sq, sdo;
-  float st_lse = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
+  float st_stat = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
 
   auto stage_load = [&](int it) {
-    const int hq = it / nqt, qt = qt_first + it % nqt;
-    const int head = kvh * rep + hq;
-    const bf16* qb = q + (int64_t)bi * q_sb + (int64_t)head * q_sh;
-    const bf16* dob = dout + (int64_t)bi * do_sb + (int64_t)head * do_sh;
-    sq.load(qb, q_ss, qt * 64, tid);
-    sdo.load(dob, do_ss, qt * 64, tid);
-    const int64_t stat = ((int64_t)bi * nq + head) * s + qt * 64;
-    if (tid < 64) st_lse = lse[stat + tid] * kLog2e;
-    else if (tid < 128) st_lse = delta[stat + tid - 64];
+    const int qt = qt_first + it;
+    sq.load(qb, ql.s_, qt * 64, tid);
+    sdo.load(dob, dol.s_, qt * 64, tid);
+    if (tid < 64) st_stat = lse[stat0 + qt * 64 + tid] * kLog2e;
+    else if (tid < 128) st_stat = delta[stat0 + qt * 64 + tid - 64];
   };
   auto stage_store = [&](int buf) {
     bf16* base = smem + buf * STAGE;
     sq.store(base, tid);
     sdo.store(base + TILE_ELEMS, tid);
     float* stats = reinterpret_cast<float*>(base + 2 * TILE_ELEMS);
-    if (tid < 128) stats[tid] = st_lse;
+    if (tid < 128) stats[tid] = st_stat;
   };
 
   stage_load(0);
@@ -400,7 +413,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   for (int it = 0; it < niter; ++it) {
     const int cur = it & 1;
     if (it + 1 < niter) stage_load(it + 1);
-    const int q0 = (qt_first + it % nqt) * 64;
+    const int q0 = (qt_first + it) * 64;
     const bf16* qtile = smem + cur * STAGE;
     const bf16* dotile = qtile + TILE_ELEMS;
     const float* stats = reinterpret_cast<const float*>(qtile + 2 * TILE_ELEMS);
@@ -451,30 +464,85 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     __syncthreads();
   }
 
-  bf16* dkp = dk + (int64_t)bi * dk_sb + (int64_t)kvh * dk_sh + (int64_t)krow * dk_ss;
-  bf16* dvp = dv + (int64_t)bi * dv_sb + (int64_t)kvh * dv_sh + (int64_t)krow * dv_ss;
+  if (PARTIAL) {
+    float* pk = part_k + (stat0 + krow) * HD;
+    float* pv = part_v + (stat0 + krow) * HD;
 #pragma unroll
-  for (int dt = 0; dt < HD / 32; ++dt)
+    for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      bf16x4 a, b;
+      for (int g = 0; g < 4; ++g) {
+        f32x4 a, b;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        a[e] = (bf16)(dkacc[dt][g * 4 + e] * scale);
-        b[e] = (bf16)dvacc[dt][g * 4 + e];
+        for (int e = 0; e < 4; ++e) {
+          a[e] = dkacc[dt][g * 4 + e] * scale;
+          b[e] = dvacc[dt][g * 4 + e];
+        }
+        *reinterpret_cast<f32x4*>(pk + dt * 32 + g * 8 + h * 4) = a;
+        *reinterpret_cast<f32x4*>(pv + dt * 32 + g * 8 + h * 4) = b;
       }
-      *reinterpret_cast<bf16x4*>(dkp + dt * 32 + g * 8 + h * 4) = a;
-      *reinterpret_cast<bf16x4*>(dvp + dt * 32 + g * 8 + h * 4) = b;
+  } else {
+    bf16* dkp = dk + dkl.at(bi, kvh) + (int64_t)krow * dkl.s_;
+    bf16* dvp = dv + dvl.at(bi, kvh) + (int64_t)krow * dvl.s_;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 a, b;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = (bf16)(dkacc[dt][g * 4 + e] * scale);
+          b[e] = (bf16)dvacc[dt][g * 4 + e];
+        }
+        *reinterpret_cast<bf16x4*>(dkp + dt * 32 + g * 8 + h * 4) = a;
+        *reinterpret_cast<bf16x4*>(dvp + dt * 32 + g * 8 + h * 4) = b;
+      }
+  }
+}
+
+// dk/dv[b, kvh, i, :] = sum over the group's query heads of the fp32 partials; one thread per
+// 8 channels (two 16-byte reads per partial, one 16-byte bf16 store).
+__global__ __launch_bounds__(256) void attn_group_reduce_kernel(
+    const float* __restrict__ part_k, const float* __restrict__ part_v, bf16* __restrict__ dk,
+    bf16* __restrict__ dv, int s, int nq, int nkv, int64_t total, KLayout dkl, KLayout dvl) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (bi, kvh, si, chunk of 8)
+  if (idx >= total) return;
+  const int c = (int)(idx & 15);
+  const int si = (int)((idx >> 4) % s);
+  const int kvh = (int)((idx >> 4) / s % nkv);
+  const int bi = (int)((idx >> 4) / ((int64_t)s * nkv));
+  const int per = nq / nkv;
+  float ak[8], av[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ak[e] = av[e] = 0.f;
+  for (int j = 0; j < per; ++j) {
+    const int64_t off = ((((int64_t)bi * nq + kvh * per + j) * s) + si) * HD + c * 8;
+    const f32x4 k0 = *reinterpret_cast<const f32x4*>(part_k + off);
+    const f32x4 k1 = *reinterpret_cast<const f32x4*>(part_k + off + 4);
+    const f32x4 v0 = *reinterpret_cast<const f32x4*>(part_v + off);
+    const f32x4 v1 = *reinterpret_cast<const f32x4*>(part_v + off + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ak[e] += k0[e];
+      ak[4 + e] += k1[e];
+      av[e] += v0[e];
+      av[4 + e] += v1[e];
     }
+  }
+  bf16x8 ok, ov;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    ok[e] = (bf16)ak[e];
+    ov[e] = (bf16)av[e];
+  }
+  stg8(dk + dkl.at(bi, kvh) + (int64_t)si * dkl.s_ + c * 8, ok);
+  stg8(dv + dvl.at(bi, kvh) + (int64_t)si * dvl.s_ + c * 8, ov);
 }
 
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, int64_t q_ss,
-    int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh, int64_t v_ss,
-    int64_t v_sb, int64_t v_sh, int64_t do_ss, int64_t do_sb, int64_t do_sh, int64_t dq_ss,
-    int64_t dq_sb, int64_t dq_sh) {
+    bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
+    KLayout kl, KLayout vl, QLayout dol, QLayout dql) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   constexpr int STAGE = 2 * TILE_ELEMS;  // K tile | V tile, both swizzled [64][128]
 
@@ -484,15 +552,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   const int qt = nqt - 1 - (lid % nqt);
   const int head = (lid / nqt) % nq;
   const int bi = lid / (nqt * nq);
-  const int kvh = head / (nq / nkv);
+  const int per = nq / nkv;
+  const int kvh = head / per;
   const int q0 = qt * BQ;
   const int qw0 = q0 + wave * 32;
   const int qrow = qw0 + (lane & 31);
 
-  const bf16* qp = q + (int64_t)bi * q_sb + (int64_t)head * q_sh + (int64_t)qrow * q_ss;
-  const bf16* dop = dout + (int64_t)bi * do_sb + (int64_t)head * do_sh + (int64_t)qrow * do_ss;
-  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
-  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
+  const bf16* qp = q + ql.at(bi, head, per) + (int64_t)qrow * ql.s_;
+  const bf16* dop = dout + dol.at(bi, head, per) + (int64_t)qrow * dol.s_;
+  const bf16* kb = k + kl.at(bi, kvh);
+  const bf16* vb = v + vl.at(bi, kvh);
   bf16x8 qf[HD / 16], dof[HD / 16];
 #pragma unroll
   for (int kk = 0; kk < HD / 16; ++kk) {
@@ -511,8 +580,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
 
   const int ntiles = (q0 + BQ) / BKV;
   TileStager sk, sv;
-  sk.load(kb, k_ss, 0, tid);
-  sv.load(vb, v_ss, 0, tid);
+  sk.load(kb, kl.s_, 0, tid);
+  sv.load(vb, vl.s_, 0, tid);
   sk.store(smem, tid);
   sv.store(smem + TILE_ELEMS, tid);
   __syncthreads();
@@ -520,8 +589,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   for (int j = 0; j < ntiles; ++j) {
     const int cur = j & 1;
     if (j + 1 < ntiles) {
-      sk.load(kb, k_ss, (j + 1) * BKV, tid);
-      sv.load(vb, v_ss, (j + 1) * BKV, tid);
+      sk.load(kb, kl.s_, (j + 1) * BKV, tid);
+      sv.load(vb, vl.s_, (j + 1) * BKV, tid);
     }
     const int key0 = j * BKV;
     if (key0 <= qw0 + 31) {
@@ -567,7 +636,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     __syncthreads();
   }
 
-  bf16* dqp = dq + (int64_t)bi * dq_sb + (int64_t)head * dq_sh + (int64_t)qrow * dq_ss;
+  bf16* dqp = dq + dql.at(bi, head, per) + (int64_t)qrow * dql.s_;
 #pragma unroll
   for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
@@ -579,61 +648,94 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     }
 }
 
+template __global__ void attn_bwd_dkdv_kernel<false>(const bf16*, const bf16*, const bf16*, const bf16*,
+                                                     const float*, const float*, bf16*, bf16*, float*,
+                                                     float*, int, int, int, float, float, QLayout,
+                                                     KLayout, KLayout, QLayout, KLayout, KLayout);
+template __global__ void attn_bwd_dkdv_kernel<true>(const bf16*, const bf16*, const bf16*, const bf16*,
+                                                    const float*, const float*, bf16*, bf16*, float*,
+                                                    float*, int, int, int, float, float, QLayout,
+                                                    KLayout, KLayout, QLayout, KLayout, KLayout);
+
 }  // namespace
 
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
   if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
-  return (size_t)b * nq * s * sizeof(float);
+  size_t bytes = (size_t)b * nq * s * sizeof(float);  // delta
+  if (nq != nkv) bytes += 2 * (size_t)b * nq * s * hd * sizeof(float);  // per-query-head dK, dV
+  return bytes;
 }
 
 extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                            const void* o, const float* lse, void* dq, void* dk, void* dv,
                            void* workspace, int s, int b, int nq, int nkv, int hd, float scale,
-                           int64_t q_ss, int64_t q_sb, int64_t q_sh, int64_t k_ss, int64_t k_sb,
-                           int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss,
-                           int64_t o_sb, int64_t o_sh, int64_t do_ss, int64_t do_sb, int64_t do_sh,
-                           int64_t dq_ss, int64_t dq_sb, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb,
-                           int64_t dk_sh, int64_t dv_ss, int64_t dv_sb, int64_t dv_sh,
-                           void* stream) {
+                           int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss,
+                           int64_t k_sb, int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh,
+                           int64_t o_ss, int64_t o_sb, int64_t o_sg, int64_t o_sh, int64_t do_ss,
+                           int64_t do_sb, int64_t do_sg, int64_t do_sh, int64_t dq_ss, int64_t dq_sb,
+                           int64_t dq_sg, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh,
+                           int64_t dv_ss, int64_t dv_sb, int64_t dv_sh, void* stream) {
   if (!dout || !q || !k || !v || !o || !lse || !dq || !dk || !dv || !workspace) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
   const void* ptrs[] = {dout, q, k, v, o, dq, dk, dv, workspace};
   for (const void* p : ptrs)
     if (!kr_aligned16(p)) return KR_EINVAL;
-  if ((q_ss | q_sb | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sh | do_ss |
-       do_sb | do_sh | dq_ss | dq_sb | dq_sh | dk_ss | dk_sb | dk_sh | dv_ss | dv_sb | dv_sh) % 8)
+  if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
+       o_sh | do_ss | do_sb | do_sg | do_sh | dq_ss | dq_sb | dq_sg | dq_sh | dk_ss | dk_sb |
+       dk_sh | dv_ss | dv_sb | dv_sh) % 8)
     return KR_EINVAL;
   hipStream_t st = (hipStream_t)stream;
+  const QLayout ql{q_ss, q_sb, q_sg, q_sh}, ol{o_ss, o_sb, o_sg, o_sh}, dol{do_ss, do_sb, do_sg, do_sh},
+      dql{dq_ss, dq_sb, dq_sg, dq_sh};
+  const KLayout kl{k_ss, k_sb, k_sh}, vl{v_ss, v_sb, v_sh}, dkl{dk_ss, dk_sb, dk_sh},
+      dvl{dv_ss, dv_sb, dv_sh};
   float* delta = (float*)workspace;
+  const int64_t rows = (int64_t)b * nq * s;
+  float* part_k = delta + rows;
+  float* part_v = part_k + rows * hd;
+  const bool partial = nq != nkv;
   constexpr size_t lds_dkdv = 2 * (2 * TILE_ELEMS + 256) * sizeof(bf16);
   constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
-  static std::once_flag once;
-  static hipError_t attr_status = hipSuccess;
-  std::call_once(once, [&] {
-    attr_status = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
-    if (attr_status == hipSuccess)
-      attr_status = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel,
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
-  });
+  static const hipError_t attr_status = [] {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+    return e;
+  }();
   if (attr_status != hipSuccess) return KR_ELAUNCH;
 
-  const int64_t rows = (int64_t)b * nq * s;
+  const int per = nq / nkv;
   hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
-                     (const bf16*)dout, (const bf16*)o, delta, s, nq, rows, do_ss, do_sb, do_sh,
-                     o_ss, o_sb, o_sh);
+                     (const bf16*)dout, (const bf16*)o, delta, s, nq, per, rows, dol, ol);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
-  hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3((s / 128) * nkv * b), dim3(256), lds_dkdv, st,
-                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
-                     (const float*)delta, (bf16*)dk, (bf16*)dv, s, nq, nkv, scale, scale_log2, q_ss,
-                     q_sb, q_sh, k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, do_ss, do_sb, do_sh, dk_ss,
-                     dk_sb, dk_sh, dv_ss, dv_sb, dv_sh);
+  const dim3 grid_kv((s / 128) * nq * b);
+  if (partial) {
+    hipLaunchKernelGGL(attn_bwd_dkdv_kernel<true>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
+                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, scale, scale_log2, ql, kl,
+                       vl, dol, dkl, dvl);
+    if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+    const int64_t total = (int64_t)b * nkv * s * 16;
+    hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
+                       nkv, total, dkl, dvl);
+  } else {
+    hipLaunchKernelGGL(attn_bwd_dkdv_kernel<false>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
+                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, scale, scale_log2, ql, kl,
+                       vl, dol, dkl, dvl);
+  }
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3((s / BQ) * nq * b), dim3(256), lds_dq, st,
                      (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
-                     (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, q_ss, q_sb, q_sh,
-                     k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, do_ss, do_sb, do_sh, dq_ss, dq_sb, dq_sh);
+                     (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
+                     dql);
   return kr_launch_status();
 }

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16* __rest
 __global__ __launch_bounds__(kThreads) void rope_kernel(
     const bf16* t, bf16* out, const float* __restrict__ freqs, int b,
     int heads, int hd, int64_t ts, int64_t tb, int64_t th, int64_t os, int64_t ob, int64_t oh,
-    float sin_sign) {
+    float sin_sign, int group_size, int group_rotate) {
   __shared__ float cs[128], sn[128];
   const int pos = blockIdx.x;
   const int half = hd / 2;
@@ -99,6 +99,13 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(
     const bf16* src = t + pos * ts + bi * tb + h * th;
     bf16* dst = out + pos * os + bi * ob + h * oh;
     bf16x8 lo = ldg8(src + c), hi = ldg8(src + half + c), olo, ohi;
+    if (h % group_size >= group_rotate) {  // a head that is carried along unrotated
+      if (dst != src) {
+        stg8(dst + c, lo);
+        stg8(dst + half + c, hi);
+      }
+      continue;
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float a = (float)lo[e], bb = (float)hi[e];
@@ -151,13 +158,15 @@ extern "C" int kr_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t ro
 
 extern "C" int kr_rope(const void* t, void* out, const float* freqs, int s, int b, int heads,
                        int hd, int64_t ts, int64_t tb, int64_t th, int64_t os, int64_t ob,
-                       int64_t oh, int backward, void* stream) {
+                       int64_t oh, int backward, int group_size, int group_rotate, void* stream) {
   if (!t || !out || !freqs || s <= 0 || b <= 0 || heads <= 0 || hd <= 0) return KR_EINVAL;
+  if (group_size <= 0 || group_rotate <= 0 || group_rotate > group_size || heads % group_size)
+    return KR_EINVAL;
   if (hd % 16 || hd > 256) return KR_EUNSUPPORTED;
   if (!kr_aligned16(t) || !kr_aligned16(out)) return KR_EINVAL;
   if ((ts | tb | th | os | ob | oh) % 8) return KR_EINVAL;
   hipLaunchKernelGGL(rope_kernel, dim3(s), dim3(kThreads), 0, (hipStream_t)stream,
                      (const bf16*)t, (bf16*)out, freqs, b, heads, hd, ts, tb, th, os, ob, oh,
-                     backward ? -1.0f : 1.0f);
+                     backward ? -1.0f : 1.0f, group_size, group_rotate);
   return kr_launch_status();
 }

@@ -13,7 +13,7 @@ namespace {
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * KR_WAVE;
-constexpr int kMaxBwdBlocks = 1024;
+constexpr int kMaxBwdBlocks = 512;
 
 template <int NCHUNK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __restrict__ x,
@@ -143,15 +143,21 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
   }
 }
 
-// dgamma[col] = sum over partial rows; one thread per column, coalesced across columns.
+// dgamma[col] = sum over partial rows.  A block owns 64 columns; its 4 waves each sum every
+// fourth partial row (256-byte coalesced reads) and combine through LDS.
 __global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* __restrict__ partial,
                                                              bf16* __restrict__ dgamma,
                                                              int nparts, int cols) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col >= cols) return;
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + lane;
   float acc = 0.f;
-  for (int p = 0; p < nparts; ++p) acc += partial[(int64_t)p * cols + col];
-  dgamma[col] = (bf16)acc;
+  if (col < cols)
+    for (int p = wave; p < nparts; p += 4) acc += partial[(int64_t)p * cols + col];
+  red[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && col < cols)
+    dgamma[col] = (bf16)(red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane]);
 }
 
 inline int bwd_blocks(int rows) {
@@ -209,7 +215,7 @@ extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, 
                                            rstd, (const bf16*)gamma, (bf16*)dx, (float*)workspace,
                                            rows, cols));
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
-  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 255) / 256), dim3(256), 0,
+  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 63) / 64), dim3(256), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
   return kr_launch_status();
 }

@@ -1,6 +1,7 @@
 """Causal grouped-query attention operator.
 
-Inputs ``main`` (query ``[s, b, nq, hd]``), ``key`` and ``value`` (``[s, b, nkv, hd]``);
+Inputs ``main`` (query ``[s, b, nq, hd]``, or the grouped view ``[s, b, nkv, nq/nkv, hd]``
+the QKV-split operator produces), ``key`` and ``value`` (``[s, b, nkv, hd]``);
 output ``[s, b, nq*hd]``.  Softmax scale ``1/sqrt(hd)``; query head ``i`` attends KV head
 ``i // (nq/nkv)``; causal mask aligned top-left (``sq == sk``); saves q, k, v, the
 output and the fp32 log-sum-exp ``[b, nq, s]``
@@ -46,12 +47,13 @@ class TEDotProductAttentionOp(BasicOperation, PartitionableOperator):
                       basic_op_next_ops, basic_op_kwargs):
         key, value = basic_op_extra_inputs[0]
         q = input_
-        if q.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+        if q.dim() not in (4, 5) or key.dim() != 4 or value.dim() != 4:
             raise ValueError("attention expects [s, b, heads, head_dim] tensors")
-        s, b, nq, hd = q.shape
+        s, b, hd = q.shape[0], q.shape[1], q.shape[-1]
+        nq = q.shape[2] * q.shape[3] if q.dim() == 5 else q.shape[2]
         if key.shape != value.shape or key.shape[0] != s or key.shape[1] != b or key.shape[3] != hd:
             raise ValueError(f"q {tuple(q.shape)}, k {tuple(key.shape)}, v {tuple(value.shape)} do not match")
-        if nq % key.shape[2]:
+        if nq % key.shape[2] or (q.dim() == 5 and q.shape[2] != key.shape[2]):
             raise ValueError("query heads must be a multiple of KV heads")
         scale = self.softmax_scale if self.softmax_scale is not None else 1.0 / math.sqrt(hd)
         ctx = basic_op_ctxs[0]

@@ -6,6 +6,11 @@ gets no gradient (kareus/megatron/core/extensions/ops/rotary_embedding.py:50-171
 math kareus/megatron/core/models/common/embedding/rope_utils.py:147-222; the fused
 path evaluates the trigonometry in fp32 from the fp32 table,
 kareus/apex/transformer/functional/fused_rope.py:27-46).
+
+When query and key arrive as views of one fused QKV buffer (as the QKV-split operator
+hands them over) and the backend offers it, both are rotated in place with a single
+launch; the fused buffer has no other reader, so nothing observes the overwrite.  The
+same holds for the gradient views coming out of the attention backward.
 """
 
 from __future__ import annotations
@@ -43,6 +48,11 @@ class RotaryEmbeddingOp(BasicOperation, PartitionableOperator):
     def get_output_channels(self) -> List[Channel]:
         return [Channel(0, "main"), Channel(1, "key")]
 
+    @staticmethod
+    def _shared_fused(a, b):
+        fa, fb = getattr(a, "_kr_fused5", None), getattr(b, "_kr_fused5", None)
+        return fa if (fa is not None and fa is fb) else None
+
     def fuser_forward(self, basic_op_ctxs, input_, *, basic_op_extra_inputs, basic_op_prev_ops,
                       basic_op_next_ops, basic_op_kwargs):
         key, freqs = basic_op_extra_inputs[0]
@@ -52,8 +62,13 @@ class RotaryEmbeddingOp(BasicOperation, PartitionableOperator):
             raise ValueError(f"rotary table covers {freqs.shape[0]} positions, sequence has {input_.shape[0]}")
         ctx = basic_op_ctxs[0]
         be = get_backend(self._backend_name)
-        q_out = be.rope_fwd(input_, freqs)
-        k_out = be.rope_fwd(key, freqs)
+        fused = self._shared_fused(input_, key)
+        if fused is not None and hasattr(be, "rope_fused_inplace"):
+            be.rope_fused_inplace(fused, fused.shape[3] - 2, freqs, False)
+            q_out, k_out = input_, key
+        else:
+            q_out = be.rope_fwd(input_, freqs)
+            k_out = be.rope_fwd(key, freqs)
         if ctx.requires_grad:
             ctx.save_for_backward(freqs)
         return q_out, [(k_out,)]
@@ -62,6 +77,11 @@ class RotaryEmbeddingOp(BasicOperation, PartitionableOperator):
         (freqs,) = basic_op_ctxs[0].saved_tensors
         (grad_key,) = basic_op_grad_extra_outputs[0]
         be = get_backend(self._backend_name)
-        dq = be.rope_bwd(grad_output, freqs)
-        dk = be.rope_bwd(grad_key, freqs)
+        fused = self._shared_fused(grad_output, grad_key)
+        if fused is not None and hasattr(be, "rope_fused_inplace"):
+            be.rope_fused_inplace(fused, fused.shape[3] - 2, freqs, True)
+            dq, dk = grad_output, grad_key
+        else:
+            dq = be.rope_bwd(grad_output, freqs)
+            dk = be.rope_bwd(grad_key, freqs)
         return dq, [()], [(dk, None)]
