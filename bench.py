@@ -183,6 +183,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--nanobatches", type=int, default=0, help="override the workload's nanobatch count")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip serial/partition/energy legs")
     args = ap.parse_args()
@@ -192,7 +193,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a HIP device")
 
-    w = WORKLOADS[args.workload]
+    w = dict(WORKLOADS[args.workload])
+    if args.nanobatches:
+        w["nnb"] = args.nanobatches
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     gen = torch.Generator().manual_seed(42)

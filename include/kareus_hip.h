@@ -40,13 +40,18 @@ const char* kr_error_string(int code);
  *   KR_GEMM_NN  :847-859  dx = dy . W      A = dy [M,K] row-major, B = W  [K,N] row-major
  *   KR_GEMM_NT  :898-909  dW = dy^T . x    A = dy [K,M] row-major, B = x  [K,N] row-major
  * C is [M,N] row-major.  M, N, K, lda, ldb, ldc must be multiples of 8.
- * accumulate != 0 adds the product to the existing contents of C (rounded once).          */
+ * accumulate != 0 adds the product to the existing contents of C (rounded once).
+ * workspace may be NULL.  If it holds at least kr_gemm_workspace_bytes() bytes, shapes whose
+ * output has too few tiles to occupy the GPU (weight gradients) are computed split-K through
+ * fp32 partial tiles kept there; otherwise one workgroup walks the whole contraction.       */
 #define KR_GEMM_TN 0
 #define KR_GEMM_NN 1
 #define KR_GEMM_NT 2
+size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K);
 int kr_gemm_bf16(int layout, int M, int N, int K,
                  const void* A, int64_t lda, const void* B, int64_t ldb,
-                 void* C, int64_t ldc, int accumulate, void* stream);
+                 void* C, int64_t ldc, int accumulate,
+                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- RMSNorm ---------------------------------------------------------------------------
  * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd

@@ -23,8 +23,9 @@ _c_void_p, _c_int, _c_i64, _c_float, _c_size_t = (
 _SIGNATURES = {
     "kr_version": (_c_int, []),
     "kr_error_string": (ctypes.c_char_p, [_c_int]),
+    "kr_gemm_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int, _c_int]),
     "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
-                              _c_void_p, _c_i64, _c_int, _c_void_p]),
+                              _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p]),
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_void_p]),
@@ -98,8 +99,11 @@ class HipBackend:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
             out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+        ws_bytes = self.lib.kr_gemm_workspace_bytes(layout, m, n, k)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
-                                   out.data_ptr(), out.stride(0), int(accumulate), self._stream())
+                                   out.data_ptr(), out.stride(0), int(accumulate),
+                                   ws.data_ptr() if ws is not None else None, ws_bytes, self._stream())
         self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k})")
         return out
 

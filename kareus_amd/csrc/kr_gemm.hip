@@ -33,6 +33,10 @@
 //     tile has landed.
 //   * Workgroup ids are remapped so that the tiles resident on one XCD (ids congruent mod 8)
 //     form a compact band of C and share A/B panels in that XCD's L2.
+//   * Split-K: when C has too few tiles to fill 256 CUs (weight gradients: a small N x K
+//     output contracted over all tokens), the contraction is cut into up to 16 ranges, each
+//     workgroup writes an fp32 partial tile into a caller-provided workspace, and a small
+//     HBM-bound kernel sums the partials and rounds to bf16.
 #include "kr_common.h"
 
 namespace {
@@ -175,8 +179,18 @@ template <bool A_T, bool B_T>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int64_t lda,
                                                         const bf16* __restrict__ B, int64_t ldb,
                                                         bf16* __restrict__ C, int64_t ldc, int M,
-                                                        int N, int K, int accumulate) {
+                                                        int N, int K, int accumulate, int k_per,
+                                                        float* __restrict__ partial) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  // split-K: blockIdx.y owns contraction range [y*k_per, y*k_per + K) and writes an fp32
+  // partial tile instead of C (k_per is a multiple of 64)
+  if (partial != nullptr) {
+    const int k0 = blockIdx.y * k_per;
+    A += A_T ? (int64_t)k0 * lda : k0;
+    B += B_T ? (int64_t)k0 * ldb : k0;
+    K = (K - k0) < k_per ? (K - k0) : k_per;
+    partial += (int64_t)blockIdx.y * M * N;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -289,6 +303,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       for (int g = 0; g < 4; ++g) {
         const int n = n0 + (wn * TN + j) * 32 + 8 * g + 4 * h;
         if (n >= N) continue;
+        if (partial != nullptr) {
+          f32x4 pv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
+          *reinterpret_cast<f32x4*>(partial + (int64_t)m * N + n) = pv;
+          continue;
+        }
         bf16* dst = C + (int64_t)m * ldc + n;
         bf16x4 o;
         if (accumulate) {
@@ -307,15 +328,61 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 
 // the three layouts the library serves
 template __global__ void gemm_kernel<false, false>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                   int64_t, int, int, int, int);
+                                                   int64_t, int, int, int, int, int, float*);
 template __global__ void gemm_kernel<false, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                  int64_t, int, int, int, int);
+                                                  int64_t, int, int, int, int, int, float*);
 template __global__ void gemm_kernel<true, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                 int64_t, int, int, int, int);
+                                                 int64_t, int, int, int, int, int, float*);
+
+// C = bf16(sum over splits of the fp32 partial tiles [+ C]); one thread per 8 columns.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
+                                                            bf16* __restrict__ C, int64_t ldc, int M,
+                                                            int N, int splits, int accumulate) {
+  const int nv = N / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * nv) return;
+  const int m = (int)(idx / nv), n = (int)(idx % nv) * 8;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    const float* src = partial + ((int64_t)sp * M + m) * N + n;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(src);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[e] += a[e];
+      acc[4 + e] += b[e];
+    }
+  }
+  bf16* dst = C + (int64_t)m * ldc + n;
+  if (accumulate) {
+    const bf16x8 old = ldg8(dst);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += (float)old[e];
+  }
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (bf16)acc[e];
+  stg8(dst, o);
+}
+
+// How many ways to cut the contraction so that enough workgroups exist to fill 256 CUs.
+// 1 = no split.  Every split keeps at least 8 K-steps of 64.
+inline int choose_splits(int M, int N, int K) {
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (tiles >= 192) return 1;
+  int splits = (512 + tiles - 1) / tiles;
+  const int max_by_k = K / (8 * BK);
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > 16) splits = 16;
+  return splits < 2 ? 1 : splits;
+}
 
 template <bool A_T, bool B_T>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
-           int N, int K, int accumulate, hipStream_t stream) {
+           int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
+           hipStream_t stream) {
   constexpr size_t lds_bytes = 2 * STAGE * sizeof(bf16);
   // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
   static const hipError_t attr_status =
@@ -323,18 +390,40 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles), dim3(NTHREADS), lds_bytes, stream, A, lda,
-                     B, ldb, C, ldc, M, N, K, accumulate);
+  int splits = choose_splits(M, N, K);
+  if (workspace == nullptr || (size_t)splits * M * N * sizeof(float) > workspace_bytes) splits = 1;
+  if (splits == 1) {
+    hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles), dim3(NTHREADS), lds_bytes, stream, A, lda,
+                       B, ldb, C, ldc, M, N, K, accumulate, 0, (float*)nullptr);
+    return kr_launch_status();
+  }
+  int k_per = (K + splits - 1) / splits;
+  k_per = (k_per + BK - 1) / BK * BK;
+  splits = (K + k_per - 1) / k_per;
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles, splits), dim3(NTHREADS), lds_bytes, stream,
+                     A, lda, B, ldb, C, ldc, M, N, K, 0, k_per, workspace);
+  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+  const int64_t work = (int64_t)M * (N / 8);
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream,
+                     (const float*)workspace, C, ldc, M, N, splits, accumulate);
   return kr_launch_status();
 }
 
 }  // namespace
 
+extern "C" size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K) {
+  (void)layout;
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const int splits = choose_splits(M, N, K);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
 extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int64_t lda,
                             const void* B, int64_t ldb, void* C, int64_t ldc, int accumulate,
-                            void* stream) {
+                            void* workspace, size_t workspace_bytes, void* stream) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return KR_EINVAL;
   if (!kr_aligned16(A) || !kr_aligned16(B) || !kr_aligned16(C)) return KR_EINVAL;
+  if (workspace && !kr_aligned16(workspace)) return KR_EINVAL;
   if ((M | N | K) % 8 || (lda | ldb | ldc) % 8) return KR_EUNSUPPORTED;
   // chunk offsets inside an operand are kept in 32 bits
   const int64_t a_rows = layout == KR_GEMM_NT ? 64 : M, b_rows = layout == KR_GEMM_TN ? N : 64;
@@ -342,17 +431,18 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   const bf16* a = (const bf16*)A;
   const bf16* b = (const bf16*)B;
   bf16* c = (bf16*)C;
+  float* ws = (float*)workspace;
   hipStream_t st = (hipStream_t)stream;
   switch (layout) {
     case KR_GEMM_TN:  // A [M,K], B [N,K]
       if (lda < K || ldb < K || ldc < N) return KR_EINVAL;
-      return launch<false, false>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<false, false>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
     case KR_GEMM_NN:  // A [M,K], B [K,N]
       if (lda < K || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<false, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<false, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
     case KR_GEMM_NT:  // A [K,M], B [K,N]
       if (lda < M || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<true, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, st);
+      return launch<true, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
     default:
       return KR_EINVAL;
   }
