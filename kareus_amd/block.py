@@ -32,6 +32,7 @@ from .operators import (
     TERowParallelLinearOp,
     rotary_frequencies,
 )
+from .partitions.streams import stream_api
 from .partitions import (
     CommunicationType,
     ComputeOp,
@@ -198,11 +199,12 @@ class LayerStack(torch.nn.Module):
 
     def _streams(self):
         c = self.config
-        if not c.use_streams or c.num_nanobatches < 2 or not torch.cuda.is_available():
+        api = stream_api()
+        if not c.use_streams or c.num_nanobatches < 2 or not api.available():
             c.nanobatch_streams = None
             return None
         if c.nanobatch_streams is None:
-            c.nanobatch_streams = [torch.cuda.Stream() for _ in range(c.num_nanobatches)]
+            c.nanobatch_streams = [api.new_stream() for _ in range(c.num_nanobatches)]
         return c.nanobatch_streams
 
     def _get_all_params(self) -> List[torch.nn.Parameter]:

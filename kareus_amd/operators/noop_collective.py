@@ -33,6 +33,8 @@ from typing import Optional
 
 import torch
 
+from ..partitions.streams import stream_api
+
 
 class NoOpAllReduce(torch.nn.Module):
     def __init__(self, batch_idx: int = 0, world_size: int = 1, comm_stream=None) -> None:
@@ -49,14 +51,14 @@ class NoOpAllReduce(torch.nn.Module):
         self.last_resource_shape = (None, None)
         self.calls = 0
         if comm_stream is not None:
-            self.wait_event = torch.cuda.Event()
-            self.done_event = torch.cuda.Event()
+            self.wait_event = stream_api().new_event()
+            self.done_event = stream_api().new_event()
 
     def set_stream(self, stream) -> None:
         self.comm_stream = stream
         if stream is not None and self.wait_event is None:
-            self.wait_event = torch.cuda.Event()
-            self.done_event = torch.cuda.Event()
+            self.wait_event = stream_api().new_event()
+            self.done_event = stream_api().new_event()
 
     def event_record(self, stream) -> None:
         if self.comm_stream is not None and stream is not None:

@@ -26,6 +26,7 @@ import torch
 from torch import Tensor
 
 from .context_manager import NanoBatchContext, TensorStore
+from .streams import stream_api
 from .tensor_graph import TensorGraph
 
 # Non-tensor arguments that follow the nanobatch inputs, rotary table and mask.
@@ -66,7 +67,7 @@ def _nanobatch_streams(config, n: int) -> List[Optional[object]]:
 def _fork(streams: Sequence[Optional[object]]) -> None:
     """Side streams start after everything already enqueued on the caller's stream."""
     if any(s is not None for s in streams):
-        here = torch.cuda.current_stream()
+        here = stream_api().current_stream()
         for s in streams:
             if s is not None and s != here:
                 s.wait_stream(here)
@@ -75,7 +76,7 @@ def _fork(streams: Sequence[Optional[object]]) -> None:
 def _join(streams: Sequence[Optional[object]]) -> None:
     """The caller's stream continues after everything enqueued on the side streams."""
     if any(s is not None for s in streams):
-        here = torch.cuda.current_stream()
+        here = stream_api().current_stream()
         for s in streams:
             if s is not None and s != here:
                 here.wait_stream(s)

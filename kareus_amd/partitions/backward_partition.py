@@ -62,6 +62,7 @@ class BackwardPartition(PartitionBase):
                     )
                 op_ctx.saved_tensors = None
 
+            self._op_done(idx)
             if idx == start - 1:
                 self.comm_op.event_record(_current_stream())
 

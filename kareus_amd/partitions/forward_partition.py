@@ -51,6 +51,7 @@ class ForwardPartition(PartitionBase):
                 basic_op_kwargs=[{}],
             )
 
+            self._op_done(idx)
             if idx == start - 1:
                 self.comm_op.event_record(_current_stream())
 

@@ -24,6 +24,7 @@ from typing import Any, Dict, List, Optional, Tuple, Union
 import torch
 
 from .context_manager import NanoBatchContext
+from .streams import stream_api
 from .tensor_graph import CommunicationOp, ComputeOp
 
 OverlapWindow = Tuple[Union[int, str], Union[int, str]]
@@ -82,7 +83,7 @@ def _resolve_slot(slots: Dict[str, int], name: str) -> int:
 
 def _current_stream():
     """The HIP stream kernels are being enqueued on (None on a host-only run)."""
-    return torch.cuda.current_stream() if torch.cuda.is_available() else None
+    return stream_api().current_stream()
 
 
 class _TimerScope:
@@ -208,13 +209,16 @@ class PartitionBase:
             return contextlib.nullcontext()
         return _TimerScope(t, self)
 
+    def _op_done(self, idx: int) -> None:
+        t = PartitionBase.timer
+        if t is not None and hasattr(t, "op_done"):
+            t.op_done(self, idx)
+
     # -- stream scoping -----------------------------------------------------------
     @staticmethod
     def _on_stream(ctx: NanoBatchContext):
         """Context manager making the nanobatch's own stream current (if it has one)."""
-        if ctx.stream is None:
-            return contextlib.nullcontext()
-        return torch.cuda.stream(ctx.stream)
+        return stream_api().stream(ctx.stream)
 
     def execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext):
         raise NotImplementedError

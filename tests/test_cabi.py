@@ -1,0 +1,47 @@
+"""The C-ABI library loads on a machine without a GPU and exports exactly what include/*.h declares."""
+
+import ctypes
+import glob
+import os
+import re
+
+from kareus_amd.backend import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    names = set()
+    for header in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+        names.update(re.findall(r"\b(kr_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    declared = _declared()
+    assert {"kr_gemm_bf16", "kr_attn_fwd", "kr_attn_bwd", "kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rope",
+            "kr_swiglu_fwd", "kr_swiglu_bwd", "kr_add", "kr_version", "kr_error_string"} <= declared
+    lib = ctypes.CDLL(hip.library_path())
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
+    # and the Python binding table covers the same set
+    assert set(hip._SIGNATURES) == declared
+
+
+def test_argument_checks_run_without_a_device():
+    lib = hip.load_library()
+    assert lib.kr_version() >= 100
+    assert lib.kr_error_string(0) == b"ok" and b"unknown" in lib.kr_error_string(-99)
+    # invalid arguments are rejected before anything touches the GPU
+    assert lib.kr_add(None, None, None, 8, None) == -1
+    assert lib.kr_swiglu_fwd(16, 16, 4, 12, None) == -2          # F not a multiple of 8
+    assert lib.kr_rmsnorm_fwd(16, 16, 16, 16, 4, 8200, 1e-5, None) == -2
+    assert lib.kr_gemm_bf16(0, 8, 8, 7, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -2
+    assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1
+    assert lib.kr_gemm_bf16(0, 8, 8, 8, 16, 8, 16, 8, 18, 8, 0, None, 0, None) == -1   # misaligned C
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 64) == 0  # head_dim 64 unsupported
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 4, 128) == 256 * 4 * 4
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 128) == 256 * 4 * 4 + 2 * 256 * 4 * 128 * 4
+    assert lib.kr_gemm_workspace_bytes(2, 1536, 4096, 16384) > 0 and lib.kr_gemm_workspace_bytes(0, 4096, 7168, 4096) == 0
+    assert lib.kr_rmsnorm_bwd_workspace_bytes(8192, 4096) == 512 * 4096 * 4

@@ -1,0 +1,235 @@
+"""The partition engine end to end on the host: BASELINE config 1 (fp32 plumbing layer) through
+graph -> partitions -> contexts -> single autograd node, with the eager backend, against the CPU
+oracle; nanobatch counts 1, 2 and 4, with and without activation recompute, with and without a
+schedule; host-forceable error paths; and the stream/event ordering rules replayed without a GPU."""
+
+import os
+
+import pytest
+import torch
+
+from kareus_amd import LayerConfig, LayerStack
+from kareus_amd.operators import NoOpAllReduce, QKVPostProcessOp
+from kareus_amd.partitions import NanoBatchContext, TensorStore, TransformerBlockAutogradFunction
+from kareus_amd.partitions.autograd_function import _flatten_grad_params
+from kareus_amd.partitions.partition_base import PartitionBase
+from kareus_amd.partitions.streams import use_stream_api
+from kareus_amd.schedule_check import RecordingStreams
+from kareus_amd.scheduler import CommConfig, PipelineCommScheduler, ScheduleItem
+from oracle import llama_layer_ref as R
+
+C1 = dict(hidden_size=512, num_attention_heads=8, num_query_groups=8, kv_channels=64, ffn_hidden_size=1376)
+PARAMS = [("input_layernorm", "ln1"), ("linear_qkv", "w_qkv"), ("linear_proj", "w_proj"),
+          ("pre_mlp_layernorm", "ln2"), ("linear_fc1", "w_fc1"), ("linear_fc2", "w_fc2")]
+
+
+def _oracle(layers, s, b, seed=42, dims=None):
+    dims = dims or R.LayerDims(512, 8, 8, 64, 1376)
+    gen = torch.Generator().manual_seed(1234)
+    params = [R.init_layer_params(dims, gen) for _ in range(layers)]
+    gd = torch.Generator().manual_seed(seed)
+    x, go = torch.randn(s, b, dims.hidden, generator=gd), torch.randn(s, b, dims.hidden, generator=gd)
+    return x, go, R.stack_forward_backward(x, params, dims, go)
+
+
+def _run(model, x, go):
+    xx = x.clone().requires_grad_(True)
+    y = model(xx)
+    y.backward(go)
+    return y.detach(), xx.grad
+
+
+def _check(model, x, go, ref, tol=2e-4):
+    y, dx = _run(model, x, go)
+    ry, rdx, rgrads = ref
+    assert (y - ry).abs().max() <= tol * ry.abs().max()
+    assert (dx - rdx).abs().max() <= tol * rdx.abs().max()
+    for li, layer in enumerate(model.layers):
+        for attr, name in PARAMS:
+            g, rg = getattr(layer, attr).weight.grad, rgrads[li][name]
+            assert (g - rg).abs().max() <= tol * rg.abs().max(), (li, name)
+
+
+@pytest.mark.parametrize("nnb", [1, 2, 4])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_config1_matches_oracle(nnb, recompute):
+    # BASELINE config 1 is b=2, s=256, 2 nanobatches; b=4 here so that 4 nanobatches divide it
+    x, go, ref = _oracle(layers=1, s=256, b=4)
+    cfg = LayerConfig(**C1, num_layers=1, num_nanobatches=nnb, params_dtype=torch.float32,
+                      backend="eager", checkpoint_activations=recompute)
+    _check(LayerStack(cfg, seed=1234), x, go, ref)
+
+
+def test_config1_exact_shape_two_layers():
+    x, go, ref = _oracle(layers=2, s=256, b=2)
+    cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
+    _check(LayerStack(cfg, seed=1234), x, go, ref)
+
+
+def test_gqa_layer_and_dense_query_view():
+    dims = R.LayerDims(hidden=64, nq=6, nkv=2, hd=16, ffn=40)
+    x, go, ref = _oracle(layers=1, s=24, b=2, dims=dims)
+    cfg = LayerConfig(hidden_size=64, num_attention_heads=6, num_query_groups=2, kv_channels=16, ffn_hidden_size=40,
+                      num_layers=1, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
+    m = LayerStack(cfg, seed=1234)
+    _check(m, x, go, ref)
+    # the reference's dense [s, b, nq, hd] query layout gives the same numbers
+    m.layers[0].qkv_postprocess.grouped_query_view = False
+    for p in m.parameters():
+        p.grad = None
+    _check(m, x, go, ref)
+    op = QKVPostProcessOp(2, 6, 16)
+    mixed = torch.arange(2 * 3 * 160, dtype=torch.float32).reshape(2, 3, 160)
+    q, k, v = op.split(mixed)
+    rq, rk, rv = R.split_qkv(mixed, 6, 2, 16)
+    assert torch.equal(q.flatten(2, 3), rq) and torch.equal(k, rk) and torch.equal(v, rv)
+    assert q.data_ptr() == mixed.data_ptr()  # a view, not a copy
+    assert torch.equal(op.merge(q.flatten(2, 3), k, v), mixed)  # merge inverts split
+
+
+def test_schedule_driven_run_matches_and_records_shapes(fixtures_dir):
+    x, go, ref = _oracle(layers=1, s=64, b=2)
+    cfg = LayerConfig(**C1, num_layers=1, num_nanobatches=2, params_dtype=torch.float32,
+                      backend="eager", checkpoint_activations=True)
+    m = LayerStack(cfg, seed=1234)
+    sch = PipelineCommScheduler(os.path.join(fixtures_dir, "scheds_pipeline_00324.py"), pp_rank=1,
+                                num_microbatches=8, use_activation_checkpointing=True)
+    cfg.kareus_scheduler = sch
+    xx = x.clone().requires_grad_(True)
+    sch.on_step_begin()
+    sch.on_instruction_begin("forward")
+    y = m(xx)
+    assert m.allreduce_comm_ops[1].last_resource_shape == (18, 1024)  # NB1's last carrier: fwd_mlp of item 0
+    assert m.allreduce_comm_ops[0].last_resource_shape == (20, 1024)  # fwd_trail default
+    sch.on_instruction_begin("backward")
+    y.backward(go)  # recompute pass reads rec_attn/rec_mlp, backward reads bwd_attn/bwd_mlp
+    assert m.allreduce_comm_ops[1].last_resource_shape == (21, 1024)  # bwd_attn 'rope_0-none-21-1024'
+    ry, rdx, _ = ref
+    assert (y.detach() - ry).abs().max() <= 2e-4 * ry.abs().max()
+    assert (xx.grad - rdx).abs().max() <= 2e-4 * rdx.abs().max()
+    assert m.allreduce_comm_ops[0].calls > 0 and m.allreduce_comm_ops[1].calls > 0
+
+
+def test_host_error_paths():
+    cfg = LayerConfig(**C1, num_layers=1, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
+    m = LayerStack(cfg, seed=0)
+    with pytest.raises(ValueError, match="multiple of 2 nanobatches"):
+        m(torch.randn(8, 1, 512))
+    with pytest.raises(ValueError, match="multiple of 2 nanobatches"):
+        m(torch.randn(8, 3, 512))
+    with pytest.raises(ValueError, match=r"\[s, b, 512\]"):
+        m(torch.randn(8, 2, 256))
+    with pytest.raises(NotImplementedError):
+        m(torch.randn(8, 2, 512), attention_mask=torch.ones(1))
+    with pytest.raises(NotImplementedError):
+        m(torch.randn(8, 2, 512), packed_seq_params=object())
+    with pytest.raises(ValueError, match="rotary table covers"):
+        m(torch.randn(8, 2, 512), rotary_pos_emb=m.rotary_pos_emb(4))
+    with pytest.raises(RuntimeError, match="executed by the partition engine"):
+        m.layers[0](torch.randn(1))
+    with pytest.raises(NotImplementedError):
+        LayerStack(LayerConfig(**C1, hidden_dropout=0.1, params_dtype=torch.float32, backend="eager"))
+    with pytest.raises(NotImplementedError):
+        LayerStack(LayerConfig(**C1, add_bias_linear=True, params_dtype=torch.float32, backend="eager"))
+    with pytest.raises(NotImplementedError):
+        NoOpAllReduce(world_size=2)
+    with pytest.raises(ValueError, match="unknown backend"):
+        LayerStack(LayerConfig(**C1, params_dtype=torch.float32, backend="triton"))(torch.randn(8, 2, 512))
+    store = TensorStore()
+    with pytest.raises(KeyError, match="tensor_id 't_9' not found"):
+        store.get("t_9")
+    with pytest.raises(AssertionError, match="Parameter gradient count mismatch"):
+        _flatten_grad_params({0: [None], 1: [None]}, 3)
+    with pytest.raises(AssertionError, match="parameter list repeated"):
+        TransformerBlockAutogradFunction.apply(torch.randn(2, 1, 512), torch.randn(2, 1, 512), None, None, m.forward_partitions,
+                                               m.backward_partitions, m.forward_tensor_graph, m.backward_tensor_graph,
+                                               None, cfg, m.seed_config, True, False, *m._get_all_params()[:5])
+
+
+def test_hip_backend_refuses_host_tensors_and_missing_library(monkeypatch):
+    from kareus_amd.backend import hip
+
+    if os.path.exists(hip.library_path()):
+        be = hip.HipBackend()
+        with pytest.raises(RuntimeError, match="HIP device"):
+            be.add(torch.zeros(8, dtype=torch.bfloat16), torch.zeros(8, dtype=torch.bfloat16))
+    monkeypatch.setattr(hip, "_LIB_NAME", "libdoes_not_exist.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        hip.load_library()
+
+
+def test_saved_tensor_bookkeeping():
+    ctx = NanoBatchContext(batch_idx=0)
+    a, b, c = torch.ones(1), torch.ones(2), torch.ones(3)
+    ctx.create_op_context(5).save_for_backward(c)
+    ctx.create_op_context(2).save_for_backward(a, b)
+    ctx.create_op_context(3)  # saves nothing
+    flat = ctx.flatten_saved_tensors()
+    assert [t.numel() for t in flat] == [1, 2, 3]  # op id order, not creation order
+    assert ctx.get_op_context(2).to_save is None
+    ctx.restore_saved_tensors(tuple(flat))
+    assert ctx.get_op_context(5).saved_tensors[0] is c and ctx.get_op_context(3).saved_tensors is None
+    ctx.clear_saved_tensors_except({id(a)})
+    assert a.numel() == 1 and b.numel() == 0 and c.numel() == 0
+
+
+def _replay(window, nnb=2, layers=1):
+    rec = RecordingStreams()
+    with use_stream_api(rec):
+        cfg = LayerConfig(hidden_size=64, num_attention_heads=2, num_query_groups=1, kv_channels=32, ffn_hidden_size=64,
+                          num_layers=layers, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager")
+        m = LayerStack(cfg, seed=1)
+        if window is not None:
+            cc = CommConfig(window, (20, 1024))
+
+            class Sch:
+                current_schedule = ScheduleItem(cc, cc, cc, cc)  # trail partitions keep the default window
+
+            cfg.kareus_scheduler = Sch()
+        PartitionBase.timer = rec
+        try:
+            x = torch.randn(16, 2 * nnb, 64, requires_grad=True)
+            m(x).sum().backward()
+        finally:
+            PartitionBase.timer = None
+    return rec
+
+
+def test_stream_protocol_replay():
+    # slot "none": a hand-over is released only after the carrying partition's compute, so from the
+    # second segment on the two nanobatches strictly alternate
+    rec = _replay(("none", "none"))
+    assert rec.violations == []
+    f = lambda key, nb: rec.find("ForwardPartition", key, nb)
+    assert rec.ordered(f("fwd_attn", 1), f("fwd_mlp", 0))   # NB0 seg 1 waits for NB1 seg 0
+    assert rec.ordered(f("fwd_mlp", 0), f("fwd_mlp", 1))    # NB1 seg 1 waits for NB0 seg 1
+    assert rec.may_overlap(f("fwd_attn", 0), f("fwd_attn", 1))  # nothing to hand over yet
+    # a nanobatch's own partitions are always ordered (same stream)
+    assert rec.ordered(f("fwd_attn", 0), f("fwd_mlp", 0)) and rec.ordered(f("fwd_attn", 1), f("fwd_mlp", 1))
+    b = lambda key, nb: rec.find("BackwardPartition", key, nb)
+    assert rec.ordered(b("bwd_mlp", 1), b("bwd_attn", 0)) and rec.ordered(b("bwd_attn", 0), b("bwd_attn", 1))
+    # forward finished on every stream before backward starts anywhere (join / fork)
+    assert rec.ordered(f("fwd_trail", 0), b("bwd_mlp", 1)) and rec.ordered(f("-", 1), b("bwd_mlp", 0))
+
+    # slot 0 (default window, or "norm_0"): released before the first op -> compute may overlap
+    for window in (None, ("norm_0", "none")):
+        rec = _replay(window)
+        assert rec.violations == []
+        f = lambda key, nb: rec.find("ForwardPartition", key, nb)
+        assert rec.may_overlap(f("fwd_attn", 1), f("fwd_mlp", 0))
+        assert rec.may_overlap(f("fwd_mlp", 0), f("fwd_mlp", 1))
+        assert rec.ordered(f("fwd_attn", 0), f("fwd_mlp", 0))
+        # the carrier still waits, at its end, until the owner has passed the hand-over
+        assert not rec.ordered(f("fwd_mlp", 1), f("fwd_attn", 0))
+
+    # a mid-partition slot: NB1's next segment may start once NB0's carrier passed that op
+    rec = _replay(("linear_0", "none"))
+    carrier, owner_next = rec.find("ForwardPartition", "fwd_mlp", 0), rec.find("ForwardPartition", "fwd_mlp", 1)
+    slot = carrier_slot = 3  # bda, fork, ln | fc1  -> linear_0 is op 3
+    assert rec.happens_before(carrier.op_done[slot - 1], owner_next.begin)
+    assert not rec.happens_before(carrier.op_done[slot], owner_next.begin)
+    assert rec.violations == []
+
+    for nnb in (1, 4):
+        rec = _replay(("norm_0", "none"), nnb=nnb, layers=2)
+        assert rec.violations == [] and len(rec.spans) == 2 * nnb * 5

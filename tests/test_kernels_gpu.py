@@ -1,0 +1,184 @@
+"""Parity of every HIP kernel with the CPU oracle, called through the C ABI (ctypes) on the same
+seeded inputs.  Integer-exact where the arithmetic is exact (residual add, index maps), otherwise
+bf16 tolerance: max |err| / max |ref| <= 2e-2 against the fp32 oracle evaluated on the bf16-rounded
+inputs (BASELINE's stated tolerance); observed errors are ~3e-3, one bf16 ulp."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import llama_layer_ref as R
+
+pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not torch.cuda.is_available(), reason="needs a HIP device")]
+TOL = 2e-2
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def be():
+    from kareus_amd.backend import get_backend
+
+    return get_backend("hip")
+
+
+def rel(got, want):
+    got, want = got.float().cpu(), want.float().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def rnd(*shape, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(DEV, torch.bfloat16)
+
+
+# ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("n", [8, 1000 * 512, 4096 * 4096, 13 * 8 + 5])
+def test_add_is_exact(be, n):
+    a, b = rnd(n, seed=1), rnd(n, seed=2)
+    assert torch.equal(be.add(a, b), a + b)
+    assert torch.equal(be.add(a, a), a + a)  # aliasing inputs (ResidualFork with identical grads)
+
+
+@pytest.mark.parametrize("rows,f", [(512, 1376), (64, 8), (1000, 1024), (2048, 3584)])
+def test_swiglu(be, rows, f):
+    x, dy = rnd(rows, 2 * f, seed=3), rnd(rows, f, seed=4)
+    assert rel(be.swiglu_fwd(x), R.swiglu(x.float())) <= TOL
+    assert rel(be.swiglu_bwd(dy, x), R.swiglu_bwd_formula(dy.float(), x.float())) <= TOL
+    big = torch.full((8, 16), 30.0, device=DEV, dtype=torch.bfloat16)  # saturated gate: y = x1*x2, finite
+    big[:, :8] *= -1
+    assert torch.isfinite(be.swiglu_fwd(big)).all() and be.swiglu_fwd(big).abs().max() < 1e-8
+
+
+@pytest.mark.parametrize("s,b,heads,hd", [(256, 2, 8, 128), (64, 1, 3, 64), (4096, 1, 2, 128)])
+def test_rope(be, s, b, heads, hd):
+    t = rnd(s, b, heads, hd, seed=5)
+    f = R.rope_table(s, hd, 500000.0).to(DEV)
+    y = be.rope_fwd(t, f)
+    assert rel(y, R.rope(t.float().cpu(), f.cpu())) <= TOL
+    assert rel(be.rope_bwd(t, f), R.rope(t.float().cpu(), -f.cpu())) <= TOL
+    assert torch.equal(y[0], t[0])  # position 0 is the identity, exactly
+    # strided input (a view into a wider buffer) gives the same result as its contiguous copy
+    wide = rnd(s, b, heads + 2, hd, seed=6)
+    assert torch.equal(be.rope_fwd(wide[:, :, 1:-1], f), be.rope_fwd(wide[:, :, 1:-1].contiguous(), f))
+
+
+def test_rope_fused_in_place_leaves_value_heads(be):
+    s, b, ng, per, hd = 128, 2, 2, 3, 128
+    fused = rnd(s, b, ng, per + 2, hd, seed=7)
+    before = fused.clone()
+    f = R.rope_table(s, hd, 500000.0).to(DEV)
+    be.rope_fused_inplace(fused, per, f, False)
+    ref = R.rope(before[:, :, :, : per + 1].flatten(2, 3).float().cpu(), f.cpu()).view(s, b, ng, per + 1, hd)
+    assert rel(fused[:, :, :, : per + 1], ref) <= TOL
+    assert torch.equal(fused[:, :, :, per + 1], before[:, :, :, per + 1])
+    be.rope_fused_inplace(fused, per, f, True)  # backward rotation undoes it up to rounding
+    assert rel(fused, before) <= TOL
+
+
+# ------------------------------------------------------------------ rmsnorm
+@pytest.mark.parametrize("rows,cols", [(1024, 512), (4096, 3072), (1000, 4096), (3, 8), (70, 8192), (257, 1376)])
+def test_rmsnorm(be, rows, cols):
+    x, dy = rnd(rows, cols, seed=8), rnd(rows, cols, seed=9)
+    g = (1 + 0.1 * torch.randn(cols, generator=torch.Generator().manual_seed(10))).to(DEV, torch.bfloat16)
+    y, rstd = be.rmsnorm_fwd(x, g, 1e-5)
+    assert rel(y, R.rmsnorm(x.float(), g.float(), 1e-5)) <= TOL
+    assert rel(rstd, torch.rsqrt(x.float().pow(2).mean(-1) + 1e-5)) <= 1e-5
+    dx, dg = be.rmsnorm_bwd(dy, x, rstd, g)
+    rdx, rdg = R.rmsnorm_bwd_formula(dy.float(), x.float(), g.float(), 1e-5)
+    assert rel(dx, rdx) <= TOL and rel(dg, rdg) <= TOL
+    const = torch.full((4, cols), 3.0, device=DEV, dtype=torch.bfloat16)  # closed form for a constant row
+    yc, _ = be.rmsnorm_fwd(const, torch.ones(cols, device=DEV, dtype=torch.bfloat16), 1e-5)
+    assert (yc.float() - 3.0 / math.sqrt(9.0 + 1e-5)).abs().max() < 1e-2
+
+
+# ------------------------------------------------------------------ GEMM
+SHAPES = [(256, 256, 64), (512, 768, 512), (264, 520, 200), (1024, 2752, 512), (2048, 512, 1376),
+          (8, 8, 8), (4096, 640, 384), (40, 1536, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_three_layouts(be, m, n, k):
+    x, w, dy = rnd(m, k, seed=11), rnd(n, k, scale=0.05, seed=12), rnd(m, n, seed=13)
+    assert rel(be.linear_fwd(x, w), x.float() @ w.float().t()) <= TOL
+    assert rel(be.linear_dgrad(dy, w), dy.float() @ w.float()) <= TOL
+    assert rel(be.linear_wgrad(dy, x), dy.float().t() @ x.float()) <= TOL
+
+
+def test_gemm_closed_forms(be):
+    eye = torch.eye(512, device=DEV, dtype=torch.bfloat16)
+    x = rnd(264, 512, seed=14)
+    assert torch.equal(be.linear_fwd(x, eye), x) and torch.equal(be.linear_dgrad(x, eye), x)  # identity weight
+    ones = torch.ones(128, 512, device=DEV, dtype=torch.bfloat16)
+    small = (torch.arange(264 * 512) % 7 - 3).reshape(264, 512).to(DEV, torch.bfloat16)  # exact small ints
+    assert torch.equal(be.linear_fwd(small, ones).float(), small.float().sum(1, keepdim=True).expand(264, 128))
+    onehot = torch.zeros(264, 8, device=DEV, dtype=torch.bfloat16)  # dW = dy^T x with one-hot dy picks rows of x
+    onehot[5, 3] = 1
+    dw = be.linear_wgrad(onehot, x)
+    assert torch.equal(dw[3], x[5]) and dw.abs().sum() == x[5].abs().sum()
+
+
+def test_gemm_split_k_accumulate_and_strides(be):
+    for (m, n, k) in [(512, 768, 4096), (264, 520, 2440)]:
+        dy, x = rnd(k, m, scale=0.1, seed=15), rnd(k, n, seed=16)
+        assert be.lib.kr_gemm_workspace_bytes(2, m, n, k) > 0  # this shape is computed split-K
+        ref = dy.float().t() @ x.float()
+        assert rel(be.linear_wgrad(dy, x), ref) <= TOL
+        c0 = rnd(m, n, seed=17)
+        assert rel(be.gemm(2, dy, x, m, n, k, out=c0.clone(), accumulate=True), ref + c0.float()) <= TOL
+    a, w, c0 = rnd(296, 512, seed=18), rnd(264, 512, seed=19), rnd(296, 264, seed=20)
+    assert rel(be.gemm(0, a, w, 296, 264, 512, out=c0.clone(), accumulate=True), a.float() @ w.float().t() + c0.float()) <= TOL
+    wide = rnd(296, 1024, seed=21)  # lda > K: operand is a column slice of a wider matrix
+    assert torch.equal(be.gemm(0, wide[:, 256:768], w, 296, 264, 512), be.gemm(0, wide[:, 256:768].contiguous(), w, 296, 264, 512))
+    with pytest.raises(RuntimeError, match="not supported"):
+        be.gemm(0, a[:295], w, 295, 264, 512)
+
+
+# ------------------------------------------------------------------ attention
+def _grouped(s, b, nq, nkv, hd, seed):
+    per = nq // nkv
+    fused = rnd(s, b, nkv, per + 2, hd, seed=seed)
+    return fused, fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1]
+
+
+@pytest.mark.parametrize("s,b,nq,nkv", [(128, 1, 1, 1), (256, 2, 4, 2), (512, 1, 3, 1), (384, 1, 8, 8), (1024, 1, 4, 1)])
+def test_attention_forward_backward(be, s, b, nq, nkv):
+    hd = 128
+    _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=22)
+    do = rnd(s, b, nq, hd, seed=23)
+    o, lse = be.attn_fwd(q, k, v, hd ** -0.5)
+    qf, kf, vf = (t.float().cpu().clone().requires_grad_(True) for t in (q.flatten(2, 3), k, v))
+    ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
+    assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
+    ro.backward(do.float().cpu())
+    dq, dk, dv = be.attn_bwd(do, q, k, v, o, lse, hd ** -0.5)
+    assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
+    assert dq._kr_mixed.shape == (s, b, (nq + 2 * nkv) * hd)  # gradients share one fused buffer
+    # dense [s, b, nq, hd] tensors go through the same kernels
+    qd = q.flatten(2, 3).contiguous()
+    od, lsed = be.attn_fwd(qd, k.contiguous(), v.contiguous(), hd ** -0.5)
+    assert torch.equal(od, o) and torch.equal(lsed, lse)
+    dqd, dkd, dvd = be.attn_bwd(do, qd, k.contiguous(), v.contiguous(), od, lsed, hd ** -0.5)
+    assert torch.equal(dqd, dq.flatten(2, 3)) and torch.equal(dkd, dk) and torch.equal(dvd, dv)
+
+
+def test_attention_special_cases(be):
+    hd, s = 128, 256
+    # all keys equal -> output row i is the mean of v[0..i]
+    q = rnd(s, 1, 1, hd, seed=24)
+    k = rnd(1, 1, 1, hd, seed=25).expand(s, 1, 1, hd).contiguous()
+    v = rnd(s, 1, 1, hd, seed=26)
+    o, lse = be.attn_fwd(q, k, v, hd ** -0.5)
+    want = torch.cumsum(v.float(), 0) / torch.arange(1, s + 1, device=DEV).view(s, 1, 1, 1)
+    assert rel(o, want) <= TOL
+    assert torch.equal(o[0], v[0])  # a single visible key: o = v exactly
+    # causality: changing later keys/values leaves earlier rows bit-identical
+    k2, v2 = k.clone(), v.clone()
+    k2[200:] += 1
+    v2[200:] -= 3
+    o2, _ = be.attn_fwd(q, k2, v2, hd ** -0.5)
+    assert torch.equal(o2[:200], o[:200])
+    with pytest.raises(RuntimeError, match="not supported"):
+        be.attn_fwd(rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), 1.0)  # s % 128 != 0
+    with pytest.raises(RuntimeError, match="not supported"):
+        be.attn_fwd(rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), 1.0)  # head_dim 64
