@@ -149,6 +149,26 @@ def dominant_kernel_roofline(w, nnb, device, launches=30):
     }
 
 
+def copy_calibration(device, n=1 << 29, launches=10):
+    """kr_add over n bf16 elements: reads 2*n*2 bytes, writes n*2 bytes per launch — the known-size
+    kernel against which the FETCH_SIZE / WRITE_SIZE counters are scaled."""
+    from kareus_amd.backend import get_backend
+
+    be = get_backend("hip")
+    a = torch.ones(n, device=device, dtype=torch.bfloat16)
+    b = torch.ones(n, device=device, dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(launches):
+        be.add(a, b)
+    e1.record()
+    torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3 / launches
+    return {"kernel": "add_kernel", "elements": n, "read_bytes": 4 * n, "write_bytes": 2 * n,
+            "avg_launch_us": sec * 1e6, "achieved_GBps": 6 * n / sec / 1e9}
+
+
 def cpu_baseline(w, budget_s=25.0):
     """The CPU oracle (fp32 PyTorch, autograd backward) on a bounded sample: same layer widths,
     one sequence of at most 1024 tokens, as many iterations as fit the time budget."""
@@ -186,6 +206,10 @@ def main():
     ap.add_argument("--nanobatches", type=int, default=0, help="override the workload's nanobatch count")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip serial/partition/energy legs")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the dominant-kernel leg (the command profiled under profiles/)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a residual-add kernel of known size (calibrates FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs one GPU's shard of the layer; --gpus must be 1 "
@@ -198,6 +222,12 @@ def main():
         w["nnb"] = args.nanobatches
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.roofline_only:
+        print(json.dumps({"roofline": dominant_kernel_roofline(w, w["nnb"], device)}))
+        return
+    if args.copy_calibration:
+        print(json.dumps({"copy_calibration": copy_calibration(device)}))
+        return
     gen = torch.Generator().manual_seed(42)
     x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
     go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)

@@ -84,13 +84,19 @@ struct TileLoader {
       rmax = 0;
     }
   }
-  __device__ __forceinline__ uint32_t goff(int i) const {
+  // k_left: contraction elements from this K-step's base to the end of the operand (>= 8).
+  // A chunk that would start beyond it is redirected to a valid address; it is zeroed in LDS
+  // afterwards, so what it fetches does not matter — only that the address is inside the matrix.
+  __device__ __forceinline__ uint32_t goff(int i, int k_left) const {
     if (!TRANSPOSED) {
       int r = r0 + 32 * i;
       r = r < rmax ? r : rmax;
-      return (uint32_t)(r * (int)ld + chunk);
+      const int kc = chunk + 8 <= k_left ? chunk : k_left - 8;
+      return (uint32_t)(r * (int)ld + kc);
     }
-    return (uint32_t)((r0 + 8 * i) * (int)ld + chunk);
+    int kr = r0 + 8 * i;
+    kr = kr < k_left ? kr : k_left - 1;
+    return (uint32_t)(kr * (int)ld + chunk);
   }
   // contraction index (relative to the K-step) covered by load i of this lane
   __device__ __forceinline__ int k_of(int i, int wave4, int lane) const {
@@ -100,11 +106,12 @@ struct TileLoader {
     }
     return 2 * (wave4 + 4 * i) + (lane >> 5);
   }
-  __device__ __forceinline__ void issue(const bf16* __restrict__ kbase, bf16* tile, int wave4) const {
+  __device__ __forceinline__ void issue(const bf16* __restrict__ kbase, bf16* tile, int wave4,
+                                        int k_left) const {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int b = wave4 + 4 * i;
-      __builtin_amdgcn_global_load_lds(kbase + goff(i), (KR_LDS void*)(tile + b * 512), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(kbase + goff(i, k_left), (KR_LDS void*)(tile + b * 512), 16, 0, 0);
     }
   }
   // zero this lane's chunks whose contraction index is >= k_valid (tile already landed)
@@ -257,8 +264,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       la.init(lda, m0, M, wave4, l2);
       lb.init(ldb, n0, N, wave4, l2);
       bf16* st = smem + (t & 1) * STAGE;
-      la.issue(A + t * a_step, st, wave4);
-      lb.issue(B + t * b_step, st + TILE, wave4);
+      la.issue(A + t * a_step, st, wave4, K - t * BK);
+      lb.issue(B + t * b_step, st + TILE, wave4, K - t * BK);
     };
     auto land_tile = [&](int t) {  // all of this wave's outstanding loads are done; fix a K tail
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
