@@ -120,6 +120,15 @@ def partition_times(model, x, go, iters=3):
     return {k: v / iters for k, v in timer.totals().items()}
 
 
+# HBM-side bytes per launch of the TN GEMM, from hardware counters (FETCH_SIZE and WRITE_SIZE of
+# two profiler runs of `bench.py --roofline-only`, each scaled by what the same counter reads for
+# `bench.py --copy-calibration`: x2.000 and x1.000).  Keyed by (M, N, K); shapes that were not
+# profiled report null.
+MEASURED_TRAFFIC_BYTES = {
+    (4096, 7168, 4096): 369.3e6 + 59.8e6,
+}
+
+
 def dominant_kernel_roofline(w, nnb, device, launches=30):
     """fc1 forward GEMM, y[T_nb, 2F] = x[T_nb, h] . W[2F, h]^T, timed with HIP events on the
     stream it is launched on (torch's current stream)."""
@@ -145,7 +154,8 @@ def dominant_kernel_roofline(w, nnb, device, launches=30):
         "bound": "mfma", "kernel": "gemm_kernel<TN> (fc1 forward)", "shape": [m, n, k],
         "flops_per_launch": flops, "avg_launch_us": sec * 1e6,
         "achieved": achieved, "peak": MFMA_PEAK_BF16 / 1e12, "unit": "TFLOP/s",
-        "frac": achieved * 1e12 / MFMA_PEAK_BF16, "traffic": None,
+        "frac": achieved * 1e12 / MFMA_PEAK_BF16,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((m, n, k)),
     }
 
 
