@@ -10,15 +10,21 @@
 //   * The waves form two groups of four, one wave of each group per SIMD.  Time is cut into
 //     half-periods by workgroup barriers.  In every half-period one group only issues MFMAs
 //     (all 32 of a K-step, operands already in registers) while the other group only moves
-//     data: it reads its operand fragments for the same K-step out of LDS and (group 0) issues
-//     the global loads of a later K-step.  Then the roles swap.  The matrix pipe of every SIMD
-//     always has exactly one wave feeding it, and no wave ever waits on memory in the middle
-//     of its MFMA burst.
+//     data: it issues the global loads of one operand tile of K-step k+2 and reads its operand
+//     fragments of the next K-step out of LDS.  Then the roles swap.  The matrix pipe of every
+//     SIMD always has exactly one wave feeding it, and no wave ever waits on memory in the
+//     middle of its MFMA burst.
 //   * Global memory goes straight into LDS (global_load_lds_dwordx4): no staging registers, no
 //     LDS store instructions.  The hardware places the 64 lanes of such a load contiguously in
 //     LDS, so bank conflicts are avoided by an XOR swizzle applied on the *global* side — each
-//     lane fetches the 16-byte chunk that belongs at its LDS slot.  Two LDS stages; the tile
-//     of K-step k+2 is requested while step k is being consumed.
+//     lane fetches the 16-byte chunk that belongs at its LDS slot.
+//   * All 160 KB of LDS form a ring of five 32 KB slots, one operand tile (A or B of one
+//     K-step) per slot: two slots are being consumed, three are being filled.  Group 1 requests
+//     the A tiles (a flight window of three half-periods), group 0 the B tiles (two
+//     half-periods), so the texture-address path sees an even 32 KB per half-period — half of
+//     what it can carry — and every load has at least a full half-period to land after the
+//     last request of its tile went out.  With only two 64 KB stages the loads of a whole
+//     K-step had to be pushed out back to back and their tail had no time left.
 //   * Loads are 16-byte vectors along whichever dimension is contiguous in memory.  An operand
 //     whose contraction dimension is contiguous ("K-major") is fetched from LDS with
 //     ds_read_b128; an operand whose contraction dimension is the row index ("transposed": the
@@ -46,7 +52,7 @@ constexpr int BM = 256, BN = 256;
 constexpr int TM = 4, TN = 2;  // 32x32 MFMA tiles per wave: 128 rows x 64 columns
 constexpr int NTHREADS = 512;
 constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
-constexpr int STAGE = 2 * TILE;
+constexpr int NSLOTS = 5;          // 5 x 32 KB = the whole 160 KB of LDS
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;
 
@@ -58,6 +64,25 @@ __device__ __forceinline__ int kmajor_off(int row, int chunk) {
 // transposed tile [64 k-rows][256]: 512-byte rows, chunk index XORed with 4*(krow&3).
 __device__ __forceinline__ int transp_off(int krow, int col) {
   return krow * 256 + ((((col >> 3) ^ ((krow & 3) << 2))) << 3) + (col & 7);
+}
+
+// ---- direct global -> LDS loads ---------------------------------------------------------------
+// Issued through inline assembly on purpose.  A workgroup barrier is a release fence for LDS,
+// and the compiler drains every LDS-direct load it knows of (vmcnt(0)) in front of one — which
+// would empty the prefetch pipeline twice per K-step.  Written this way the loads are invisible
+// to its wait-count bookkeeping; their completion is tracked by hand with explicit vmcnt waits
+// placed before the barrier that publishes the data.  The loads have no register destination,
+// so nothing can be clobbered behind the register allocator's back.
+// base: wave-uniform global address; byte_off: this lane's unsigned 32-bit byte offset from it;
+// lds_byte: wave-uniform LDS byte address of a 1-KiB block (lane p lands at +16p).
+__device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, uint32_t lds_byte) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_byte), "v"(byte_off), "s"(base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const bf16* p) {
+  return (uint32_t)(uintptr_t)(KR_LDS const bf16*)p;
 }
 
 // ---- direct global -> LDS tile loads, issued by the 4 waves of the loading group -----------
@@ -111,7 +136,7 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int b = wave4 + 4 * i;
-      __builtin_amdgcn_global_load_lds(kbase + goff(i, k_left), (KR_LDS void*)(tile + b * 512), 16, 0, 0);
+      dma_b128(kbase, goff(i, k_left) * 2u, lds_addr(tile + b * 512));
     }
   }
   // zero this lane's chunks whose contraction index is >= k_valid (tile already landed)
@@ -147,24 +172,39 @@ struct FragReader {
         base[t] = transp_off(krow, row0 + 32 * t + ((lane >> 4) & 1) * 16 + (p & 3) * 4);
     }
   }
-  __device__ __forceinline__ bf16x8 read(const bf16* tile, int t, int kk) const {
+  // LDS byte address of this lane's base n inside `tile`, made opaque so that the compiler adds
+  // nothing but instruction immediates (all below 64 KiB) to it and keeps no per-slot copies.
+  __device__ __forceinline__ uint32_t addr(const bf16* tile, int n) const {
+    uint32_t v = (uint32_t)(uintptr_t)(KR_LDS const bf16*)tile + 2u * (uint32_t)base[n];
+    asm volatile("" : "+v"(v));
+    return v;
+  }
+  static constexpr int NBASE = TRANSPOSED ? NTILES : BK / 16;
+  // a[]: addr(tile, n) for every base n
+  __device__ __forceinline__ bf16x8 read(const uint32_t (&a)[NBASE], int t, int kk) const {
     if (!TRANSPOSED) {
-      return *reinterpret_cast<const bf16x8*>(tile + base[kk] + t * 32 * BK);
+      return *(KR_LDS const bf16x8*)(a[kk] + 2u * (uint32_t)(t * 32 * BK));
     } else {
       // Transposing read: within each group of 16 lanes, lane p supplies the address of 4
       // consecutive row-of-C elements in contraction row (p/4); it receives, for its own
       // row-of-C, the elements of the group's 4 contraction rows.
-      const bf16* a0 = tile + base[t] + kk * 16 * 256;
+      const uint32_t a0 = a[t] + 2u * (uint32_t)(kk * 16 * 256);
       union {
         struct { s16x4 lo, hi; } s;
         bf16x8 v;
       } u;
       u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
-      u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 4 * 256));
+      u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 2u * 4 * 256));
       return u.v;
     }
   }
 };
+
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, int tiles_n,
                                             int& tm, int& tn) {
@@ -227,15 +267,20 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   FragReader<B_T, TN> fb;
   fa.init(wm * TM * 32, lane);
   fb.init(wn * TN * 32, lane);
-  auto read_frags = [&](int stage) {
-    const bf16* at = smem + stage * STAGE;
-    const bf16* bt = at + TILE;
+  auto read_frags = [&](int t) {
+    const bf16* at = smem + ((2 * t) % NSLOTS) * TILE;
+    const bf16* bt = smem + ((2 * t + 1) % NSLOTS) * TILE;
+    uint32_t aa[fa.NBASE], ba[fb.NBASE];
+#pragma unroll
+    for (int n = 0; n < fa.NBASE; ++n) aa[n] = fa.addr(at, n);
+#pragma unroll
+    for (int n = 0; n < fb.NBASE; ++n) ba[n] = fb.addr(bt, n);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) af[kk][i] = fa.read(at, i, kk);
+      for (int i = 0; i < TM; ++i) af[kk][i] = fa.read(aa, i, kk);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bfr[kk][j] = fb.read(bt, j, kk);
+      for (int j = 0; j < TN; ++j) bfr[kk][j] = fb.read(ba, j, kk);
     }
   };
   auto compute = [&]() {
@@ -251,49 +296,80 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     __builtin_amdgcn_s_setprio(0);
   };
 
-  if (group == 0) {
-    TileLoader<A_T> la;
-    TileLoader<B_T> lb;
-    la.init(lda, m0, M, wave4, lane);
-    lb.init(ldb, n0, N, wave4, lane);
-    auto issue_tile = [&](int t) {
-      // The per-lane load coordinates are recomputed here from an opaque copy of the lane id:
-      // keeping them alive across the MFMA phases would push the wave over its register budget.
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));
+  // LDS is a ring of five 32 KB slots; operand tile x (0 = A, 1 = B) of K-step t lives in slot
+  // (2t + x) mod 5.  Two slots hold the K-step being consumed, three are being filled.
+  auto slot_of = [&](int t, int x) { return smem + ((2 * t + x) % NSLOTS) * TILE; };
+  // Each group loads one operand: group 1 the A tiles, group 0 the B tiles, 8 loads per wave.
+  // The per-lane load coordinates are recomputed from an opaque copy of the lane id every time:
+  // keeping them alive across the MFMA phases would push the wave over its register budget.
+  auto issue_mine = [&](int t) {
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));
+    if (group) {
+      TileLoader<A_T> la;
       la.init(lda, m0, M, wave4, l2);
+      la.issue(A + t * a_step, slot_of(t, 0), wave4, K - t * BK);
+    } else {
+      TileLoader<B_T> lb;
       lb.init(ldb, n0, N, wave4, l2);
-      bf16* st = smem + (t & 1) * STAGE;
-      la.issue(A + t * a_step, st, wave4, K - t * BK);
-      lb.issue(B + t * b_step, st + TILE, wave4, K - t * BK);
-    };
-    auto land_tile = [&](int t) {  // all of this wave's outstanding loads are done; fix a K tail
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
-      if (t == nk - 1 && k_tail < BK) {
-        bf16* st = smem + (t & 1) * STAGE;
-        la.zero_tail(st, k_tail, wave4, lane);
-        lb.zero_tail(st + TILE, k_tail, wave4, lane);
-      }
-    };
-    issue_tile(0);
-    land_tile(0);
-    if (nk > 1) issue_tile(1);
-    __syncthreads();  // tile 0 visible to everyone
+      lb.issue(B + t * b_step, slot_of(t, 1), wave4, K - t * BK);
+    }
+  };
+  // After this wave's loads of tile t have landed: zero a contraction tail of the last K-step.
+  auto fix_tail_mine = [&](int t) {
+    if (t != nk - 1 || k_tail == BK) return;
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));
+    if (group) {
+      TileLoader<A_T> la;
+      la.init(lda, m0, M, wave4, l2);
+      la.zero_tail(slot_of(t, 0), k_tail, wave4, l2);
+    } else {
+      TileLoader<B_T> lb;
+      lb.init(ldb, n0, N, wave4, l2);
+      lb.zero_tail(slot_of(t, 1), k_tail, wave4, l2);
+    }
+  };
+
+  // prologue: K-steps 0 and 1 complete in LDS
+  issue_mine(0);
+  if (nk > 1) issue_mine(1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
+  if (nk == 1) fix_tail_mine(0);
+  __syncthreads();
+
+  if (group == 0) {
     read_frags(0);
     for (int ks = 0; ks < nk; ++ks) {
-      __syncthreads();  // half-period 2ks: this group computes, the other reads fragments
+      lds_barrier();  // half-period 2ks: this group computes, the other moves data
       compute();
-      if (ks + 1 < nk) land_tile(ks + 1);
-      __syncthreads();  // half-period 2ks+1: this group moves data, the other computes
-      if (ks + 2 < nk) issue_tile(ks + 2);  // stage ks&1 is free: both groups hold step ks in registers
-      if (ks + 1 < nk) read_frags((ks + 1) & 1);
+      if (ks + 1 < nk) {
+        // B of step ks+1 was requested one K-step ago
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        fix_tail_mine(ks + 1);
+      }
+      lds_barrier();  // half-period 2ks+1: this group moves data, the other computes
+      // B(ks+2) replaces A(ks), which group 1 finished reading before the barrier above
+      if (ks + 2 < nk) issue_mine(ks + 2);
+      if (ks + 1 < nk) read_frags(ks + 1);
     }
   } else {
-    __syncthreads();
     for (int ks = 0; ks < nk; ++ks) {
-      __syncthreads();
-      read_frags(ks & 1);
-      __syncthreads();
+      lds_barrier();
+      // A(ks+2) replaces B(ks-1), dead since the previous K-step
+      if (ks + 2 < nk) issue_mine(ks + 2);
+      read_frags(ks);
+      if (ks + 1 < nk) {
+        // A of step ks+1 (requested one K-step ago) must be in LDS before group 0 reads it
+        // after the next barrier; the 8 loads just issued may stay in flight (loads retire in
+        // order)
+        if (ks + 2 < nk)
+          __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+        else
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+        fix_tail_mine(ks + 1);
+      }
+      lds_barrier();
       compute();
     }
   }
@@ -390,7 +466,7 @@ template <bool A_T, bool B_T>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
            hipStream_t stream) {
-  constexpr size_t lds_bytes = 2 * STAGE * sizeof(bf16);
+  constexpr size_t lds_bytes = NSLOTS * TILE * sizeof(bf16);
   // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
   static const hipError_t attr_status =
       hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T>,
