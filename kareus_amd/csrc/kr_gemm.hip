@@ -131,6 +131,10 @@ struct TileLoader {
     }
     return 2 * (wave4 + 4 * i) + (lane >> 5);
   }
+  __device__ __forceinline__ void issue_one(const bf16* __restrict__ kbase, bf16* tile, int wave4,
+                                            int k_left, int i) const {
+    dma_b128(kbase, goff(i, k_left) * 2u, lds_addr(tile + (wave4 + 4 * i) * 512));
+  }
   __device__ __forceinline__ void issue(const bf16* __restrict__ kbase, bf16* tile, int wave4,
                                         int k_left) const {
 #pragma unroll
@@ -315,6 +319,49 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       lb.issue(B + t * b_step, slot_of(t, 1), wave4, K - t * BK);
     }
   };
+  // The data-movement half-period: read this wave's fragments of K-step t_read and request
+  // this wave's 8 blocks of K-step t_load, one request after every third fragment read.  The
+  // texture-address path takes about as long to accept a group's 32 KB as LDS takes to deliver
+  // its fragments; back to back the two would outlast the other group's MFMA burst, woven
+  // together they fit inside it.
+  auto move_data = [&](int t_read, int t_load) {
+    const bf16* at = smem + ((2 * t_read) % NSLOTS) * TILE;
+    const bf16* bt = smem + ((2 * t_read + 1) % NSLOTS) * TILE;
+    uint32_t aa[fa.NBASE], ba[fb.NBASE];
+#pragma unroll
+    for (int n = 0; n < fa.NBASE; ++n) aa[n] = fa.addr(at, n);
+#pragma unroll
+    for (int n = 0; n < fb.NBASE; ++n) ba[n] = fb.addr(bt, n);
+    auto body = [&](const auto& loader, const bf16* kbase, bf16* dst) {
+      const int k_left = K - t_load * BK;
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          af[kk][i] = fa.read(aa, i, kk);
+          const int n = kk * (TM + TN) + i;
+          if (n % 3 == 2) loader.issue_one(kbase, dst, wave4, k_left, n / 3);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          bfr[kk][j] = fb.read(ba, j, kk);
+          const int n = kk * (TM + TN) + TM + j;
+          if (n % 3 == 2) loader.issue_one(kbase, dst, wave4, k_left, n / 3);
+        }
+      }
+    };
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));
+    if (group) {
+      TileLoader<A_T> la;
+      la.init(lda, m0, M, wave4, l2);
+      body(la, A + t_load * a_step, slot_of(t_load, 0));
+    } else {
+      TileLoader<B_T> lb;
+      lb.init(ldb, n0, N, wave4, l2);
+      body(lb, B + t_load * b_step, slot_of(t_load, 1));
+    }
+  };
   // After this wave's loads of tile t have landed: zero a contraction tail of the last K-step.
   auto fix_tail_mine = [&](int t) {
     if (t != nk - 1 || k_tail == BK) return;
@@ -350,15 +397,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       }
       lds_barrier();  // half-period 2ks+1: this group moves data, the other computes
       // B(ks+2) replaces A(ks), which group 1 finished reading before the barrier above
-      if (ks + 2 < nk) issue_mine(ks + 2);
-      if (ks + 1 < nk) read_frags(ks + 1);
+      if (ks + 2 < nk)
+        move_data(ks + 1, ks + 2);
+      else if (ks + 1 < nk)
+        read_frags(ks + 1);
     }
   } else {
     for (int ks = 0; ks < nk; ++ks) {
       lds_barrier();
       // A(ks+2) replaces B(ks-1), dead since the previous K-step
-      if (ks + 2 < nk) issue_mine(ks + 2);
-      read_frags(ks);
+      if (ks + 2 < nk)
+        move_data(ks, ks + 2);
+      else
+        read_frags(ks);
       if (ks + 1 < nk) {
         // A of step ks+1 (requested one K-step ago) must be in LDS before group 0 reads it
         // after the next barrier; the 8 loads just issued may stay in flight (loads retire in
