@@ -216,6 +216,8 @@ def main():
     ap.add_argument("--nanobatches", type=int, default=0, help="override the workload's nanobatch count")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip serial/partition/energy legs")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="run every nanobatch on the caller's stream (no overlap; for profiling)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant-kernel leg (the command profiled under profiles/)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -244,7 +246,7 @@ def main():
     tokens = w["b"] * w["s"]
     flops = total_flops(w)
 
-    model = make_model(w, w["nnb"], device)
+    model = make_model(w, w["nnb"], device, use_streams=not args.one_stream)
     sec = time_steps(model, x, go, args.steps, args.warmup)
 
     out = {

@@ -24,8 +24,15 @@ class EagerBackend:
     def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
         return dy @ w
 
-    def linear_wgrad(self, dy: Tensor, x: Tensor) -> Tensor:
-        return dy.t() @ x
+    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False) -> Tensor:
+        dw = dy.t() @ x
+        if out is None:
+            return dw
+        if accumulate:
+            out.add_(dw)
+        else:
+            out.copy_(dw)
+        return out
 
     # rs = rsqrt(mean(x^2) + eps) in fp32, y = (x * rs) * gamma
     # (3rdparty/TransformerEngine/transformer_engine/common/normalization/rmsnorm/

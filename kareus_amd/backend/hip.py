@@ -113,8 +113,9 @@ class HipBackend:
     def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
         return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1])
 
-    def linear_wgrad(self, dy: Tensor, x: Tensor) -> Tensor:
-        return self.gemm(KR_GEMM_NT, dy, x, dy.shape[1], x.shape[1], dy.shape[0])
+    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False) -> Tensor:
+        return self.gemm(KR_GEMM_NT, dy, x, dy.shape[1], x.shape[1], dy.shape[0], out=out,
+                         accumulate=accumulate)
 
     # -- RMSNorm ----------------------------------------------------------------------
     def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:

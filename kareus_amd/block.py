@@ -67,6 +67,8 @@ class LayerConfig:
     backend: str = "hip"
     use_streams: bool = True
     checkpoint_activations: bool = False
+    # weight gradients of all nanobatches are summed inside the wgrad GEMM instead of by autograd
+    fuse_wgrad_accumulation: bool = True
     hidden_dropout: float = 0.0
     attention_dropout: float = 0.0
     add_bias_linear: bool = False

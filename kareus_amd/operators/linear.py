@@ -22,6 +22,7 @@ import torch
 
 from ..backend import get_backend
 from ..partitions.op_context import BasicOperation
+from ..partitions.streams import stream_api
 from ..partitions.tensor_graph import (
     Channel,
     CommunicationOpSpec,
@@ -82,8 +83,37 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
             dy = dy.contiguous()
         be = get_backend(self._backend_name)
         dx = be.linear_dgrad(dy, self.weight.detach())
-        dw = be.linear_wgrad(dy, x2d) if self.weight.requires_grad else None
+        dw = self._weight_grad(be, ctx, dy, x2d) if self.weight.requires_grad else None
         return dx.view(*grad_output.shape[:-1], k), (dw,)
+
+    @staticmethod
+    def _weight_grad(be, ctx, dy, x2d):
+        """``dW = dy^T . x``.  When the engine attached a ``wgrad_sink`` — one dict shared by
+        this layer's contexts of all nanobatches of one backward pass — the first nanobatch to
+        get here allocates the gradient and every later one adds its product into the same
+        buffer inside the GEMM (the role of ``accumulate_into_main_grad``,
+        kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:898-909), after waiting for
+        the previous writer's event; later nanobatches then report ``None`` so that autograd
+        does not sum a second time."""
+        sink = getattr(ctx, "wgrad_sink", None)
+        if sink is None:
+            return be.linear_wgrad(dy, x2d)
+        api = stream_api()
+        here = api.current_stream()
+        buf = sink.get("buf")
+        if buf is None:
+            buf = sink["buf"] = be.linear_wgrad(dy, x2d)
+            ret = buf
+        else:
+            if here is not None and sink.get("event") is not None:
+                here.wait_event(sink["event"])
+            be.linear_wgrad(dy, x2d, out=buf, accumulate=True)
+            ret = None
+        if here is not None:
+            ev = api.new_event()
+            ev.record(here)
+            sink["event"] = ev
+        return ret
 
     def __repr__(self) -> str:
         return (f"{type(self).__name__}(in_features={self.weight.shape[1]}, "

@@ -157,6 +157,7 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         func_ctx.rotary_pos_emb = rotary
         func_ctx.attention_mask = mask
         func_ctx.checkpoint_activations = checkpoint_activations
+        func_ctx.fuse_wgrad_accumulation = bool(getattr(config, "fuse_wgrad_accumulation", False))
 
         if checkpoint_activations:
             func_ctx.forward_partitions = fwd_parts
@@ -209,6 +210,13 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         for c, g in zip(ctxs, grad_outs):
             c.tensor_store = TensorStore()
             c.tensor_store.set(seed.bwd_grad_tid, g)
+
+        if func_ctx.fuse_wgrad_accumulation and n > 1:
+            # one sink per layer operator, shared by that operator's contexts of all nanobatches
+            sinks: Dict[int, dict] = {}
+            for c in ctxs:
+                for op_id, op_ctx in c.op_contexts.items():
+                    op_ctx.wgrad_sink = sinks.setdefault(op_id, {})
 
         protected = {id(t) for t in (rotary, mask) if t is not None}
         per_nb: List[Dict[int, List]] = [{} for _ in range(n)]

@@ -60,6 +60,24 @@ def test_config1_matches_oracle(nnb, recompute):
     _check(LayerStack(cfg, seed=1234), x, go, ref)
 
 
+@pytest.mark.parametrize("recompute", [False, True])
+def test_fused_weight_gradient_accumulation_equals_autograd_sum(recompute):
+    """With the fusion on, the first nanobatch's wgrad buffer receives the other nanobatches'
+    products (later copies report None); with it off autograd sums N separate gradients.  Both
+    must give the oracle's gradient."""
+    x, go, ref = _oracle(layers=2, s=128, b=4)
+    grads = {}
+    for fuse in (True, False):
+        cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=4, params_dtype=torch.float32,
+                          backend="eager", checkpoint_activations=recompute,
+                          fuse_wgrad_accumulation=fuse)
+        model = LayerStack(cfg, seed=1234)
+        _check(model, x, go, ref)
+        grads[fuse] = [p.grad.clone() for p in model.parameters()]
+    for a, b in zip(grads[True], grads[False]):
+        assert (a - b).abs().max() <= 1e-5 * b.abs().max()
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
