@@ -227,51 +227,57 @@ __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, i
 }
 
 template <bool A_T, bool B_T>
-__global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int64_t lda,
-                                                        const bf16* __restrict__ B, int64_t ldb,
-                                                        bf16* __restrict__ C, int64_t ldc, int M,
+__global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
+                                                        const bf16* __restrict__ B, int ldb,
+                                                        bf16* __restrict__ C, int ldc, int M,
                                                         int N, int K, int accumulate, int k_per,
-                                                        float* __restrict__ partial) {
+                                                        int splits, float* __restrict__ partial) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  // split-K: blockIdx.y owns contraction range [y*k_per, y*k_per + K) and writes an fp32
-  // partial tile instead of C (k_per is a multiple of 64)
-  if (partial != nullptr) {
-    const int k0 = blockIdx.y * k_per;
-    A += A_T ? (int64_t)k0 * lda : k0;
-    B += B_T ? (int64_t)k0 * ldb : k0;
-    K = (K - k0) < k_per ? (K - k0) : k_per;
-    partial += (int64_t)blockIdx.y * M * N;
-  }
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int group = wave >> 2;  // 0: loads + computes first, 1: computes second
+  const int group = wave >> 2;  // 0: computes first and requests the B tiles, 1: the A tiles
   const int wave4 = wave & 3;
   const int wm = group, wn = wave4;  // wave tile: rows wm*128.., columns wn*64..
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  int tile_m, tile_n;
-  remap_block(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int nk = (K + BK - 1) / BK;
-  const int k_tail = K - (nk - 1) * BK;  // valid contraction rows of the last K-step (1..64)
-  const int64_t a_step = A_T ? (int64_t)BK * lda : BK;
-  const int64_t b_step = B_T ? (int64_t)BK * ldb : BK;
+  const int ntiles = tiles_m * tiles_n;
+  const bool split_k = partial != nullptr;
+
+  // Persistent workgroups: work item v = (output tile, split-K range); this workgroup takes
+  // items blockIdx.x, blockIdx.x + gridDim.x, ...  The state below describes the current item.
+  // (element offsets fit 32 bits: the host checks rows * ld < 2^31 and the workspace size)
+  int m0, n0, nk, k_tail, kc = K, a_off = 0, b_off = 0, p_off = 0;
+  auto select_item = [&](int v) {
+    const int split = v / ntiles;
+    int tile_m, tile_n;
+    remap_block(v - split * ntiles, ntiles, tiles_m, tiles_n, tile_m, tile_n);
+    m0 = tile_m * BM;
+    n0 = tile_n * BN;
+    if (split_k) {
+      // split-K: contraction range [split*k_per, split*k_per + kc), fp32 partial tile out
+      // (k_per is a multiple of 64)
+      const int k0 = split * k_per;
+      a_off = A_T ? k0 * lda : k0;
+      b_off = B_T ? k0 * ldb : k0;
+      kc = (K - k0) < k_per ? (K - k0) : k_per;
+      p_off = split * M * N;
+    }
+    nk = (kc + BK - 1) / BK;
+    k_tail = kc - (nk - 1) * BK;  // valid contraction rows of the last K-step (1..64)
+  };
 
   f32x16 acc[TN][TM];
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
-
   bf16x8 af[BK / 16][TM], bfr[BK / 16][TN];
 
-  FragReader<A_T, TM> fa;
-  FragReader<B_T, TN> fb;
-  fa.init(wm * TM * 32, lane);
-  fb.init(wn * TN * 32, lane);
+  // Per-lane fragment offsets are recomputed from an opaque copy of the lane id whenever
+  // fragments are read (a handful of VALU instructions in the data-movement half-period)
+  // instead of occupying eight registers through the MFMA phases.
   auto read_frags = [&](int t) {
+    int lf = lane;
+    asm volatile("" : "+v"(lf));
+    FragReader<A_T, TM> fa;
+    FragReader<B_T, TN> fb;
+    fa.init(wm * TM * 32, lf);
+    fb.init(wn * TN * 32, lf);
     const bf16* at = smem + ((2 * t) % NSLOTS) * TILE;
     const bf16* bt = smem + ((2 * t + 1) % NSLOTS) * TILE;
     uint32_t aa[fa.NBASE], ba[fb.NBASE];
@@ -312,11 +318,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     if (group) {
       TileLoader<A_T> la;
       la.init(lda, m0, M, wave4, l2);
-      la.issue(A + t * a_step, slot_of(t, 0), wave4, K - t * BK);
+      la.issue(A + a_off + (int64_t)t * (A_T ? BK * lda : BK), slot_of(t, 0), wave4, kc - t * BK);
     } else {
       TileLoader<B_T> lb;
       lb.init(ldb, n0, N, wave4, l2);
-      lb.issue(B + t * b_step, slot_of(t, 1), wave4, K - t * BK);
+      lb.issue(B + b_off + (int64_t)t * (B_T ? BK * ldb : BK), slot_of(t, 1), wave4, kc - t * BK);
     }
   };
   // The data-movement half-period: read this wave's fragments of K-step t_read and request
@@ -325,6 +331,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // its fragments; back to back the two would outlast the other group's MFMA burst, woven
   // together they fit inside it.
   auto move_data = [&](int t_read, int t_load) {
+    int lf = lane;
+    asm volatile("" : "+v"(lf));
+    FragReader<A_T, TM> fa;
+    FragReader<B_T, TN> fb;
+    fa.init(wm * TM * 32, lf);
+    fb.init(wn * TN * 32, lf);
     const bf16* at = smem + ((2 * t_read) % NSLOTS) * TILE;
     const bf16* bt = smem + ((2 * t_read + 1) % NSLOTS) * TILE;
     uint32_t aa[fa.NBASE], ba[fb.NBASE];
@@ -333,7 +345,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
     for (int n = 0; n < fb.NBASE; ++n) ba[n] = fb.addr(bt, n);
     auto body = [&](const auto& loader, const bf16* kbase, bf16* dst) {
-      const int k_left = K - t_load * BK;
+      const int k_left = kc - t_load * BK;
 #pragma unroll
       for (int kk = 0; kk < BK / 16; ++kk) {
 #pragma unroll
@@ -355,11 +367,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     if (group) {
       TileLoader<A_T> la;
       la.init(lda, m0, M, wave4, l2);
-      body(la, A + t_load * a_step, slot_of(t_load, 0));
+      body(la, A + a_off + (int64_t)t_load * (A_T ? BK * lda : BK), slot_of(t_load, 0));
     } else {
       TileLoader<B_T> lb;
       lb.init(ldb, n0, N, wave4, l2);
-      body(lb, B + t_load * b_step, slot_of(t_load, 1));
+      body(lb, B + b_off + (int64_t)t_load * (B_T ? BK * ldb : BK), slot_of(t_load, 1));
     }
   };
   // After this wave's loads of tile t have landed: zero a contraction tail of the last K-step.
@@ -378,12 +390,24 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     }
   };
 
-  // prologue: K-steps 0 and 1 complete in LDS
+  const int total_items = ntiles * (split_k ? splits : 1);
+  int item = blockIdx.x;
+  select_item(item);
+  // K-steps 0 and 1 of the first item
   issue_mine(0);
   if (nk > 1) issue_mine(1);
+
+  for (;;) {
+  // K-steps 0 and 1 complete in LDS (requested above, or before the previous item's epilogue)
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
   if (nk == 1) fix_tail_mine(0);
   __syncthreads();
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
 
   if (group == 0) {
     read_frags(0);
@@ -425,23 +449,36 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     }
   }
 
+
+  // Every LDS read of this item finished before the last barrier, so the ring is free: request
+  // the first two K-steps of the next item now and let them fly during the epilogue.
+  const int out_m0 = m0, out_n0 = n0;
+  float* const out_partial = split_k ? partial + p_off : nullptr;
+  const int next = item + (int)gridDim.x;
+  const bool more = next < total_items;
+  if (more) {
+    select_item(next);
+    issue_mine(0);
+    if (nk > 1) issue_mine(1);
+  }
+
   // epilogue: lane holds C[m][n..n+3] for m = tile row (lane%32), n = 8g + 4*(lane/32)
   const int h = lane >> 5;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m0 + (wm * TM + i) * 32 + (lane & 31);
+    const int m = out_m0 + (wm * TM + i) * 32 + (lane & 31);
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int n = n0 + (wn * TN + j) * 32 + 8 * g + 4 * h;
+        const int n = out_n0 + (wn * TN + j) * 32 + 8 * g + 4 * h;
         if (n >= N) continue;
-        if (partial != nullptr) {
+        if (out_partial != nullptr) {
           f32x4 pv;
 #pragma unroll
           for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
-          *reinterpret_cast<f32x4*>(partial + (int64_t)m * N + n) = pv;
+          *reinterpret_cast<f32x4*>(out_partial + (int64_t)m * N + n) = pv;
           continue;
         }
         bf16* dst = C + (int64_t)m * ldc + n;
@@ -458,15 +495,18 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       }
     }
   }
+  if (!more) break;
+  item = next;
+  }
 }
 
 // the three layouts the library serves
-template __global__ void gemm_kernel<false, false>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                   int64_t, int, int, int, int, int, float*);
-template __global__ void gemm_kernel<false, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                  int64_t, int, int, int, int, int, float*);
-template __global__ void gemm_kernel<true, true>(const bf16*, int64_t, const bf16*, int64_t, bf16*,
-                                                 int64_t, int, int, int, int, int, float*);
+template __global__ void gemm_kernel<false, false>(const bf16*, int, const bf16*, int, bf16*,
+                                                   int, int, int, int, int, int, int, float*);
+template __global__ void gemm_kernel<false, true>(const bf16*, int, const bf16*, int, bf16*,
+                                                  int, int, int, int, int, int, int, float*);
+template __global__ void gemm_kernel<true, true>(const bf16*, int, const bf16*, int, bf16*,
+                                                 int, int, int, int, int, int, int, float*);
 
 // C = bf16(sum over splits of the fp32 partial tiles [+ C]); one thread per 8 columns.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
@@ -525,17 +565,29 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   int splits = choose_splits(M, N, K);
-  if (workspace == nullptr || (size_t)splits * M * N * sizeof(float) > workspace_bytes) splits = 1;
+  if (workspace == nullptr || (size_t)splits * M * N * sizeof(float) > workspace_bytes ||
+      (int64_t)splits * M * N >= ((int64_t)1 << 31))
+    splits = 1;
+  // one persistent workgroup per compute unit (a workgroup owns a whole CU's LDS)
+  static const int num_cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
   if (splits == 1) {
-    hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles), dim3(NTHREADS), lds_bytes, stream, A, lda,
-                       B, ldb, C, ldc, M, N, K, accumulate, 0, (float*)nullptr);
+    const int grid = tiles < num_cus ? tiles : num_cus;
+    hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
+                       (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr);
     return kr_launch_status();
   }
   int k_per = (K + splits - 1) / splits;
   k_per = (k_per + BK - 1) / BK * BK;
   splits = (K + k_per - 1) / k_per;
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(tiles, splits), dim3(NTHREADS), lds_bytes, stream,
-                     A, lda, B, ldb, C, ldc, M, N, K, 0, k_per, workspace);
+  const int items = tiles * splits;
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(items < num_cus ? items : num_cus), dim3(NTHREADS),
+                     lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream,
@@ -561,7 +613,8 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   if ((M | N | K) % 8 || (lda | ldb | ldc) % 8) return KR_EUNSUPPORTED;
   // chunk offsets inside an operand are kept in 32 bits
   const int64_t a_rows = layout == KR_GEMM_NT ? 64 : M, b_rows = layout == KR_GEMM_TN ? N : 64;
-  if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31) return KR_EUNSUPPORTED;
+  if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31 || ldc >= (int64_t)1 << 31)
+    return KR_EUNSUPPORTED;
   const bf16* a = (const bf16*)A;
   const bf16* b = (const bf16*)B;
   bf16* c = (bf16*)C;
