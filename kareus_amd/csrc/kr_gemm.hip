@@ -541,16 +541,28 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   stg8(dst, o);
 }
 
-// How many ways to cut the contraction so that enough workgroups exist to fill 256 CUs.
-// 1 = no split.  Every split keeps at least 8 K-steps of 64.
+// How many ways to cut the contraction when the output has too few tiles to occupy the GPU.
+// 1 = no split.  Picks the count with the smallest estimated time, in units of one K-step of
+// one workgroup (~1.5 us): rounds of work items over the CUs, each item paying its K-steps plus
+// a fixed prologue/epilogue, plus the traffic of the fp32 partial tiles (written once, read once
+// by the reduce kernel at ~5 TB/s).  More splits than that only add partial-tile traffic.
 inline int choose_splits(int M, int N, int K) {
+  constexpr int kCus = 256, kItemOverhead = 4;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles >= 192) return 1;
-  int splits = (512 + tiles - 1) / tiles;
-  const int max_by_k = K / (8 * BK);
-  if (splits > max_by_k) splits = max_by_k;
-  if (splits > 16) splits = 16;
-  return splits < 2 ? 1 : splits;
+  const int nk = (K + BK - 1) / BK;
+  const double reduce_per_split = (double)M * N * 8.0 / 5.0e12 / 1.5e-6;
+  int best = 1;
+  double best_cost = (double)((tiles + kCus - 1) / kCus) * (nk + kItemOverhead);
+  for (int sp = 2; sp <= 16 && nk / sp >= 8; ++sp) {
+    const int items = tiles * sp, rounds = (items + kCus - 1) / kCus;
+    const double cost = (double)rounds * ((nk + sp - 1) / sp + kItemOverhead) + sp * reduce_per_split;
+    if (cost < best_cost * 0.95) {  // a split must pay for itself clearly
+      best_cost = cost;
+      best = sp;
+    }
+  }
+  return best;
 }
 
 template <bool A_T, bool B_T>
