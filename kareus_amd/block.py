@@ -206,7 +206,9 @@ class LayerStack(torch.nn.Module):
             c.nanobatch_streams = None
             return None
         if c.nanobatch_streams is None:
-            c.nanobatch_streams = [api.new_stream() for _ in range(c.num_nanobatches)]
+            many = getattr(api, "new_streams", None)
+            c.nanobatch_streams = (many(c.num_nanobatches) if many is not None
+                                   else [api.new_stream() for _ in range(c.num_nanobatches)])
         return c.nanobatch_streams
 
     def _get_all_params(self) -> List[torch.nn.Parameter]:

@@ -126,3 +126,17 @@ def test_full_size_properties_config4():
     _, dx_double, _ = _run(_build(dims, 1, 4), x, 2 * go)
     assert torch.equal(dx_double, 2 * dx4)
     assert torch.isfinite(y4).all() and torch.isfinite(dx4).all()
+
+
+def test_nanobatch_streams_do_not_share_a_hardware_queue():
+    """Streams handed to the nanobatches must overlap for real: a short kernel on one finishes
+    while a spinning kernel occupies the other."""
+    from kareus_amd.partitions.streams import _run_concurrently, stream_api
+
+    two = stream_api().new_streams(2)
+    assert len(two) == 2 and two[0] != two[1]
+    assert _run_concurrently(two[0], two[1]) and _run_concurrently(two[1], two[0])
+    four = stream_api().new_streams(4)
+    assert len({s.cuda_stream for s in four}) == 4
+    # one stream cannot overtake itself: the probe must say so
+    assert not _run_concurrently(two[0], two[0])
