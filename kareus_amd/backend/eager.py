@@ -18,13 +18,14 @@ class EagerBackend:
 
     # y = x . W^T, dx = dy . W, dW = dy^T . x   (reference call sites:
     # kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:571-582, 847-859, 898-909)
-    def linear_fwd(self, x: Tensor, w: Tensor) -> Tensor:
+    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
         return x @ w.t()
 
-    def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
+    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
         return dy @ w
 
-    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False) -> Tensor:
+    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False,
+                     split_k: bool = True) -> Tensor:
         dw = dy.t() @ x
         if out is None:
             return dw

@@ -92,14 +92,17 @@ class HipBackend:
 
     # -- GEMM -------------------------------------------------------------------------
     def gemm(self, layout: int, a: Tensor, b: Tensor, m: int, n: int, k: int,
-             out: Tensor = None, accumulate: bool = False) -> Tensor:
+             out: Tensor = None, accumulate: bool = False, split_k: bool = True) -> Tensor:
+        """``split_k=False`` withholds the workspace, so a small output is computed by as many
+        workgroups as it has tiles.  That is the cheaper way in CU-time and the right choice when
+        kernels of other streams are there to use the remaining CUs."""
         self._dev(a, b)
         self._bf16(a, b)
         if a.stride(-1) != 1 or b.stride(-1) != 1:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
             out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-        ws_bytes = self.lib.kr_gemm_workspace_bytes(layout, m, n, k)
+        ws_bytes = self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else 0
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
                                    out.data_ptr(), out.stride(0), int(accumulate),
@@ -107,15 +110,16 @@ class HipBackend:
         self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k})")
         return out
 
-    def linear_fwd(self, x: Tensor, w: Tensor) -> Tensor:
-        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1])
+    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
+        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1], split_k=split_k)
 
-    def linear_dgrad(self, dy: Tensor, w: Tensor) -> Tensor:
-        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1])
+    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
+        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1], split_k=split_k)
 
-    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False) -> Tensor:
+    def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False,
+                     split_k: bool = True) -> Tensor:
         return self.gemm(KR_GEMM_NT, dy, x, dy.shape[1], x.shape[1], dy.shape[0], out=out,
-                         accumulate=accumulate)
+                         accumulate=accumulate, split_k=split_k)
 
     # -- RMSNorm ----------------------------------------------------------------------
     def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:

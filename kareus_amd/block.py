@@ -193,6 +193,9 @@ class LayerStack(torch.nn.Module):
             raise NotImplementedError("one GPU: the tensor-parallel group has a single member")
         n = self.config.num_nanobatches
         streams = self._streams()
+        for layer in self.layers:
+            for op in (layer.linear_qkv, layer.linear_proj, layer.linear_fc1, layer.linear_fc2):
+                op.split_k = streams is None
         self.allreduce_comm_ops = [
             NoOpAllReduce(batch_idx=i, world_size=1, comm_stream=streams[(i - 1) % n] if streams else None)
             for i in range(n)

@@ -61,6 +61,9 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
             torch.nn.init.normal_(weight, mean=0.0, std=0.02)
         self.weight = torch.nn.Parameter(weight)
         self._backend_name = backend
+        # False when kernels of other nanobatch streams fill the GPU next to this layer's GEMMs:
+        # then the contraction is not split, which costs the least CU-time (set by the block driver)
+        self.split_k = True
 
     def op_forward(self, ctx, input_, *, prev_op=None, next_op=None):
         n, k = self.weight.shape
@@ -69,7 +72,7 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         x2d = input_.reshape(-1, k)
         if not x2d.is_contiguous():
             x2d = x2d.contiguous()
-        y = get_backend(self._backend_name).linear_fwd(x2d, self.weight.detach())
+        y = get_backend(self._backend_name).linear_fwd(x2d, self.weight.detach(), split_k=self.split_k)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d)
             ctx.input_requires_grad = True
@@ -82,12 +85,12 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         if not dy.is_contiguous():
             dy = dy.contiguous()
         be = get_backend(self._backend_name)
-        dx = be.linear_dgrad(dy, self.weight.detach())
-        dw = self._weight_grad(be, ctx, dy, x2d) if self.weight.requires_grad else None
+        dx = be.linear_dgrad(dy, self.weight.detach(), split_k=self.split_k)
+        dw = self._weight_grad(be, ctx, dy, x2d, self.split_k) if self.weight.requires_grad else None
         return dx.view(*grad_output.shape[:-1], k), (dw,)
 
     @staticmethod
-    def _weight_grad(be, ctx, dy, x2d):
+    def _weight_grad(be, ctx, dy, x2d, split_k=True):
         """``dW = dy^T . x``.  When the engine attached a ``wgrad_sink`` — one dict shared by
         this layer's contexts of all nanobatches of one backward pass — the first nanobatch to
         get here allocates the gradient and every later one adds its product into the same
@@ -97,17 +100,17 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         does not sum a second time."""
         sink = getattr(ctx, "wgrad_sink", None)
         if sink is None:
-            return be.linear_wgrad(dy, x2d)
+            return be.linear_wgrad(dy, x2d, split_k=split_k)
         api = stream_api()
         here = api.current_stream()
         buf = sink.get("buf")
         if buf is None:
-            buf = sink["buf"] = be.linear_wgrad(dy, x2d)
+            buf = sink["buf"] = be.linear_wgrad(dy, x2d, split_k=split_k)
             ret = buf
         else:
             if here is not None and sink.get("event") is not None:
                 here.wait_event(sink["event"])
-            be.linear_wgrad(dy, x2d, out=buf, accumulate=True)
+            be.linear_wgrad(dy, x2d, out=buf, accumulate=True, split_k=split_k)
             ret = None
         if here is not None:
             ev = api.new_event()

@@ -26,7 +26,13 @@ def _build(dims, layers, nnb, **kw):
     cfg = LayerConfig(hidden_size=dims.hidden, num_attention_heads=dims.nq, num_query_groups=dims.nkv,
                       kv_channels=dims.hd, ffn_hidden_size=dims.ffn, num_layers=layers, num_nanobatches=nnb,
                       backend="hip", **kw)
-    return LayerStack(cfg, device="cuda", seed=1234)
+    model = LayerStack(cfg, device="cuda", seed=1234)
+    # split-K changes the order of the contraction sum; the driver switches it off when nanobatch
+    # streams run side by side, so for bit-exact comparisons across modes it is off everywhere
+    for layer in model.layers:
+        for op in (layer.linear_qkv, layer.linear_proj, layer.linear_fc1, layer.linear_fc2):
+            op.split_k = False
+    return model
 
 
 def _run(model, x, go):
