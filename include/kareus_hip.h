@@ -48,6 +48,12 @@ const char* kr_error_string(int code);
 #define KR_GEMM_NN 1
 #define KR_GEMM_NT 2
 size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K);
+/* Workspace for a GEMM that shares the GPU with kernels of other streams.  The split count of
+ * kr_gemm_workspace_bytes() minimises the GEMM's own latency; with latency_weight < 1 the choice
+ * leans towards the smallest total CU-time instead (0.3 is a good value beside other nanobatch
+ * streams), which never asks for more splits.  kr_gemm_bf16 uses as many splits as the workspace
+ * it is handed holds, at most the latency-optimal count.                                      */
+size_t kr_gemm_workspace_bytes_shared(int layout, int M, int N, int K, float latency_weight);
 int kr_gemm_bf16(int layout, int M, int N, int K,
                  const void* A, int64_t lda, const void* B, int64_t ldb,
                  void* C, int64_t ldc, int accumulate,

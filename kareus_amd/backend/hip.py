@@ -24,6 +24,7 @@ _SIGNATURES = {
     "kr_version": (_c_int, []),
     "kr_error_string": (ctypes.c_char_p, [_c_int]),
     "kr_gemm_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int, _c_int]),
+    "kr_gemm_workspace_bytes_shared": (_c_size_t, [_c_int, _c_int, _c_int, _c_int, _c_float]),
     "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
                               _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p]),
@@ -93,16 +94,18 @@ class HipBackend:
     # -- GEMM -------------------------------------------------------------------------
     def gemm(self, layout: int, a: Tensor, b: Tensor, m: int, n: int, k: int,
              out: Tensor = None, accumulate: bool = False, split_k: bool = True) -> Tensor:
-        """``split_k=False`` withholds the workspace, so a small output is computed by as many
-        workgroups as it has tiles.  That is the cheaper way in CU-time and the right choice when
-        kernels of other streams are there to use the remaining CUs."""
+        """``split_k=True``: the GEMM has the GPU to itself and splits the contraction of a small
+        output for the shortest latency.  ``split_k=False``: kernels of other streams are there
+        to use the CUs a small output leaves idle, so the split count is chosen mostly for the
+        least CU-time (often no split at all)."""
         self._dev(a, b)
         self._bf16(a, b)
         if a.stride(-1) != 1 or b.stride(-1) != 1:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
             out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-        ws_bytes = self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else 0
+        ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
+                    self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
                                    out.data_ptr(), out.stride(0), int(accumulate),

@@ -542,23 +542,35 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }
 
 // How many ways to cut the contraction when the output has too few tiles to occupy the GPU.
-// 1 = no split.  Picks the count with the smallest estimated time, in units of one K-step of
-// one workgroup (~1.5 us): rounds of work items over the CUs, each item paying its K-steps plus
-// a fixed prologue/epilogue, plus the traffic of the fp32 partial tiles (written once, read once
-// by the reduce kernel at ~5 TB/s).  More splits than that only add partial-tile traffic.
-inline int choose_splits(int M, int N, int K) {
+// 1 = no split.  Two estimates, in units of one K-step of one workgroup (~1.5 us):
+//   latency  rounds of work items over the CUs, each item paying its K-steps plus a fixed
+//            prologue/epilogue, plus the traffic of the fp32 partial tiles (written once, read
+//            once by the reduce kernel at ~5 TB/s);
+//   CU-time  the same work summed over the CUs it occupies, per CU of the device.
+// A GEMM that has the GPU to itself wants the smallest latency (latency_weight 1); one that
+// runs beside kernels of other streams, which can use the CUs it leaves idle, should mostly
+// keep its CU-time small (latency_weight ~0.3).
+inline int choose_splits(int M, int N, int K, float latency_weight) {
   constexpr int kCus = 256, kItemOverhead = 4;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   if (tiles >= 192) return 1;
+  const double w = latency_weight < 0.f ? 0.0 : (latency_weight > 1.f ? 1.0 : (double)latency_weight);
   const int nk = (K + BK - 1) / BK;
   const double reduce_per_split = (double)M * N * 8.0 / 5.0e12 / 1.5e-6;
-  int best = 1;
-  double best_cost = (double)((tiles + kCus - 1) / kCus) * (nk + kItemOverhead);
-  for (int sp = 2; sp <= 16 && nk / sp >= 8; ++sp) {
+  auto cost = [&](int sp) {
     const int items = tiles * sp, rounds = (items + kCus - 1) / kCus;
-    const double cost = (double)rounds * ((nk + sp - 1) / sp + kItemOverhead) + sp * reduce_per_split;
-    if (cost < best_cost * 0.95) {  // a split must pay for itself clearly
-      best_cost = cost;
+    const int per_item = (nk + sp - 1) / sp + kItemOverhead;
+    const double reduce = sp > 1 ? sp * reduce_per_split : 0.0;
+    const double latency = (double)rounds * per_item + reduce;
+    const double cu_time = (double)items * per_item / kCus + reduce;
+    return w * latency + (1.0 - w) * cu_time;
+  };
+  int best = 1;
+  double best_cost = cost(1);
+  for (int sp = 2; sp <= 16 && nk / sp >= 8; ++sp) {
+    const double c = cost(sp);
+    if (c < best_cost * 0.95) {  // a split must pay for itself clearly
+      best_cost = c;
       best = sp;
     }
   }
@@ -576,10 +588,16 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  int splits = choose_splits(M, N, K);
-  if (workspace == nullptr || (size_t)splits * M * N * sizeof(float) > workspace_bytes ||
-      (int64_t)splits * M * N >= ((int64_t)1 << 31))
+  // the latency-optimal count, capped by what the caller's workspace holds (a caller that wants
+  // fewer splits says so by passing the smaller workspace kr_gemm_workspace_bytes_shared sizes)
+  int splits = choose_splits(M, N, K, 1.f);
+  const size_t one = (size_t)M * N * sizeof(float);
+  if (workspace == nullptr) {
     splits = 1;
+  } else if ((size_t)splits * one > workspace_bytes) {
+    splits = (int)(workspace_bytes / one);
+  }
+  if (splits < 2 || (int64_t)splits * M * N >= ((int64_t)1 << 31)) splits = 1;
   // one persistent workgroup per compute unit (a workgroup owns a whole CU's LDS)
   static const int num_cus = [] {
     int dev = 0, n = 0;
@@ -612,7 +630,16 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
 extern "C" size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K) {
   (void)layout;
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const int splits = choose_splits(M, N, K);
+  const int splits = choose_splits(M, N, K, 1.f);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
+extern "C" size_t kr_gemm_workspace_bytes_shared(int layout, int M, int N, int K, float latency_weight) {
+  (void)layout;
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int splits = choose_splits(M, N, K, latency_weight);
+  const int cap = choose_splits(M, N, K, 1.f);
+  if (splits > cap) splits = cap;
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
