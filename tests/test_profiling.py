@@ -197,3 +197,115 @@ def test_partitions_on_the_gpu_match_the_host_engine(key):
         torch.cuda.synchronize()
         a, b = dev.executor.output(out).float().cpu(), host.executor.output(out)
         assert (a - b).abs().max() <= 2e-2 * b.abs().max(), (key, w)   # bf16 vs fp32: 2e-2 max-relative
+
+
+# ---- eval logs -> solver input ---------------------------------------------------------------------
+from kareus_amd.profiling.profile_csv import (  # noqa: E402
+    candidate_points, generate_profile_csv, layers_per_stage, pareto_optimal, read_eval_log,
+)
+from kareus_amd.scheduler.parser import _parse_config_string  # noqa: E402
+
+
+def test_pareto_filter_uses_effective_energy():
+    pts = [("a", (1.0, 100.0)), ("b", (2.0, 90.0)), ("c", (3.0, 95.0)), ("d", (1.0, 120.0)), ("e", (4.0, 150.0))]
+    # no idle power: keep strictly improving energy along increasing time
+    assert [k for k, _ in pareto_optimal(pts, 0.0)] == ["a", "b"]
+    # 20 W idle: effective energies 80, 50, 35, 100, 70 -> c now improves on b
+    assert [k for k, _ in pareto_optimal(pts, 20.0)] == ["a", "b", "c"]
+    # an improvement below the tolerance does not count
+    assert [k for k, _ in pareto_optimal([("a", (1.0, 10.0)), ("b", (2.0, 10.0 - 5e-5))], 0.0)] == ["a"]
+    assert pareto_optimal([], 85.0) == []
+
+
+def test_layers_per_stage():
+    assert layers_per_stage(32, 1) == [32]
+    assert layers_per_stage(32, 2, 15, 17) == [15, 17]
+    assert layers_per_stage(32, 2, 20, 20) == [20, 12]            # inconsistent pair: last is what is left
+    assert layers_per_stage(28, 4, 6, 6) == [6, 8, 8, 6]
+    assert layers_per_stage(29, 5, 5, 5) == [5, 7, 6, 6, 5]       # remainder goes to the earlier middle stages
+    with pytest.warns(UserWarning):
+        assert layers_per_stage(8, 3, 6, 6) == [6, 0, 2]
+    with pytest.raises(ValueError):
+        layers_per_stage(8, 0)
+
+
+def _write_logs(tmp_path, nested=False):
+    rows = {
+        "fwd_attn": [(1500, "norm_0", 1.0, 10.0), (1500, "attn_0", 0.9, 10.5), (2100, "norm_0", 0.7, 12.0)],
+        "fwd_mlp": [(1500, "linear_0", 2.0, 20.0), (2100, "linear_0", 1.5, 25.0)],
+        "bwd_attn": [(1500, "linear_1", 3.0, 30.0), (2100, "linear_1", 2.0, 36.0)],
+        "bwd_mlp": [(1500, "none", 4.0, 40.0), (2100, "none", 3.0, 50.0), (900, "none", 9.0, 30.0)],
+    }
+    for key, items in rows.items():
+        path = tmp_path / key / "eval_results.jsonl" if nested else tmp_path / f"{key}.jsonl"
+        path.parent.mkdir(parents=True, exist_ok=True)
+        with open(path, "w") as f:
+            for freq, start, t, e in items:
+                f.write(json.dumps(build_eval_record({"freq": freq, "sm": 16, "block": 1024, "overlap": (start, "none")}, t, e)) + "\n")
+            f.write("garbage\n")
+            f.write(json.dumps({"freq": 1500, "time_s": 1.0}) + "\n")                       # fields missing
+            f.write(json.dumps(build_eval_record({"freq": 1500, "sm": 8, "block": 1024, "overlap": ("x", "none")}, 1.0, None)) + "\n")
+    return rows
+
+
+def test_candidate_table_closed_form(tmp_path):
+    _write_logs(tmp_path)
+    logs = {k: read_eval_log(str(tmp_path / f"{k}.jsonl")) for k in ("fwd_attn", "fwd_mlp", "bwd_attn", "bwd_mlp")}
+    assert sorted(logs["fwd_attn"]) == [1500, 2100] and len(logs["fwd_attn"][1500]) == 2     # bad rows dropped
+    extra = {1500: {"forward-embedding": (0.5, 5.0), "forward-output": (0.25, 2.5), "loss-func": (0.125, 1.25),
+                    "backward-embedding": (1.0, 10.0), "backward-output": (2.0, 20.0)}}
+    fwd, bwd = candidate_points(logs, [3, 5], nanobatches=2, use_activation_checkpointing=True,
+                                scale_time_energy=False, nonpartition=extra)
+    # frequency 900 exists for one partition only and is left out
+    assert {k[0] for k, _ in fwd[0]} == {1500, 2100} and len(fwd[0]) == 3 and len(bwd[1]) == 3
+    f0 = dict(fwd[0])[(1500, ("norm_0", "none", 16, 1024), ("linear_0", "none", 16, 1024))]
+    assert f0 == (pytest.approx((1.0 + 2.0) * 3 * 2 + 0.5), pytest.approx((10.0 + 20.0) * 3 * 2 + 5.0))
+    f1 = dict(fwd[1])[(1500, ("norm_0", "none", 16, 1024), ("linear_0", "none", 16, 1024))]
+    assert f1 == (pytest.approx(3.0 * 5 * 2 + 0.25 + 0.125), pytest.approx(30.0 * 5 * 2 + 2.5 + 1.25))
+    key = (1500, ("attn_0", "none", 16, 1024), ("linear_0", "none", 16, 1024),
+           ("linear_1", "none", 16, 1024), ("none", "none", 16, 1024))
+    assert dict(bwd[0])[key] == (pytest.approx((0.9 + 2 + 3 + 4) * 3 * 2 + 2 * 1.0), pytest.approx((10.5 + 20 + 30 + 40) * 6 + 20.0))
+    assert dict(bwd[1])[key] == (pytest.approx(9.9 * 10 + 2.0), pytest.approx(100.5 * 10 + 20.0))
+    # 2100 MHz has no non-partition figures: zeros; scaling multiplies both by 1.15
+    fwd_s, _ = candidate_points(logs, [1], nanobatches=4, use_activation_checkpointing=False, scale_time_energy=True)
+    k2 = (2100, ("norm_0", "none", 16, 1024), ("linear_0", "none", 16, 1024))
+    assert dict(fwd_s[0])[k2] == (pytest.approx(2.2 * 1.15 * 4), pytest.approx(37.0 * 1.15 * 4))
+    with pytest.raises(RuntimeError, match="No overlapping frequencies"):
+        candidate_points(dict(logs, fwd_mlp={900: logs["bwd_mlp"][900]}), [1])
+
+
+@pytest.mark.parametrize("recompute", [True, False])
+def test_profile_csv_rows_feed_the_schedule_parser(tmp_path, recompute):
+    _write_logs(tmp_path, nested=True)
+    out = str(tmp_path / "profile.csv")
+    kept = generate_profile_csv(str(tmp_path), out, num_layers=8, pipeline_parallel_size=2,
+                                num_layers_in_first_pipeline_stage=4, num_layers_in_last_pipeline_stage=4,
+                                gpu_type="A100", use_activation_checkpointing=recompute, scale_time_energy=False)
+    lines = open(out).read().strip().splitlines()
+    header = lines[0].split(",")
+    assert header == (["stage", "instruction", "frequency", "recompute_attention_configs", "recompute_mlp_configs",
+                       "attention_configs", "mlp_configs", "time", "energy"] if recompute else
+                      ["stage", "instruction", "frequency", "attention_configs", "mlp_configs", "time", "energy"])
+    assert len(lines) - 1 == kept["forward"] + kept["backward"] and kept["forward"] >= 2 and kept["backward"] >= 2
+    for line in lines[1:]:
+        cells = line.split(",")
+        assert len(cells) == len(header) and cells[1] in ("forward", "backward") and cells[0] in ("0", "1")
+        cfg_cells = cells[3:-2]
+        if recompute and cells[1] == "forward":
+            assert cfg_cells[:2] == ["", ""]
+            cfg_cells = cfg_cells[2:]
+        for c in cfg_cells:                                   # every configuration is a schedule-file field
+            parsed = _parse_config_string(c)
+            assert parsed.resource_shape == (16, 1024) and parsed.overlap_window[1] in ("none", -1)
+        assert float(cells[-2]) > 0 and float(cells[-1]) > 0
+    # Pareto per stage and direction: times strictly increase, effective energy strictly decreases
+    for stage in ("0", "1"):
+        for inst in ("forward", "backward"):
+            pts = [(float(l.split(",")[-2]), float(l.split(",")[-1])) for l in lines[1:]
+                   if l.split(",")[0] == stage and l.split(",")[1] == inst]
+            eff = [e - 85.0 * t for t, e in pts]
+            assert pts == sorted(pts) and all(b < a for a, b in zip(eff, eff[1:]))
+    with pytest.raises(ValueError, match="Unknown GPU type"):
+        generate_profile_csv(str(tmp_path), out, 8, gpu_type="H100")
+    with pytest.raises(FileNotFoundError):
+        generate_profile_csv(str(tmp_path / "missing"), out, 8)
