@@ -62,16 +62,19 @@ int kr_gemm_bf16(int layout, int M, int N, int K,
 /* ---- RMSNorm ---------------------------------------------------------------------------
  * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd
  * (kareus/transformer_engine/pytorch/ops/basic/rmsnorm.py:210-219, 256-263).
- * x, y, dy, dx: [rows, cols] bf16 contiguous; gamma, dgamma: [cols] bf16; rstd: [rows] fp32.
+ * x, dy: [rows, cols] bf16 with row strides x_ld, dy_ld (elements, multiples of 8, >= cols; a
+ * nanobatch that is one sequence of a [seq, batch, hidden] tensor is such a matrix and needs no
+ * copy); y, dx: [rows, cols] bf16 contiguous; gamma, dgamma: [cols] bf16; rstd: [rows] fp32.
  * cols must be a multiple of 8 and at most 8192.
  * fwd: rstd = rsqrt(mean(x^2) + eps), y = (x * rstd) * gamma.
  * bwd: dx = rstd * (g - xhat * mean(g * xhat)), g = gamma * dy, xhat = x * rstd;
  *      dgamma = sum over rows of dy * xhat.  workspace: kr_rmsnorm_bwd_workspace_bytes().  */
 int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd,
-                   int rows, int cols, float eps, void* stream);
+                   int rows, int cols, int64_t x_ld, float eps, void* stream);
 size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols);
 int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
-                   void* dx, void* dgamma, void* workspace, int rows, int cols, void* stream);
+                   void* dx, void* dgamma, void* workspace, int rows, int cols,
+                   int64_t dy_ld, int64_t x_ld, void* stream);
 
 /* ---- Rotary position embedding ---------------------------------------------------------
  * Replaces fused_rotary_positional_embedding.forward / backward (Apex), called from
@@ -106,6 +109,10 @@ int kr_swiglu_bwd(const void* dy, const void* x, void* dx, int64_t rows, int F, 
  * ResidualForkOp (kareus/megatron/core/extensions/ops/residual_fork.py:104-106).
  * out may alias a or b.                                                                    */
 int kr_add(const void* a, const void* b, void* out, int64_t n, void* stream);
+/* The same sum over [rows, cols] matrices with row strides lda, ldb, ldo (elements, multiples of
+ * 8, >= cols; cols a multiple of 8): lets the residual stream stay a strided nanobatch slice.   */
+int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
+                int64_t rows, int cols, void* stream);
 
 /* ---- Causal grouped-query attention ----------------------------------------------------
  * Replaces flash_attn_2_cuda.fwd / bwd as called from

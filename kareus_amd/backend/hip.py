@@ -27,14 +27,15 @@ _SIGNATURES = {
     "kr_gemm_workspace_bytes_shared": (_c_size_t, [_c_int, _c_int, _c_int, _c_int, _c_float]),
     "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
                               _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
-    "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p]),
+    "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
-    "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_void_p]),
+    "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
                 + [_c_int, _c_int, _c_int, _c_void_p]),
     "kr_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_swiglu_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_add": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
+    "kr_add_rows": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_i64, _c_int, _c_void_p]),
     "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_void_p]),
     "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
     "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_void_p]),
@@ -125,26 +126,37 @@ class HipBackend:
                          accumulate=accumulate, split_k=split_k)
 
     # -- RMSNorm ----------------------------------------------------------------------
+    @staticmethod
+    def _rows(t: Tensor) -> Tensor:
+        """A [rows, cols] matrix the kernels can address with one row stride: unit column
+        stride, row stride a multiple of 8 elements; anything else is copied."""
+        if t.dim() == 2 and t.stride(1) == 1 and t.stride(0) % 8 == 0 and t.stride(0) >= t.shape[1]:
+            return t
+        return t.contiguous()
+
     def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
         self._dev(x, gamma)
         self._bf16(x, gamma)
+        x = self._rows(x)
         rows, cols = x.shape
-        y = torch.empty_like(x)
+        y = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
         rc = self.lib.kr_rmsnorm_fwd(x.data_ptr(), gamma.data_ptr(), y.data_ptr(), rstd.data_ptr(),
-                                     rows, cols, eps, self._stream())
+                                     rows, cols, x.stride(0), eps, self._stream())
         self._check(rc, "kr_rmsnorm_fwd")
         return y, rstd
 
     def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor) -> Tuple[Tensor, Tensor]:
         self._dev(dy, x, rstd, gamma)
         self._bf16(dy, x, gamma)
+        x, dy = self._rows(x), self._rows(dy)
         rows, cols = x.shape
-        dx = torch.empty_like(x)
+        dx = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
         dgamma = torch.empty_like(gamma)
         ws = torch.empty(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), dtype=torch.uint8, device=x.device)
         rc = self.lib.kr_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-                                     dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols, self._stream())
+                                     dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols,
+                                     dy.stride(0), x.stride(0), self._stream())
         self._check(rc, "kr_rmsnorm_bwd")
         return dx, dgamma
 
@@ -217,13 +229,26 @@ class HipBackend:
         self._bf16(a, b)
         if a.shape != b.shape:
             raise RuntimeError(f"add: shapes differ, {tuple(a.shape)} vs {tuple(b.shape)}")
-        if not a.is_contiguous():
-            a = a.contiguous()
-        if not b.is_contiguous():
-            b = b.contiguous()
-        out = torch.empty_like(a)
-        self._check(self.lib.kr_add(a.data_ptr(), b.data_ptr(), out.data_ptr(), a.numel(), self._stream()), "kr_add")
+        if a.is_contiguous() and b.is_contiguous():
+            out = torch.empty_like(a)
+            self._check(self.lib.kr_add(a.data_ptr(), b.data_ptr(), out.data_ptr(), a.numel(), self._stream()),
+                        "kr_add")
+            return out
+        # a strided nanobatch slice (one sequence of a [seq, batch, hidden] tensor) is a matrix
+        # with a long row stride: add it in place, do not copy it first
+        cols = a.shape[-1]
+        a2, b2 = self._rows(self._matrix(a, cols)), self._rows(self._matrix(b, cols))
+        out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+        self._check(self.lib.kr_add_rows(a2.data_ptr(), a2.stride(0), b2.data_ptr(), b2.stride(0),
+                                         out.data_ptr(), cols, a2.shape[0], cols, self._stream()), "kr_add_rows")
         return out
+
+    @staticmethod
+    def _matrix(t: Tensor, cols: int) -> Tensor:
+        try:
+            return t.view(-1, cols)
+        except RuntimeError:
+            return t.reshape(-1, cols)
 
     # -- attention ----------------------------------------------------------------------
     @staticmethod

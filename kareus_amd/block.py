@@ -81,6 +81,29 @@ class LayerConfig:
         return (self.num_attention_heads + 2 * self.num_query_groups) * self.kv_channels
 
 
+class _SplitNanobatches(torch.autograd.Function):
+    """``[s, b, h] -> n x [s, b/n, h]`` along the batch dimension (the reference slices with
+    ``hidden_states[:, i*nb:(i+1)*nb]``, transformer_block.py:405-527).
+
+    A nanobatch of one sequence is a matrix with row stride ``b*h``; every kernel that touches it
+    takes a row stride, so it stays a view.  Wider nanobatches cannot be addressed with a single
+    row stride and are copied into dense tensors once.  Backward writes the n gradients into one
+    ``[s, b, h]`` tensor (one concatenation) instead of autograd's zero-fill + copy + add per
+    slice."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, n):
+        nb = hidden_states.shape[1] // n
+        parts = [hidden_states[:, i * nb:(i + 1) * nb] for i in range(n)]
+        if nb > 1 or hidden_states.stride(2) != 1 or hidden_states.stride(0) % 8:
+            parts = [p.contiguous() for p in parts]
+        return tuple(parts)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        return torch.cat(grads, dim=1), None
+
+
 class DecoderLayer(torch.nn.Module):
     """Holds one layer's operators and states their execution order; it has no
     ``forward`` of its own — the partition engine runs the operators."""
@@ -243,10 +266,7 @@ class LayerStack(torch.nn.Module):
         if rotary_pos_emb is None:
             rotary_pos_emb = self.rotary_pos_emb(s, device=hidden_states.device)
 
-        nb = b // n
-        # Each nanobatch becomes a contiguous [s, b/n, h] tensor of its own, so every
-        # operator sees dense rows.
-        hs = [hidden_states[:, i * nb:(i + 1) * nb].contiguous() for i in range(n)]
+        hs = _SplitNanobatches.apply(hidden_states, n) if n > 1 else (hidden_states,)
         params = self._get_all_params()
         outs = TransformerBlockAutogradFunction.apply(
             *hs, rotary_pos_emb, None,

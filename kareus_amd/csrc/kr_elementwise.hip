@@ -25,6 +25,22 @@ __global__ __launch_bounds__(kThreads) void add_kernel(const bf16* a, const bf16
   }
 }
 
+// row-strided operands: element (r, c) of a at a[r*lda + c]; cols a multiple of 8
+__global__ __launch_bounds__(kThreads) void add_rows_kernel(const bf16* a, int64_t lda, const bf16* b,
+                                                            int64_t ldb, bf16* out, int64_t ldo,
+                                                            int64_t rows, int cols) {
+  const int nv = cols / 8;
+  const int64_t total = rows * nv, stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / nv;
+    const int c = (int)(i - r * nv) * 8;
+    bf16x8 x = ldg8(a + r * lda + c), y = ldg8(b + r * ldb + c), o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)x[e] + (float)y[e]);
+    stg8(out + r * ldo + c, o);
+  }
+}
+
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 // x [rows, 2F] -> y [rows, F]; one thread per 8 output columns.
@@ -134,6 +150,18 @@ extern "C" int kr_add(const void* a, const void* b, void* out, int64_t n, void* 
   const int64_t nvec = n / 8;
   hipLaunchKernelGGL(add_kernel, dim3(grid_for(nvec, kThreads)), dim3(kThreads), 0,
                      (hipStream_t)stream, (const bf16*)a, (const bf16*)b, (bf16*)out, nvec, n);
+  return kr_launch_status();
+}
+
+extern "C" int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* out,
+                           int64_t ldo, int64_t rows, int cols, void* stream) {
+  if (!a || !b || !out || rows <= 0 || cols <= 0 || lda < cols || ldb < cols || ldo < cols)
+    return KR_EINVAL;
+  if (cols % 8 || lda % 8 || ldb % 8 || ldo % 8) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(a) || !kr_aligned16(b) || !kr_aligned16(out)) return KR_EINVAL;
+  hipLaunchKernelGGL(add_rows_kernel, dim3(grid_for(rows * (cols / 8), kThreads)), dim3(kThreads), 0,
+                     (hipStream_t)stream, (const bf16*)a, lda, (const bf16*)b, ldb, (bf16*)out, ldo,
+                     rows, cols);
   return kr_launch_status();
 }
 

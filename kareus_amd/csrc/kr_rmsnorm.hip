@@ -20,7 +20,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
                                                                const bf16* __restrict__ gamma,
                                                                bf16* __restrict__ y,
                                                                float* __restrict__ rstd, int rows,
-                                                               int cols, float eps) {
+                                                               int cols, int64_t x_ld, float eps) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nvec = cols / 8;
   const float inv_cols = 1.0f / (float)cols;
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
     g[c] = v < nvec ? ldg8(gamma + v * 8) : zero8();
   }
   for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
-    const bf16* xr = x + (int64_t)row * cols;
+    const bf16* xr = x + (int64_t)row * x_ld;
     bf16x8 xv[NCHUNK];
     float ss = 0.f;
 #pragma unroll
@@ -67,7 +67,7 @@ template <int NCHUNK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
     const bf16* __restrict__ gamma, bf16* __restrict__ dx, float* __restrict__ partial, int rows,
-    int cols) {
+    int cols, int64_t dy_ld, int64_t x_ld) {
   __shared__ float red[kWaves - 1][64 * 8];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nvec = cols / 8;
@@ -82,8 +82,8 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     for (int e = 0; e < 8; ++e) dg[c][e] = 0.f;
   }
   for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
-    const bf16* xr = x + (int64_t)row * cols;
-    const bf16* dr = dy + (int64_t)row * cols;
+    const bf16* xr = x + (int64_t)row * x_ld;
+    const bf16* dr = dy + (int64_t)row * dy_ld;
     const float rs = rstd[row];
     bf16x8 xv[NCHUNK], dv[NCHUNK];
 #pragma unroll
@@ -181,16 +181,16 @@ inline int chunks_for(int cols) { return (cols / 8 + 63) / 64; }
   }
 
 extern "C" int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd, int rows,
-                              int cols, float eps, void* stream) {
-  if (!x || !gamma || !y || !rstd || rows <= 0 || cols <= 0) return KR_EINVAL;
-  if (cols % 8 || cols > 8192) return KR_EUNSUPPORTED;
+                              int cols, int64_t x_ld, float eps, void* stream) {
+  if (!x || !gamma || !y || !rstd || rows <= 0 || cols <= 0 || x_ld < cols) return KR_EINVAL;
+  if (cols % 8 || x_ld % 8 || cols > 8192) return KR_EUNSUPPORTED;
   if (!kr_aligned16(x) || !kr_aligned16(y) || !kr_aligned16(gamma)) return KR_EINVAL;
   int blocks = (rows + kWaves - 1) / kWaves;
   if (blocks > 256 * 8) blocks = 256 * 8;
   const int nc = chunks_for(cols);
   KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_fwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
                                            (hipStream_t)stream, (const bf16*)x, (const bf16*)gamma,
-                                           (bf16*)y, rstd, rows, cols, eps));
+                                           (bf16*)y, rstd, rows, cols, x_ld, eps));
   return kr_launch_status();
 }
 
@@ -201,10 +201,11 @@ extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
 
 extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
                               void* dx, void* dgamma, void* workspace, int rows, int cols,
-                              void* stream) {
-  if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0)
+                              int64_t dy_ld, int64_t x_ld, void* stream) {
+  if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0 ||
+      dy_ld < cols || x_ld < cols)
     return KR_EINVAL;
-  if (cols % 8 || cols > 8192) return KR_EUNSUPPORTED;
+  if (cols % 8 || dy_ld % 8 || x_ld % 8 || cols > 8192) return KR_EUNSUPPORTED;
   if (!kr_aligned16(x) || !kr_aligned16(dy) || !kr_aligned16(dx) || !kr_aligned16(gamma) ||
       !kr_aligned16(workspace))
     return KR_EINVAL;
@@ -213,7 +214,7 @@ extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, 
   KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_bwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
                                            (hipStream_t)stream, (const bf16*)dy, (const bf16*)x,
                                            rstd, (const bf16*)gamma, (bf16*)dx, (float*)workspace,
-                                           rows, cols));
+                                           rows, cols, dy_ld, x_ld));
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 63) / 64), dim3(256), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);

@@ -69,9 +69,7 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         n, k = self.weight.shape
         if input_.shape[-1] != k:
             raise ValueError(f"linear with in_features={k} got input of shape {tuple(input_.shape)}")
-        x2d = input_.reshape(-1, k)
-        if not x2d.is_contiguous():
-            x2d = x2d.contiguous()
+        x2d = self._rows(input_.reshape(-1, k))
         y = get_backend(self._backend_name).linear_fwd(x2d, self.weight.detach(), split_k=self.split_k)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d)
@@ -81,13 +79,20 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
     def op_backward(self, ctx, grad_output):
         (x2d,) = ctx.saved_tensors
         n, k = self.weight.shape
-        dy = grad_output.reshape(-1, n)
-        if not dy.is_contiguous():
-            dy = dy.contiguous()
+        dy = self._rows(grad_output.reshape(-1, n))
         be = get_backend(self._backend_name)
         dx = be.linear_dgrad(dy, self.weight.detach(), split_k=self.split_k)
         dw = self._weight_grad(be, ctx, dy, x2d, self.split_k) if self.weight.requires_grad else None
         return dx.view(*grad_output.shape[:-1], k), (dw,)
+
+    @staticmethod
+    def _rows(t2d):
+        """GEMM operands may be row-strided (a one-sequence nanobatch slice of a
+        [seq, batch, hidden] tensor is); the reference copies such slices
+        (basic_linear.py:565-569), here only layouts a leading dimension cannot express are."""
+        if t2d.stride(1) == 1 and t2d.stride(0) % 8 == 0 and t2d.stride(0) >= t2d.shape[1]:
+            return t2d
+        return t2d.contiguous()
 
     @staticmethod
     def _weight_grad(be, ctx, dy, x2d, split_k=True):

@@ -25,9 +25,7 @@ class RMSNorm(BasicOperation):
         h = self.weight.shape[0]
         if input_.shape[-1] != h:
             raise ValueError(f"RMSNorm over {h} features got input of shape {tuple(input_.shape)}")
-        x2d = input_.reshape(-1, h)
-        if not x2d.is_contiguous():
-            x2d = x2d.contiguous()
+        x2d = input_.reshape(-1, h)   # a view when the rows have one stride, else a dense copy
         y, rstd = get_backend(self._backend_name).rmsnorm_fwd(x2d, self.weight.detach(), self.eps)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d, rstd)
@@ -36,8 +34,6 @@ class RMSNorm(BasicOperation):
     def op_backward(self, ctx, grad_output):
         x2d, rstd = ctx.saved_tensors
         dy = grad_output.reshape(x2d.shape)
-        if not dy.is_contiguous():
-            dy = dy.contiguous()
         dx, dgamma = get_backend(self._backend_name).rmsnorm_bwd(dy, x2d, rstd, self.weight.detach())
         return dx.view(grad_output.shape), (dgamma,)
 

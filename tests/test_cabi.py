@@ -36,7 +36,12 @@ def test_argument_checks_run_without_a_device():
     # invalid arguments are rejected before anything touches the GPU
     assert lib.kr_add(None, None, None, 8, None) == -1
     assert lib.kr_swiglu_fwd(16, 16, 4, 12, None) == -2          # F not a multiple of 8
-    assert lib.kr_rmsnorm_fwd(16, 16, 16, 16, 4, 8200, 1e-5, None) == -2
+    assert lib.kr_rmsnorm_fwd(16, 16, 16, 16, 4, 8200, 8200, 1e-5, None) == -2    # wider than 8192
+    assert lib.kr_rmsnorm_fwd(16, 16, 16, 16, 4, 64, 32, 1e-5, None) == -1        # row stride < width
+    assert lib.kr_rmsnorm_bwd(16, 16, 16, 16, 16, 16, 16, 4, 64, 64, 68, None) == -2  # stride not x8
+    assert lib.kr_add_rows(16, 64, 16, 64, 16, 32, 4, 64, None) == -1             # output stride < width
+    assert lib.kr_add_rows(16, 64, 16, 64, 16, 64, 4, 60, None) == -2             # width not x8
+    assert lib.kr_gemm_workspace_bytes_shared(2, 1536, 4096, 4096, 0.3) <= lib.kr_gemm_workspace_bytes(2, 1536, 4096, 4096)
     assert lib.kr_gemm_bf16(0, 8, 8, 7, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -2
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1
     assert lib.kr_gemm_bf16(0, 8, 8, 8, 16, 8, 16, 8, 18, 8, 0, None, 0, None) == -1   # misaligned C

@@ -92,6 +92,31 @@ def test_rmsnorm(be, rows, cols):
     assert (yc.float() - 3.0 / math.sqrt(9.0 + 1e-5)).abs().max() < 1e-2
 
 
+def test_row_strided_nanobatch_slices_need_no_copy(be):
+    """One sequence out of a [seq, batch, hidden] tensor is a matrix with row stride batch*hidden:
+    RMSNorm (forward and backward) and the residual add must read it in place and give exactly
+    what they give on a dense copy."""
+    seq, batch, hidden = 384, 4, 1024
+    full, gfull = rnd(seq, batch, hidden, seed=30), rnd(seq, batch, hidden, seed=31)
+    g = (1 + 0.1 * torch.randn(hidden, generator=torch.Generator().manual_seed(32))).to(DEV, torch.bfloat16)
+    xs, dys = full[:, 2, :], gfull[:, 1, :]
+    assert not xs.is_contiguous() and xs.stride(0) == batch * hidden
+    y, rstd = be.rmsnorm_fwd(xs, g, 1e-5)
+    yd, rstdd = be.rmsnorm_fwd(xs.contiguous(), g, 1e-5)
+    assert torch.equal(y, yd) and torch.equal(rstd, rstdd) and y.is_contiguous()
+    dx, dg = be.rmsnorm_bwd(dys, xs, rstd, g)
+    dxd, dgd = be.rmsnorm_bwd(dys.contiguous(), xs.contiguous(), rstd, g)
+    assert torch.equal(dx, dxd) and torch.equal(dg, dgd)
+    dense = rnd(seq, 1, hidden, seed=33)
+    out = be.add(full[:, 2:3, :], dense)                      # strided + dense, 3-D as the engine passes them
+    assert out.shape == dense.shape and out.is_contiguous()
+    assert torch.equal(out, full[:, 2:3, :] + dense)
+    assert torch.equal(be.add(dense, gfull[:, 0:1, :]), dense + gfull[:, 0:1, :])
+    assert torch.equal(be.add(full[:, 0:1, :], gfull[:, 3:4, :]), full[:, 0:1, :] + gfull[:, 3:4, :])
+    wide = be.add(full[:, 0:2, :], gfull[:, 2:4, :])           # two sequences: no single row stride, copied
+    assert torch.equal(wide, full[:, 0:2, :] + gfull[:, 2:4, :])
+
+
 # ------------------------------------------------------------------ GEMM
 SHAPES = [(256, 256, 64), (512, 768, 512), (264, 520, 200), (1024, 2752, 512), (2048, 512, 1376),
           (8, 8, 8), (4096, 640, 384), (40, 1536, 4096)]
