@@ -29,7 +29,7 @@ constexpr int LDKT = HD + 8;  // K tile row length in LDS (elements)
 constexpr int LDVT = HD + 32; // V tile row length in LDS (elements)
 constexpr int K_ELEMS = BKV * LDKT;
 constexpr int V_ELEMS = BKV * LDVT;
-constexpr int FWD_THREADS = 256;
+constexpr int FWD_THREADS = 256;   // threads of one half of a workgroup (4 waves x 32 queries)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr int kXcds = 8;
@@ -79,7 +79,17 @@ __device__ __forceinline__ bf16x8 read_vt_frag(const bf16* vt, int key0, int d0,
   return u.v;
 }
 
-__global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
+// A workgroup owns 128 queries of one (batch, head).  Its eight waves form two halves of four;
+// both halves hold the same queries (wave w and wave w+4 the same 32 rows) and walk the key
+// tiles alternately — half 0 the even 64-key tiles, half 1 the odd ones — each with its own
+// double-buffered K/V staging area and its own running (max, sum, output).  At the end half 1
+// hands its state to half 0 through LDS and half 0 merges the two softmax partials.  The longest
+// rows of a causal problem thus take half as many steps, which is what bounds the kernel when
+// there are only as many workgroups as CUs (a nanobatch of one sequence).  With plenty of
+// workgroups (HALVES = 1: four waves, every key tile, two workgroups per CU) the coupling of the
+// halves at every barrier costs more than the shorter tail gains, so the host picks per launch.
+template <int HALVES>
+__global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void attn_fwd_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
     int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
@@ -88,7 +98,9 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   constexpr int STAGE = K_ELEMS + V_ELEMS;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int half = HALVES == 1 ? 0 : (int)(threadIdx.x >> 8);  // which key tiles this wave walks
+  const int tid = threadIdx.x & (FWD_THREADS - 1);   // thread index inside the half
+  const int lane = tid & 63, wave = tid >> 6, h = lane >> 5;
   const int nqt = s / BQ;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qt = nqt - 1 - (lid % nqt);  // longest rows first inside each (batch, head)
@@ -115,18 +127,19 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
     for (int e = 0; e < 16; ++e) oacc[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int ntiles = (q0 + BQ) / BKV;
+  const int nsteps = (q0 + BQ) / (HALVES * BKV);  // key tiles per half (the tile count is even)
+  bf16* const area = smem + half * 2 * STAGE;  // this half's two staging buffers
   KVStager st;
-  st.load(kb, vb, k_ss, v_ss, 0, tid);
-  st.store(smem, smem + K_ELEMS, tid);
+  st.load(kb, vb, k_ss, v_ss, half * BKV, tid);
+  st.store(area, area + K_ELEMS, tid);
   __syncthreads();
 
-  for (int j = 0; j < ntiles; ++j) {
+  for (int j = 0; j < nsteps; ++j) {
     const int cur = j & 1;
-    if (j + 1 < ntiles) st.load(kb, vb, k_ss, v_ss, (j + 1) * BKV, tid);
-    const int key0 = j * BKV;
+    if (j + 1 < nsteps) st.load(kb, vb, k_ss, v_ss, (HALVES * (j + 1) + half) * BKV, tid);
+    const int key0 = (HALVES * j + half) * BKV;
     if (key0 <= qw0 + 31) {  // wave-uniform: this tile has keys some of the wave's rows may see
-      const bf16* kt = smem + cur * STAGE;
+      const bf16* kt = area + cur * STAGE;
       const bf16* vt = kt + K_ELEMS;
       f32x16 sacc[2];
 #pragma unroll
@@ -184,8 +197,35 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
             oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[t][k2], oacc[dt], 0, 0, 0);
           }
     }
-    if (j + 1 < ntiles) st.store(smem + (cur ^ 1) * STAGE, smem + (cur ^ 1) * STAGE + K_ELEMS, tid);
+    if (j + 1 < nsteps) st.store(area + (cur ^ 1) * STAGE, area + (cur ^ 1) * STAGE + K_ELEMS, tid);
     __syncthreads();
+  }
+
+  // merge the two halves' partial softmax: half 1 -> LDS -> half 0 (the staging areas are free:
+  // the loop ended with a barrier).  Layout [value][wave][lane] so that lanes read consecutively.
+  if (HALVES == 2) {
+    float* xch = reinterpret_cast<float*>(smem);
+    const int slot = wave * 64 + lane;
+    if (half == 1) {
+      xch[slot] = m_run;
+      xch[256 + slot] = l_run;
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) xch[(2 + dt * 16 + e) * 256 + slot] = oacc[dt][e];
+    }
+    __syncthreads();
+    if (half == 1) return;
+    const float m_b = xch[slot], l_b = xch[256 + slot];
+    const float m_new = fmaxf(m_run, m_b);
+    const float a_a = __builtin_amdgcn_exp2f(m_run - m_new), a_b = __builtin_amdgcn_exp2f(m_b - m_new);
+    m_run = m_new;
+    l_run = l_run * a_a + l_b * a_b;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        oacc[dt][e] = oacc[dt][e] * a_a + xch[(2 + dt * 16 + e) * 256 + slot] * a_b;
   }
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
@@ -203,6 +243,14 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void attn_fwd_kernel(
   if (h == 0)
     lse[((int64_t)bi * nq + head) * s + qrow] = (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
+
+#define KR_ATTN_FWD_ARGS                                                                        \
+  const bf16*, const bf16*, const bf16*, bf16*, float*, int, int, int, float, int64_t, int64_t,  \
+      int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,  \
+      int64_t, int64_t
+template __global__ void attn_fwd_kernel<1>(KR_ATTN_FWD_ARGS);
+template __global__ void attn_fwd_kernel<2>(KR_ATTN_FWD_ARGS);
+#undef KR_ATTN_FWD_ARGS
 
 }  // namespace
 
@@ -224,15 +272,28 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
   if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
        o_sh) % 8)
     return KR_EINVAL;
-  constexpr size_t lds_bytes = 2 * (K_ELEMS + V_ELEMS) * sizeof(bf16);
-  static const hipError_t attr_status = hipFuncSetAttribute(
-      (const void*)attn_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  constexpr size_t lds_one = 2 * (K_ELEMS + V_ELEMS) * sizeof(bf16);  // two buffers per half
+  static const hipError_t attr_status = [] {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<1>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_one);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute((const void*)attn_fwd_kernel<2>,
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds_one));
+  }();
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   const int blocks = (s / BQ) * nq * b;
-  hipLaunchKernelGGL(attn_fwd_kernel, dim3(blocks), dim3(FWD_THREADS), lds_bytes,
-                     (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
-                     lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
-                     v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
+  // few workgroups (at most four per CU): the longest causal rows set the time -> split the keys
+  if (blocks <= 4 * 256) {
+    hipLaunchKernelGGL(attn_fwd_kernel<2>, dim3(blocks), dim3(2 * FWD_THREADS), 2 * lds_one,
+                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
+                       lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
+  } else {
+    hipLaunchKernelGGL(attn_fwd_kernel<1>, dim3(blocks), dim3(FWD_THREADS), lds_one,
+                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
+                       lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
+  }
   return kr_launch_status();
 }
 

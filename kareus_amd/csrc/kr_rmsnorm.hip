@@ -143,21 +143,37 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
   }
 }
 
-// dgamma[col] = sum over partial rows.  A block owns 64 columns; its 4 waves each sum every
-// fourth partial row (256-byte coalesced reads) and combine through LDS.
-__global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* __restrict__ partial,
-                                                             bf16* __restrict__ dgamma,
-                                                             int nparts, int cols) {
-  __shared__ float red[4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col = blockIdx.x * 64 + lane;
-  float acc = 0.f;
-  if (col < cols)
-    for (int p = wave; p < nparts; p += 4) acc += partial[(int64_t)p * cols + col];
-  red[wave][lane] = acc;
+// dgamma[col] = sum over partial rows.  A block of 16 waves owns 32 columns; half-waves take
+// different partial rows (128-byte coalesced reads), 32 row-lanes in all, each summing every
+// 32nd row into four independent accumulators so that many loads are in flight; the row-lanes
+// are combined through LDS in a fixed order.
+constexpr int kDgammaThreads = 1024;
+__global__ __launch_bounds__(kDgammaThreads) void rmsnorm_dgamma_kernel(const float* __restrict__ partial,
+                                                                        bf16* __restrict__ dgamma,
+                                                                        int nparts, int cols) {
+  __shared__ float red[32][33];
+  const int c = threadIdx.x & 31, rl = threadIdx.x >> 5;  // column in block, row-lane 0..31
+  const int col = blockIdx.x * 32 + c;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (col < cols) {
+    const float* src = partial + col;
+    int p = rl;
+    for (; p + 96 < nparts; p += 128) {
+      a0 += src[(int64_t)p * cols];
+      a1 += src[(int64_t)(p + 32) * cols];
+      a2 += src[(int64_t)(p + 64) * cols];
+      a3 += src[(int64_t)(p + 96) * cols];
+    }
+    for (; p < nparts; p += 32) a0 += src[(int64_t)p * cols];
+  }
+  red[rl][c] = (a0 + a1) + (a2 + a3);
   __syncthreads();
-  if (wave == 0 && col < cols)
-    dgamma[col] = (bf16)(red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane]);
+  if (rl == 0 && col < cols) {
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) sum += red[r][c];
+    dgamma[col] = (bf16)sum;
+  }
 }
 
 inline int bwd_blocks(int rows) {
@@ -216,7 +232,7 @@ extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, 
                                            rstd, (const bf16*)gamma, (bf16*)dx, (float*)workspace,
                                            rows, cols, dy_ld, x_ld));
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
-  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 63) / 64), dim3(256), 0,
+  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 31) / 32), dim3(kDgammaThreads), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
   return kr_launch_status();
 }

@@ -187,6 +187,21 @@ def test_attention_forward_backward(be, s, b, nq, nkv):
     assert torch.equal(dqd, dq.flatten(2, 3)) and torch.equal(dkd, dk) and torch.equal(dvd, dv)
 
 
+def test_attention_forward_variants_agree(be):
+    """Up to 1024 workgroups the forward splits each row's keys between two halves of a workgroup
+    and merges two softmax partials; above, one half walks all keys.  Same numbers either way."""
+    s, nq, nkv, hd, b = 1024, 8, 2, 128, 17                   # 8 query tiles x 8 heads x 17 = 1088 workgroups
+    q, k, v = rnd(s, b, nq, hd, seed=40), rnd(s, b, nkv, hd, seed=41), rnd(s, b, nkv, hd, seed=42)
+    o_all, lse_all = be.attn_fwd(q, k, v, hd ** -0.5)          # unsplit variant
+    for bi in (0, 9, 16):
+        o1, lse1 = be.attn_fwd(q[:, bi:bi + 1].contiguous(), k[:, bi:bi + 1].contiguous(),
+                               v[:, bi:bi + 1].contiguous(), hd ** -0.5)   # 64 workgroups: split variant
+        assert rel(o_all[:, bi:bi + 1], o1) <= 1e-2
+        assert (lse_all[bi] - lse1[0]).abs().max() <= 1e-3
+    ro, _ = R.causal_gqa_attention(q[:, 3:4].float(), k[:, 3:4].float(), v[:, 3:4].float(), return_lse=True)
+    assert rel(o_all[:, 3:4], ro) <= TOL
+
+
 def test_attention_special_cases(be):
     hd, s = 128, 256
     # all keys equal -> output row i is the mean of v[0..i]
