@@ -599,7 +599,11 @@ __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
   stg8(dv + dvl.at(bi, kvh) + (int64_t)si * dvl.s_ + c * 8, ov);
 }
 
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
+// HALVES = 2: as in the forward kernel, two halves of an 8-wave workgroup own the same 128
+// queries and walk the even / odd key tiles; half 1's dQ partial is added to half 0's through
+// LDS at the end.  Chosen by the host when there are few workgroups.
+template <int HALVES>
+__global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
     bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
@@ -607,7 +611,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   constexpr int STAGE = 2 * TILE_ELEMS;  // K tile | V tile, both swizzled [64][128]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int half = HALVES == 1 ? 0 : (int)(threadIdx.x >> 8);
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
   const int nqt = s / BQ;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qt = nqt - 1 - (lid % nqt);
@@ -639,23 +644,24 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) dqacc[dt][e] = 0.f;
 
-  const int ntiles = (q0 + BQ) / BKV;
+  const int ntiles = (q0 + BQ) / (HALVES * BKV);  // key tiles per half (the tile count is even)
+  bf16* const area = smem + half * 2 * STAGE;
   TileStager sk, sv;
-  sk.load(kb, kl.s_, 0, tid);
-  sv.load(vb, vl.s_, 0, tid);
-  sk.store(smem, tid);
-  sv.store(smem + TILE_ELEMS, tid);
+  sk.load(kb, kl.s_, half * BKV, tid);
+  sv.load(vb, vl.s_, half * BKV, tid);
+  sk.store(area, tid);
+  sv.store(area + TILE_ELEMS, tid);
   __syncthreads();
 
   for (int j = 0; j < ntiles; ++j) {
     const int cur = j & 1;
     if (j + 1 < ntiles) {
-      sk.load(kb, kl.s_, (j + 1) * BKV, tid);
-      sv.load(vb, vl.s_, (j + 1) * BKV, tid);
+      sk.load(kb, kl.s_, (HALVES * (j + 1) + half) * BKV, tid);
+      sv.load(vb, vl.s_, (HALVES * (j + 1) + half) * BKV, tid);
     }
-    const int key0 = j * BKV;
+    const int key0 = (HALVES * j + half) * BKV;
     if (key0 <= qw0 + 31) {
-      const bf16* ktile = smem + cur * STAGE;
+      const bf16* ktile = area + cur * STAGE;
       const bf16* vtile = ktile + TILE_ELEMS;
       const bool need_mask = key0 + BKV - 1 > qw0;
 #pragma unroll
@@ -691,10 +697,27 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
       }
     }
     if (j + 1 < ntiles) {
-      sk.store(smem + (cur ^ 1) * STAGE, tid);
-      sv.store(smem + (cur ^ 1) * STAGE + TILE_ELEMS, tid);
+      sk.store(area + (cur ^ 1) * STAGE, tid);
+      sv.store(area + (cur ^ 1) * STAGE + TILE_ELEMS, tid);
     }
     __syncthreads();
+  }
+
+  if (HALVES == 2) {  // half 1 -> LDS -> half 0 ([value][wave][lane]; the staging areas are free)
+    float* xch = reinterpret_cast<float*>(smem);
+    const int slot = wave * 64 + lane;
+    if (half == 1) {
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) xch[(dt * 16 + e) * 256 + slot] = dqacc[dt][e];
+    }
+    __syncthreads();
+    if (half == 1) return;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dqacc[dt][e] += xch[(dt * 16 + e) * 256 + slot];
   }
 
   bf16* dqp = dq + dql.at(bi, head, per) + (int64_t)qrow * dql.s_;
@@ -708,6 +731,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
       *reinterpret_cast<bf16x4*>(dqp + dt * 32 + g * 8 + h * 4) = a;
     }
 }
+
+#define KR_ATTN_DQ_ARGS                                                                          \
+  const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, int, int, \
+      int, float, float, QLayout, KLayout, KLayout, QLayout, QLayout
+template __global__ void attn_bwd_dq_kernel<1>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
+#undef KR_ATTN_DQ_ARGS
 
 template __global__ void attn_bwd_dkdv_kernel<false>(const bf16*, const bf16*, const bf16*, const bf16*,
                                                      const float*, const float*, bf16*, bf16*, float*,
@@ -765,8 +795,11 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
       e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel,
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds_dq));
     return e;
   }();
   if (attr_status != hipSuccess) return KR_ELAUNCH;
@@ -794,9 +827,17 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
                        vl, dol, dkl, dvl);
   }
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
-  hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3((s / BQ) * nq * b), dim3(256), lds_dq, st,
-                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
-                     (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
-                     dql);
+  const int dq_blocks = (s / BQ) * nq * b;
+  if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<2>, dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
+                       (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
+                       (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
+                       dql);
+  } else {
+    hipLaunchKernelGGL(attn_bwd_dq_kernel<1>, dim3(dq_blocks), dim3(256), lds_dq, st,
+                       (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
+                       (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
+                       dql);
+  }
   return kr_launch_status();
 }

@@ -200,6 +200,14 @@ def test_attention_forward_variants_agree(be):
         assert (lse_all[bi] - lse1[0]).abs().max() <= 1e-3
     ro, _ = R.causal_gqa_attention(q[:, 3:4].float(), k[:, 3:4].float(), v[:, 3:4].float(), return_lse=True)
     assert rel(o_all[:, 3:4], ro) <= TOL
+    # the query-gradient kernel has the same two variants
+    do = rnd(s, b, nq, hd, seed=43)
+    dq_all, dk_all, dv_all = be.attn_bwd(do, q, k, v, o_all, lse_all, hd ** -0.5)
+    for bi in (0, 16):
+        sl = slice(bi, bi + 1)
+        one = [t[:, sl].contiguous() for t in (do, q, k, v, o_all)]
+        dq1, dk1, dv1 = be.attn_bwd(one[0], one[1], one[2], one[3], one[4], lse_all[sl].contiguous(), hd ** -0.5)
+        assert rel(dq_all[:, sl], dq1) <= 1e-2 and rel(dk_all[:, sl], dk1) <= 1e-2 and rel(dv_all[:, sl], dv1) <= 1e-2
 
 
 def test_attention_special_cases(be):
