@@ -409,7 +409,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
     bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
-    float* __restrict__ part_v, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
+    float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, float scale, float scale_log2,
+    QLayout ql,
     KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   // stage layout: Q tile | dO tile | lse[64] fp32 | delta[64] fp32
@@ -417,7 +418,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
   const int nkt = s / 128;
-  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  // qsplit workgroups share a key tile and take every qsplit-th query tile (fp32 partials, summed
+  // by the group-reduce kernel): with few workgroups the first key tiles, which see all queries,
+  // would otherwise set the kernel's time
+  const int lid_all = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int part = lid_all % qsplit, lid = lid_all / qsplit;
   const int kt = lid % nkt;  // low key tiles see the most queries: they come first
   const int head = (lid / nkt) % nq;
   const int bi = lid / (nkt * nq);
@@ -445,7 +450,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     }
 
   const int qt_first = key0 / 64;
-  const int niter = s / 64 - qt_first;  // query tiles of 64 at or below the diagonal
+  const int niter = (s / 64 - qt_first - part + qsplit - 1) / qsplit;  // this part's query tiles of 64
   const bf16* qb = q + ql.at(bi, head, per);
   const bf16* dob = dout + dol.at(bi, head, per);
   const int64_t stat0 = ((int64_t)bi * nq + head) * s;
@@ -453,7 +458,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   float st_stat = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
 
   auto stage_load = [&](int it) {
-    const int qt = qt_first + it;
+    const int qt = qt_first + it * qsplit + part;
     sq.load(qb, ql.s_, qt * 64, tid);
     sdo.load(dob, dol.s_, qt * 64, tid);
     if (tid < 64) st_stat = lse[stat0 + qt * 64 + tid] * kLog2e;
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   for (int it = 0; it < niter; ++it) {
     const int cur = it & 1;
     if (it + 1 < niter) stage_load(it + 1);
-    const int q0 = (qt_first + it) * 64;
+    const int q0 = (qt_first + it * qsplit + part) * 64;
     const bf16* qtile = smem + cur * STAGE;
     const bf16* dotile = qtile + TILE_ELEMS;
     const float* stats = reinterpret_cast<const float*>(qtile + 2 * TILE_ELEMS);
@@ -526,8 +531,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   }
 
   if (PARTIAL) {
-    float* pk = part_k + (stat0 + krow) * HD;
-    float* pv = part_v + (stat0 + krow) * HD;
+    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + krow;
+    float* pk = part_k + prow * HD;
+    float* pv = part_v + prow * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
@@ -564,7 +570,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
 // 8 channels (two 16-byte reads per partial, one 16-byte bf16 store).
 __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
     const float* __restrict__ part_k, const float* __restrict__ part_v, bf16* __restrict__ dk,
-    bf16* __restrict__ dv, int s, int nq, int nkv, int64_t total, KLayout dkl, KLayout dvl) {
+    bf16* __restrict__ dv, int s, int nq, int nkv, int qsplit, int64_t total, KLayout dkl, KLayout dvl) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (bi, kvh, si, chunk of 8)
   if (idx >= total) return;
   const int c = (int)(idx & 15);
@@ -575,8 +581,8 @@ __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
   float ak[8], av[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) ak[e] = av[e] = 0.f;
-  for (int j = 0; j < per; ++j) {
-    const int64_t off = ((((int64_t)bi * nq + kvh * per + j) * s) + si) * HD + c * 8;
+  for (int j = 0; j < per * qsplit; ++j) {  // (query head of the group, query-tile part) pairs are consecutive
+    const int64_t off = (((((int64_t)bi * nq + kvh * per) * qsplit + j) * s) + si) * HD + c * 8;
     const f32x4 k0 = *reinterpret_cast<const f32x4*>(part_k + off);
     const f32x4 k1 = *reinterpret_cast<const f32x4*>(part_k + off + 4);
     const f32x4 v0 = *reinterpret_cast<const f32x4*>(part_v + off);
@@ -741,19 +747,25 @@ template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
 
 template __global__ void attn_bwd_dkdv_kernel<false>(const bf16*, const bf16*, const bf16*, const bf16*,
                                                      const float*, const float*, bf16*, bf16*, float*,
-                                                     float*, int, int, int, float, float, QLayout,
-                                                     KLayout, KLayout, QLayout, KLayout, KLayout);
+                                                     float*, int, int, int, int, float, float,
+                                                     QLayout, KLayout, KLayout, QLayout, KLayout, KLayout);
 template __global__ void attn_bwd_dkdv_kernel<true>(const bf16*, const bf16*, const bf16*, const bf16*,
                                                     const float*, const float*, bf16*, bf16*, float*,
-                                                    float*, int, int, int, float, float, QLayout,
-                                                    KLayout, KLayout, QLayout, KLayout, KLayout);
+                                                    float*, int, int, int, int, float, float,
+                                                    QLayout, KLayout, KLayout, QLayout, KLayout, KLayout);
 
 }  // namespace
+
+// The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
+// set by the first key tiles (they see every query): two workgroups then share each key tile.
+static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <= 2 * 256 ? 2 : 1; }
 
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
   if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
   size_t bytes = (size_t)b * nq * s * sizeof(float);  // delta
-  if (nq != nkv) bytes += 2 * (size_t)b * nq * s * hd * sizeof(float);  // per-query-head dK, dV
+  const int qsplit = dkdv_query_split(s, b, nq);
+  if (nq != nkv || qsplit > 1)  // fp32 dK, dV partials per (query head, query-tile part)
+    bytes += 2 * (size_t)b * nq * qsplit * s * hd * sizeof(float);
   return bytes;
 }
 
@@ -784,8 +796,9 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   float* delta = (float*)workspace;
   const int64_t rows = (int64_t)b * nq * s;
   float* part_k = delta + rows;
-  float* part_v = part_k + rows * hd;
-  const bool partial = nq != nkv;
+  const int qsplit = dkdv_query_split(s, b, nq);
+  float* part_v = part_k + rows * qsplit * hd;
+  const bool partial = nq != nkv || qsplit > 1;
   constexpr size_t lds_dkdv = 2 * (2 * TILE_ELEMS + 256) * sizeof(bf16);
   constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
   static const hipError_t attr_status = [] {
@@ -809,21 +822,21 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
                      (const bf16*)dout, (const bf16*)o, delta, s, nq, per, rows, dol, ol);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
-  const dim3 grid_kv((s / 128) * nq * b);
+  const dim3 grid_kv((s / 128) * nq * b * qsplit);
   if (partial) {
     hipLaunchKernelGGL(attn_bwd_dkdv_kernel<true>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
                        (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
-                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, scale, scale_log2, ql, kl,
-                       vl, dol, dkl, dvl);
+                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, qsplit, scale, scale_log2, ql,
+                       kl, vl, dol, dkl, dvl);
     if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
     const int64_t total = (int64_t)b * nkv * s * 16;
     hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                        st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
-                       nkv, total, dkl, dvl);
+                       nkv, qsplit, total, dkl, dvl);
   } else {
     hipLaunchKernelGGL(attn_bwd_dkdv_kernel<false>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
                        (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
-                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, scale, scale_log2, ql, kl,
+                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, 1, scale, scale_log2, ql, kl,
                        vl, dol, dkl, dvl);
   }
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
