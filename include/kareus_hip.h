@@ -152,6 +152,38 @@ int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                 int64_t dv_stride_s, int64_t dv_stride_b, int64_t dv_stride_h,
                 void* stream);
 
+/* ---- Ends of the layer stack: embedding and loss ------------------------------------------
+ * Token embedding of one vocabulary shard.  Replaces F.embedding / weight[masked_input] and the
+ * [b s h] -> [s b h] transpose of
+ * 3rdparty/Megatron-LM/megatron/core/tensor_parallel/layers.py:245-263 and
+ * 3rdparty/Megatron-LM/megatron/core/models/common/embeddings/language_model_embedding.py:106-116.
+ * ids: [b, s] int64 token ids; weight, dweight: [vocab_rows, hidden] bf16, the shard holding ids
+ * vocab_start .. vocab_start + vocab_rows - 1; out, dout: [s, b, hidden] bf16 contiguous.
+ * fwd: out[si, bi, :] = weight[ids[bi, si] - vocab_start, :], zeros for ids of other shards.
+ * bwd: dweight[r, :] = sum of dout over the tokens whose id is vocab_start + r, zeros for rows
+ *      without a token; every row is written, sums are taken in one fixed order (no atomics on the result, the
+ *      result is reproducible).  hidden: multiple of 8 (bwd: at most 8192, s*b below 2^26).                    */
+int kr_embedding_fwd(const int64_t* ids, const void* weight, void* out, int s, int b, int hidden,
+                     int64_t vocab_start, int64_t vocab_rows, void* stream);
+int kr_embedding_bwd(const int64_t* ids, const void* dout, void* dweight, int s, int b, int hidden,
+                     int64_t vocab_start, int64_t vocab_rows, void* stream);
+
+/* Cross entropy over rows of logits.  Replaces vocab_parallel_cross_entropy /
+ * te_parallel_cross_entropy as called from
+ * 3rdparty/Megatron-LM/megatron/core/models/common/language_module/language_module.py:71-101 for
+ * a vocabulary held by one shard.
+ * logits: [rows, vocab] bf16 with row stride ld; labels: [rows] int64; loss, lse, dloss: [rows] fp32.
+ * fwd: lse = log sum_j exp(logits[j]), loss = lse - logits[label]; a label outside [0, vocab)
+ *      marks an ignored row (loss 0).
+ * bwd: dlogits[j] = (exp(logits[j] - lse) - [j == label]) * dloss, zeros for ignored rows;
+ *      dlogits ([rows, vocab] bf16, row stride ld_out) may be the logits buffer itself.
+ * vocab, ld, ld_out: multiples of 8.                                                           */
+int kr_cross_entropy_fwd(const void* logits, const int64_t* labels, float* loss, float* lse,
+                         int64_t rows, int vocab, int64_t ld, void* stream);
+int kr_cross_entropy_bwd(const void* logits, const int64_t* labels, const float* lse,
+                         const float* dloss, void* dlogits, int64_t rows, int vocab, int64_t ld,
+                         int64_t ld_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -143,5 +143,38 @@ class EagerBackend:
         back = lambda t: t.permute(2, 0, 1, 3).contiguous()
         return back(dq).to(q.dtype), back(dk).to(k.dtype), back(dv).to(v.dtype)
 
+    # Vocabulary-shard embedding: rows of other shards give zeros
+    # (3rdparty/Megatron-LM/megatron/core/tensor_parallel/layers.py:245-263); output [s, b, h]
+    # (models/common/embeddings/language_model_embedding.py:114-116).
+    def embedding_fwd(self, ids: Tensor, weight: Tensor, vocab_start: int = 0) -> Tensor:
+        rel = ids - vocab_start
+        other = (rel < 0) | (rel >= weight.shape[0])
+        out = weight[rel.masked_fill(other, 0)]
+        out = out.masked_fill(other[..., None], 0.0)
+        return out.transpose(0, 1).contiguous()
+
+    def embedding_bwd(self, ids: Tensor, dout: Tensor, vocab_rows: int, vocab_start: int = 0) -> Tensor:
+        rel = (ids - vocab_start).transpose(0, 1).reshape(-1)          # [s, b] order like dout
+        keep = (rel >= 0) & (rel < vocab_rows)
+        dw = torch.zeros(vocab_rows, dout.shape[-1], dtype=torch.float32, device=dout.device)
+        dw.index_add_(0, rel[keep], dout.reshape(-1, dout.shape[-1])[keep].float())
+        return dw.to(dout.dtype)
+
+    # loss = logsumexp(logits) - logits[label]; rows whose label is outside [0, vocab) are ignored
+    def cross_entropy_fwd(self, logits: Tensor, labels: Tensor) -> Tuple[Tensor, Tensor]:
+        lf = logits.float()
+        lse = torch.logsumexp(lf, dim=-1)
+        live = (labels >= 0) & (labels < logits.shape[-1])
+        picked = lf.gather(1, labels.masked_fill(~live, 0)[:, None])[:, 0]
+        return torch.where(live, lse - picked, torch.zeros_like(lse)), lse
+
+    def cross_entropy_bwd(self, logits: Tensor, labels: Tensor, lse: Tensor, dloss: Tensor,
+                          in_place: bool = False) -> Tensor:
+        live = (labels >= 0) & (labels < logits.shape[-1])
+        d = torch.exp(logits.float() - lse[:, None])
+        d[live, labels[live]] -= 1.0
+        d = d * torch.where(live, dloss.float(), torch.zeros_like(lse))[:, None]
+        return d.to(logits.dtype)
+
     def default_scale(self, hd: int) -> float:
         return 1.0 / math.sqrt(hd)

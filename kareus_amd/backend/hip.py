@@ -36,6 +36,10 @@ _SIGNATURES = {
     "kr_swiglu_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_add": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
     "kr_add_rows": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_i64, _c_int, _c_void_p]),
+    "kr_embedding_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
+    "kr_embedding_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
+    "kr_cross_entropy_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p]),
+    "kr_cross_entropy_bwd": (_c_int, [_c_void_p] * 5 + [_c_i64, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_void_p]),
     "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
     "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_void_p]),
@@ -85,6 +89,11 @@ class HipBackend:
                 raise RuntimeError("the hip backend needs tensors on the HIP device")
             if t.dtype not in (torch.bfloat16, torch.float32):
                 raise RuntimeError(f"unsupported dtype {t.dtype}")
+
+    @staticmethod
+    def _on_device(index: Tensor) -> None:
+        if not index.is_cuda or index.dtype != torch.int64:
+            raise RuntimeError("index tensors must be int64 on the HIP device")
 
     @staticmethod
     def _bf16(*tensors: Tensor) -> None:
@@ -249,6 +258,63 @@ class HipBackend:
             return t.view(-1, cols)
         except RuntimeError:
             return t.reshape(-1, cols)
+
+    # -- embedding and loss ---------------------------------------------------------------
+    def embedding_fwd(self, ids: Tensor, weight: Tensor, vocab_start: int = 0) -> Tensor:
+        """ids [b, s] int64 -> [s, b, hidden]; ids outside this shard's rows give zeros."""
+        self._dev(weight)
+        self._on_device(ids)
+        self._bf16(weight)
+        if ids.dtype != torch.int64 or ids.dim() != 2:
+            raise RuntimeError("token ids must be a [batch, seq] int64 tensor")
+        ids = ids.contiguous()
+        b, s = ids.shape
+        out = torch.empty((s, b, weight.shape[1]), dtype=weight.dtype, device=weight.device)
+        rc = self.lib.kr_embedding_fwd(ids.data_ptr(), weight.data_ptr(), out.data_ptr(), s, b,
+                                       weight.shape[1], vocab_start, weight.shape[0], self._stream())
+        self._check(rc, "kr_embedding_fwd")
+        return out
+
+    def embedding_bwd(self, ids: Tensor, dout: Tensor, vocab_rows: int, vocab_start: int = 0) -> Tensor:
+        self._dev(dout)
+        self._on_device(ids)
+        self._bf16(dout)
+        ids, dout = ids.contiguous(), dout.contiguous()
+        b, s = ids.shape
+        dw = torch.empty((vocab_rows, dout.shape[-1]), dtype=dout.dtype, device=dout.device)
+        rc = self.lib.kr_embedding_bwd(ids.data_ptr(), dout.data_ptr(), dw.data_ptr(), s, b, dout.shape[-1],
+                                       vocab_start, vocab_rows, self._stream())
+        self._check(rc, "kr_embedding_bwd")
+        return dw
+
+    def cross_entropy_fwd(self, logits: Tensor, labels: Tensor) -> Tuple[Tensor, Tensor]:
+        """logits [rows, vocab] bf16, labels [rows] int64 -> (loss [rows] fp32, lse [rows] fp32)."""
+        self._dev(logits)
+        self._on_device(labels)
+        self._bf16(logits)
+        logits, labels = self._rows(logits), labels.contiguous()
+        rows, vocab = logits.shape
+        loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
+        lse = torch.empty(rows, dtype=torch.float32, device=logits.device)
+        rc = self.lib.kr_cross_entropy_fwd(logits.data_ptr(), labels.data_ptr(), loss.data_ptr(), lse.data_ptr(),
+                                           rows, vocab, logits.stride(0), self._stream())
+        self._check(rc, "kr_cross_entropy_fwd")
+        return loss, lse
+
+    def cross_entropy_bwd(self, logits: Tensor, labels: Tensor, lse: Tensor, dloss: Tensor,
+                          in_place: bool = False) -> Tensor:
+        self._dev(logits, lse, dloss)
+        self._on_device(labels)
+        self._bf16(logits)
+        logits = self._rows(logits)
+        rows, vocab = logits.shape
+        out = logits if in_place else torch.empty((rows, vocab), dtype=logits.dtype, device=logits.device)
+        dloss = dloss.to(torch.float32).contiguous()
+        rc = self.lib.kr_cross_entropy_bwd(logits.data_ptr(), labels.contiguous().data_ptr(), lse.data_ptr(),
+                                           dloss.data_ptr(), out.data_ptr(), rows, vocab, logits.stride(0),
+                                           out.stride(0), self._stream())
+        self._check(rc, "kr_cross_entropy_bwd")
+        return out
 
     # -- attention ----------------------------------------------------------------------
     @staticmethod

@@ -21,7 +21,10 @@ from .hardware import available_frequencies_mhz
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="python -m kareus_amd.profiling")
-    ap.add_argument("--partition", choices=PARTITION_KEYS, required=True)
+    ap.add_argument("--partition", choices=PARTITION_KEYS + ("nonpartition",), required=True,
+                    help="one of the four partitions, or the work outside them (embedding, output layer, loss)")
+    ap.add_argument("--vocab-rows", type=int, default=32064, help="vocabulary shard size (nonpartition)")
+    ap.add_argument("--out-dir", default=".", help="directory for the nonpartition CSV files")
     ap.add_argument("--hidden", type=int, default=4096)
     ap.add_argument("--q-heads", type=int, default=8)
     ap.add_argument("--kv-heads", type=int, default=2)
@@ -45,6 +48,17 @@ def main(argv=None) -> int:
                       kv_channels=args.head_dim, ffn_hidden_size=args.ffn, num_nanobatches=args.nanobatches,
                       backend=args.backend,
                       params_dtype=torch.bfloat16 if args.backend == "hip" else torch.float32)
+    if args.partition == "nonpartition":
+        from .nonpartition import NonPartitionProfiler
+
+        prof = NonPartitionProfiler(cfg, args.vocab_rows, args.batch, args.seq_len, device=device)
+        freq = (args.freq or [max(available_frequencies_mhz() or [0])])[0]
+        trials = prof.run(args.out_dir, freq, sampler=PowerSampler(), measurement_duration=args.duration,
+                          cooldown_duration=args.cooldown)
+        for name, t in trials.items():
+            print(json.dumps({"step": name, "freq": freq, "time_s": t.time_per_iter, "energy_j": t.energy_per_iter}),
+                  flush=True)
+        return 0
     test = PartitionTest(args.partition, cfg, args.batch, args.seq_len, device=device)
     freqs = args.freq or [max(available_frequencies_mhz() or [0])]
     configs = all_configurations(freqs, args.sm, test.overlap_windows)

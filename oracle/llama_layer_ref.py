@@ -21,6 +21,14 @@ reference reaches through third-party CUDA libraries, function by function:
                  :34-44 restated in ``swiglu_bwd_formula``
   residual adds  kareus/megatron/core/extensions/ops/bias_dropout_add.py:24-45 with p = 0, no bias
   layer order    kareus/megatron/core/transformer/transformer_layer.py:148-174
+  embedding      3rdparty/Megatron-LM/megatron/core/tensor_parallel/layers.py:245-263 (rows of
+                 one vocabulary shard, zeros for ids of other shards) and the [b s h] -> [s b h]
+                 layout change of models/common/embeddings/language_model_embedding.py:114-116
+  cross_entropy  3rdparty/Megatron-LM/megatron/core/models/common/language_module/
+                 language_module.py:71-101 (labels [b, s], logits [s, b, vocab], loss [b, s]);
+                 per-token loss = logsumexp(logits) - logits[label]
+  model order    embedding -> layers -> final RMSNorm (kareus/megatron/core/transformer/
+                 transformer_block.py:521-525) -> bias-free output layer -> loss
 
 The external pieces (flash-attention 2, Apex fused RoPE, cuBLASLt, Inductor output) are not
 in the reference tree and the reference holds no golden tensors for this path, so every
@@ -181,3 +189,34 @@ def stack_forward_backward(x: Tensor, layers: List[Dict[str, Tensor]], dims: Lay
     y = stack_forward(x, leaves, dims, freqs)
     y.backward(grad_out)
     return y.detach(), x.grad, [{k: v.grad for k, v in p.items()} for p in leaves]
+
+
+def embedding(ids: Tensor, weight: Tensor, vocab_start: int = 0) -> Tensor:
+    """ids [b, s] -> [s, b, h]; an id outside [vocab_start, vocab_start + rows) embeds to zero."""
+    rel = ids - vocab_start
+    inside = (rel >= 0) & (rel < weight.shape[0])
+    out = weight[rel.clamp(0, weight.shape[0] - 1)] * inside[..., None].to(weight.dtype)
+    return out.transpose(0, 1)
+
+
+def cross_entropy(logits: Tensor, labels: Tensor) -> Tensor:
+    """logits [s, b, vocab], labels [b, s] -> per-token loss [b, s]."""
+    lse = torch.logsumexp(logits, dim=-1)                              # [s, b]
+    picked = logits.gather(-1, labels.transpose(0, 1)[..., None])[..., 0]
+    return (lse - picked).transpose(0, 1)
+
+
+def model_forward_backward(ids: Tensor, labels: Tensor, emb: Tensor, layers: List[Dict[str, Tensor]],
+                           final_gamma: Tensor, w_out: Tensor, dims: LayerDims, loss_grad: Tensor,
+                           vocab_start: int = 0):
+    """Returns (loss [b, s], gradients dict with keys emb, layers, final_gamma, w_out)."""
+    freqs = rope_table(ids.shape[1], dims.hd, dims.rope_base, dtype=emb.dtype)
+    leaf = lambda t: t.detach().clone().requires_grad_(True)
+    emb, final_gamma, w_out = leaf(emb), leaf(final_gamma), leaf(w_out)
+    leaves = [{k: leaf(v) for k, v in p.items()} for p in layers]
+    h = stack_forward(embedding(ids, emb, vocab_start), leaves, dims, freqs)
+    logits = linear(rmsnorm(h, final_gamma, dims.eps), w_out)
+    loss = cross_entropy(logits, labels)
+    loss.backward(loss_grad)
+    return loss.detach(), {"emb": emb.grad, "layers": [{k: v.grad for k, v in p.items()} for p in leaves],
+                           "final_gamma": final_gamma.grad, "w_out": w_out.grad}

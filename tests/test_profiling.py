@@ -309,3 +309,40 @@ def test_profile_csv_rows_feed_the_schedule_parser(tmp_path, recompute):
         generate_profile_csv(str(tmp_path), out, 8, gpu_type="H100")
     with pytest.raises(FileNotFoundError):
         generate_profile_csv(str(tmp_path / "missing"), out, 8)
+
+
+def test_nonpartition_profiler_files_round_trip(tmp_path):
+    from kareus_amd.profiling.nonpartition import HEADER, STEP_NAMES, NonPartitionProfiler, read_nonpartition
+
+    prof = NonPartitionProfiler(_cfg(), vocab_rows=96, batch_size=4, seq_len=16)
+    sampler = _FakeSampler(watts=300.0)
+    trials = prof.run(str(tmp_path), 1500, sampler=sampler, world_size=2, measurement_duration=0.02,
+                      cooldown_duration=0.0, warmup_iterations=1, batch=2)
+    assert set(trials) == set(STEP_NAMES)
+    for name in STEP_NAMES:
+        lines = open(tmp_path / "nonpartition" / "1500" / f"{name}_energy.csv").read().strip().splitlines()
+        assert lines[0] == HEADER and len(lines) == 2
+        t, e, e_rank = (float(v) for v in lines[1].split(","))
+        assert t == pytest.approx(trials[name].time_per_iter) and e == pytest.approx(300.0 * t, rel=1e-6)
+        assert e_rank == pytest.approx(e / 2)
+    table = read_nonpartition(str(tmp_path), [1500])
+    assert set(table[1500]) == {"forward-embedding", "forward-output", "loss-func", "backward-embedding", "backward-output"}
+    assert table[1500]["loss-func"] == (pytest.approx(trials["loss"].time_per_iter),
+                                        pytest.approx(trials["loss"].energy_per_iter / 2))
+    # the steps compute what the model's ends compute: postprocess = final norm + output layer
+    logits = prof.step("postprocess")()
+    x = torch.cat(prof.hidden_parts, dim=1)
+    want = R.linear(R.rmsnorm(x, prof.final_gamma.detach(), 1e-5), prof.w_out.detach())
+    assert (logits - want).abs().max() <= 2e-4 * want.abs().max()
+    prof.step("preprocess_backward")()
+    assert prof.embedding.weight.grad is not None and prof.embedding.weight.grad.shape == (96, DIMS.hidden)
+    # and the table plugs into the candidate generator
+    _write_logs(tmp_path)
+    logs = {k: read_eval_log(str(tmp_path / f"{k}.jsonl")) for k in ("fwd_attn", "fwd_mlp", "bwd_attn", "bwd_mlp")}
+    fwd, _ = candidate_points(logs, [2, 2], scale_time_energy=False, nonpartition=table)
+    k = (1500, ("norm_0", "none", 16, 1024), ("linear_0", "none", 16, 1024))
+    assert dict(fwd[0])[k][0] == pytest.approx(3.0 * 2 * 2 + table[1500]["forward-embedding"][0])
+    with pytest.raises(FileNotFoundError):
+        read_nonpartition(str(tmp_path), [999])
+    with pytest.raises(ValueError, match="unknown step"):
+        prof.step("postprocess_sideways")
