@@ -462,37 +462,84 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     if (nk > 1) issue_mine(1);
   }
 
-  // epilogue: lane holds C[m][n..n+3] for m = tile row (lane%32), n = 8g + 4*(lane/32)
-  const int h = lane >> 5;
+  // Epilogue.  A lane holds C[m][n..n+3] for m = tile row (lane%32), n = 8g + 4*(lane/32):
+  // stored from there, every instruction would scatter 64 eight-byte pieces over 32 rows and
+  // the texture-address path, which takes such pieces one at a time, would need ~10 us per
+  // tile.  Instead each wave transposes through its own 4 KB of ring slot 4 (idle until K-step
+  // 2 of the next item is requested, after the next workgroup barrier): 32 rows of 128 bytes
+  // go in from the MFMA layout and come out as whole rows, 8 lanes per row, so an instruction
+  // writes 8 full 128-byte (bf16 output) or 8 contiguous row segments (fp32 partial tiles and
+  // accumulation into C, staged as fp32 so that the sum is rounded once).  Only lanes of the
+  // same wave exchange data: program order of its LDS instructions is all the ordering needed.
+  {
+    char* const stage = reinterpret_cast<char*>(smem + (NSLOTS - 1) * TILE) + wave * 4096;
+    int le = lane;  // opaque copy: nothing derived from it is kept alive through the K loop
+    asm volatile("" : "+v"(le));
+    const int r = le & 31, h = le >> 5;
+    const int wr = r * 128, wsw = (r >> 1) & 7;       // write side: row of the MFMA layout
+    const int rrow = le >> 3, rch = le & 7;           // read side: row 8q + rrow, 16-byte chunk rch
+    const int m_wave = out_m0 + wm * TM * 32, n_wave = out_n0 + wn * TN * 32;
+    auto wave_sync = [&]() {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    };
+    if (out_partial == nullptr && !accumulate) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int m = out_m0 + (wm * TM + i) * 32 + (lane & 31);
-    if (m >= M) continue;
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = out_n0 + (wn * TN + j) * 32 + 8 * g + 4 * h;
-        if (n >= N) continue;
-        if (out_partial != nullptr) {
-          f32x4 pv;
+          for (int g = 0; g < 4; ++g) {
+            bf16x4 o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
-          *reinterpret_cast<f32x4*>(out_partial + (int64_t)m * N + n) = pv;
-          continue;
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)acc[j][i][g * 4 + e];
+            *reinterpret_cast<bf16x4*>(stage + wr + (((4 * j + g) ^ wsw) << 4) + 8 * h) = o;
+          }
+        wave_sync();
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rr = 8 * q + rrow;
+          const bf16x8 v =
+              *reinterpret_cast<const bf16x8*>(stage + rr * 128 + ((rch ^ ((rr >> 1) & 7)) << 4));
+          const int m = m_wave + i * 32 + rr, n = n_wave + 8 * rch;
+          if (m < M && n < N) stg8(C + (int64_t)m * ldc + n, v);
         }
-        bf16* dst = C + (int64_t)m * ldc + n;
-        bf16x4 o;
-        if (accumulate) {
-          const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc[j][i][g * 4 + e] + (float)old[e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (bf16)acc[j][i][g * 4 + e];
-        }
-        *reinterpret_cast<bf16x4*>(dst) = o;
+        wave_sync();
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4 pv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
+            *reinterpret_cast<f32x4*>(stage + wr + (((2 * g + h) ^ wsw) << 4)) = pv;
+          }
+          wave_sync();
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int rr = 8 * q + rrow;
+            const f32x4 v =
+                *reinterpret_cast<const f32x4*>(stage + rr * 128 + ((rch ^ ((rr >> 1) & 7)) << 4));
+            const int m = m_wave + i * 32 + rr, n = n_wave + j * 32 + 4 * rch;
+            if (m >= M || n >= N) continue;
+            if (out_partial != nullptr) {
+              *reinterpret_cast<f32x4*>(out_partial + (int64_t)m * N + n) = v;
+            } else {
+              bf16* dst = C + (int64_t)m * ldc + n;
+              const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
+              bf16x4 o;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)old[e]);
+              *reinterpret_cast<bf16x4*>(dst) = o;
+            }
+          }
+          wave_sync();
+        }
     }
   }
   if (!more) break;

@@ -1,4 +1,4 @@
-"""The partition engine end to end on the host: BASELINE config 1 (fp32 plumbing layer) through
+"""The partition engine end to end on the host: benchmark configuration 1 (fp32 plumbing layer) through
 graph -> partitions -> contexts -> single autograd node, with the eager backend, against the CPU
 oracle; nanobatch counts 1, 2 and 4, with and without activation recompute, with and without a
 schedule; host-forceable error paths; and the stream/event ordering rules replayed without a GPU."""
@@ -53,7 +53,7 @@ def _check(model, x, go, ref, tol=2e-4):
 @pytest.mark.parametrize("nnb", [1, 2, 4])
 @pytest.mark.parametrize("recompute", [False, True])
 def test_config1_matches_oracle(nnb, recompute):
-    # BASELINE config 1 is b=2, s=256, 2 nanobatches; b=4 here so that 4 nanobatches divide it
+    # benchmark configuration 1 is b=2, s=256, 2 nanobatches; b=4 here so that 4 nanobatches divide it
     x, go, ref = _oracle(layers=1, s=256, b=4)
     cfg = LayerConfig(**C1, num_layers=1, num_nanobatches=nnb, params_dtype=torch.float32,
                       backend="eager", checkpoint_activations=recompute)

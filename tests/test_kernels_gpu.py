@@ -1,7 +1,7 @@
 """Parity of every HIP kernel with the CPU oracle, called through the C ABI (ctypes) on the same
 seeded inputs.  Integer-exact where the arithmetic is exact (residual add, index maps), otherwise
 bf16 tolerance: max |err| / max |ref| <= 2e-2 against the fp32 oracle evaluated on the bf16-rounded
-inputs (BASELINE's stated tolerance); observed errors are ~3e-3, one bf16 ulp."""
+inputs (the stated bf16 tolerance of the benchmark); observed errors are ~3e-3, one bf16 ulp."""
 
 import math
 

@@ -110,7 +110,7 @@ def test_streams_recompute_and_schedule_do_not_change_results(fixtures_dir):
 
 
 def test_full_size_properties_config4():
-    """BASELINE config 4 at full size (h4096, 8q/2kv, ffn 3584, MBS 4 x seq 4096): too large for the CPU
+    """Benchmark configuration 4 at full size (h4096, 8q/2kv, ffn 3584, MBS 4 x seq 4096): too large for the CPU
     oracle in test time, so check properties that hold at any size."""
     dims = R.LayerDims(4096, 8, 2, 128, 3584)
     s, b = 4096, 4
