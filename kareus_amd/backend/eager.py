@@ -92,8 +92,12 @@ class EagerBackend:
         d2 = g * x1 * sig
         return torch.cat((d1, d2), dim=-1).to(x.dtype)
 
-    def add(self, a: Tensor, b: Tensor) -> Tensor:
-        return a + b
+    def add(self, a: Tensor, b: Tensor, out: Tensor = None) -> Tensor:
+        if out is None:
+            return a + b
+        if out.shape != a.shape:
+            raise RuntimeError(f"add: out has shape {tuple(out.shape)}, operands {tuple(a.shape)}")
+        return torch.add(a, b, out=out)
 
     # Causal GQA attention on [s, b, heads, hd] tensors; query head i reads KV head
     # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32

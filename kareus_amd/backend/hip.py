@@ -233,31 +233,48 @@ class HipBackend:
                                            self._stream()), "kr_swiglu_bwd")
         return dx
 
-    def add(self, a: Tensor, b: Tensor) -> Tensor:
+    def add(self, a: Tensor, b: Tensor, out: Tensor = None) -> Tensor:
+        """``a + b``; with ``out`` the sum is written there (a slice of a larger tensor is fine as
+        long as one row stride addresses it) instead of into a new tensor."""
         self._dev(a, b)
         self._bf16(a, b)
         if a.shape != b.shape:
             raise RuntimeError(f"add: shapes differ, {tuple(a.shape)} vs {tuple(b.shape)}")
-        if a.is_contiguous() and b.is_contiguous():
+        if out is None and a.is_contiguous() and b.is_contiguous():
             out = torch.empty_like(a)
             self._check(self.lib.kr_add(a.data_ptr(), b.data_ptr(), out.data_ptr(), a.numel(), self._stream()),
                         "kr_add")
             return out
-        # a strided nanobatch slice (one sequence of a [seq, batch, hidden] tensor) is a matrix
-        # with a long row stride: add it in place, do not copy it first
-        cols = a.shape[-1]
-        a2, b2 = self._rows(self._matrix(a, cols)), self._rows(self._matrix(b, cols))
-        out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+        # a strided nanobatch slice (some sequences of a [seq, batch, hidden] tensor) is a matrix
+        # [seq, batch_slice * hidden] with a long row stride: add it in place, do not copy it first
+        a2, b2 = self._rows(self._leading_rows(a)), self._rows(self._leading_rows(b))
+        if out is None:
+            out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+        else:
+            self._dev(out)
+            self._bf16(out)
+            if out.shape != a.shape:
+                raise RuntimeError(f"add: out has shape {tuple(out.shape)}, operands {tuple(a.shape)}")
+        try:
+            o2 = out.view(a2.shape)
+        except RuntimeError:
+            o2 = None
+        if o2 is None or o2.stride(1) != 1 or o2.stride(0) % 8 or o2.stride(0) < o2.shape[1]:
+            raise RuntimeError("add: out cannot be addressed with a single row stride")
+        rows, cols = a2.shape
         self._check(self.lib.kr_add_rows(a2.data_ptr(), a2.stride(0), b2.data_ptr(), b2.stride(0),
-                                         out.data_ptr(), cols, a2.shape[0], cols, self._stream()), "kr_add_rows")
+                                         o2.data_ptr(), o2.stride(0), rows, cols, self._stream()), "kr_add_rows")
         return out
 
     @staticmethod
-    def _matrix(t: Tensor, cols: int) -> Tensor:
+    def _leading_rows(t: Tensor) -> Tensor:
+        """``[d0, ...] -> [d0, rest]`` without a copy when the trailing dimensions are dense."""
+        if t.dim() == 1:
+            return t.view(1, -1)
         try:
-            return t.view(-1, cols)
+            return t.view(t.shape[0], -1)
         except RuntimeError:
-            return t.reshape(-1, cols)
+            return t.reshape(t.shape[0], -1)
 
     # -- embedding and loss ---------------------------------------------------------------
     def embedding_fwd(self, ids: Tensor, weight: Tensor, vocab_start: int = 0) -> Tensor:

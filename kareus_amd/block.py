@@ -69,6 +69,9 @@ class LayerConfig:
     checkpoint_activations: bool = False
     # weight gradients of all nanobatches are summed inside the wgrad GEMM instead of by autograd
     fuse_wgrad_accumulation: bool = True
+    # nanobatch outputs (and input gradients) are written into slices of one tensor by the ops
+    # that produce them, so joining the nanobatches needs no concatenation
+    join_nanobatches_in_place: bool = True
     hidden_dropout: float = 0.0
     attention_dropout: float = 0.0
     add_bias_linear: bool = False
@@ -81,27 +84,79 @@ class LayerConfig:
         return (self.num_attention_heads + 2 * self.num_query_groups) * self.kv_channels
 
 
+def _dense_batch_slices(parts) -> bool:
+    """Whether a nanobatch of this width must be copied: only a nanobatch of one sequence (a
+    matrix with row stride ``b*h``) can be addressed by every kernel without a copy."""
+    return any(p.shape[1] > 1 or p.stride(2) != 1 or p.stride(0) % 8 for p in parts)
+
+
+def _whole_of(parts):
+    """The ``[s, b, h]`` tensor of which ``parts`` are the consecutive batch slices, if they are
+    exactly that (same storage, strides of the whole, back to back); else None."""
+    first = parts[0]
+    if first.dim() != 3:
+        return None
+    s, _, h = first.shape
+    b = sum(p.shape[1] for p in parts)
+    want = (b * h, h, 1)
+    storage, offset = first.untyped_storage().data_ptr(), first.storage_offset()
+    for p in parts:
+        if (p.dim() != 3 or p.shape[0] != s or p.shape[2] != h or p.dtype != first.dtype
+                or p.untyped_storage().data_ptr() != storage or p.storage_offset() != offset):
+            return None
+        if any(p.shape[d] > 1 and p.stride(d) != want[d] for d in range(3)):
+            return None
+        offset += p.shape[1] * h
+    return first.as_strided((s, b, h), want, first.storage_offset())
+
+
 class _SplitNanobatches(torch.autograd.Function):
     """``[s, b, h] -> n x [s, b/n, h]`` along the batch dimension (the reference slices with
     ``hidden_states[:, i*nb:(i+1)*nb]``, transformer_block.py:405-527).
 
     A nanobatch of one sequence is a matrix with row stride ``b*h``; every kernel that touches it
     takes a row stride, so it stays a view.  Wider nanobatches cannot be addressed with a single
-    row stride and are copied into dense tensors once.  Backward writes the n gradients into one
-    ``[s, b, h]`` tensor (one concatenation) instead of autograd's zero-fill + copy + add per
-    slice."""
+    row stride and are copied into dense tensors once.  Backward hands back the tensor the n
+    gradients are slices of when the engine wrote them side by side, else concatenates them
+    (one copy instead of autograd's zero-fill + copy + add per slice)."""
 
     @staticmethod
     def forward(ctx, hidden_states, n):
         nb = hidden_states.shape[1] // n
         parts = [hidden_states[:, i * nb:(i + 1) * nb] for i in range(n)]
-        if nb > 1 or hidden_states.stride(2) != 1 or hidden_states.stride(0) % 8:
+        if _dense_batch_slices(parts):
             parts = [p.contiguous() for p in parts]
         return tuple(parts)
 
     @staticmethod
     def backward(ctx, *grads):
-        return torch.cat(grads, dim=1), None
+        whole = _whole_of(grads)
+        return (whole if whole is not None else torch.cat(grads, dim=1)), None
+
+
+class _JoinNanobatches(torch.autograd.Function):
+    """``n x [s, b/n, h] -> [s, b, h]``: the reference concatenates
+    (transformer_block.py:405-527); when the engine already wrote the nanobatch outputs side by
+    side into one tensor that tensor is the result and nothing is copied.  Backward slices the
+    gradient the way ``_SplitNanobatches`` slices the input."""
+
+    @staticmethod
+    def forward(ctx, *outs):
+        ctx.widths = [o.shape[1] for o in outs]
+        whole = _whole_of(outs)
+        return whole if whole is not None else torch.cat(outs, dim=1)
+
+    @staticmethod
+    def backward(ctx, grad):
+        if grad.stride(2) != 1 or grad.stride(1) != grad.shape[2] or grad.stride(0) != grad.shape[1] * grad.shape[2]:
+            grad = grad.contiguous()
+        parts, lo = [], 0
+        for w in ctx.widths:
+            parts.append(grad[:, lo:lo + w])
+            lo += w
+        if _dense_batch_slices(parts):
+            parts = [p.contiguous() for p in parts]
+        return tuple(parts)
 
 
 class DecoderLayer(torch.nn.Module):
@@ -276,4 +331,4 @@ class LayerStack(torch.nn.Module):
             torch.is_grad_enabled(), self.config.checkpoint_activations,
             *(params * n),
         )
-        return outs[0] if n == 1 else torch.cat(outs, dim=1)
+        return outs[0] if n == 1 else _JoinNanobatches.apply(*outs)

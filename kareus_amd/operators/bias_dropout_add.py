@@ -16,6 +16,8 @@ from ..partitions.tensor_graph import Channel, PartitionableOperator
 
 
 class BiasDropoutAddOp(BasicOperation, PartitionableOperator):
+    forward_accepts_out_sink = True
+
     def __init__(self, has_bias: bool = False, dropout_prob: float = 0.0, training: bool = True,
                  backend="hip") -> None:
         super().__init__()
@@ -38,7 +40,9 @@ class BiasDropoutAddOp(BasicOperation, PartitionableOperator):
         ctx = basic_op_ctxs[0]
         ctx.scale = 1.0
         ctx.has_bias = False
-        out = get_backend(self._backend_name).add(residual, input_)
+        # the engine may name the tensor the sum belongs in (a slice of the block's output)
+        sink = ctx.__dict__.pop("out_sink", None)
+        out = get_backend(self._backend_name).add(residual, input_, out=sink)
         return out, [()]
 
     def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):

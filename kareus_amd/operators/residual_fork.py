@@ -13,6 +13,7 @@ from ..partitions.tensor_graph import Channel, PartitionableOperator
 
 class ResidualForkOp(BasicOperation, PartitionableOperator):
     num_extra_outputs = 1
+    backward_accepts_out_sink = True
 
     def __init__(self, backend="hip") -> None:
         super().__init__()
@@ -27,5 +28,7 @@ class ResidualForkOp(BasicOperation, PartitionableOperator):
 
     def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):
         (grad_residual,) = basic_op_grad_extra_outputs[0]
-        grad_input = get_backend(self._backend_name).add(grad_output, grad_residual)
+        # the engine may name the tensor the sum belongs in (a slice of the block's input gradient)
+        sink = basic_op_ctxs[0].__dict__.pop("out_sink", None)
+        grad_input = get_backend(self._backend_name).add(grad_output, grad_residual, out=sink)
         return grad_input, [()], [()]

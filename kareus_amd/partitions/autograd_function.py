@@ -82,6 +82,32 @@ def _join(streams: Sequence[Optional[object]]) -> None:
                 here.wait_stream(s)
 
 
+def _batch_slices(like: Sequence[Tensor]) -> Optional[List[Tensor]]:
+    """One new ``[s, b, h]`` tensor cut along the batch axis into views shaped like the given
+    per-nanobatch tensors, or None when those are not ``[s, b_i, h]`` tensors of one kind."""
+    first = like[0]
+    if first.dim() != 3 or any(
+        t.dim() != 3 or t.shape[0] != first.shape[0] or t.shape[2] != first.shape[2]
+        or t.dtype != first.dtype or t.device != first.device for t in like
+    ):
+        return None
+    widths = [t.shape[1] for t in like]
+    whole = first.new_empty((first.shape[0], sum(widths), first.shape[2]))
+    views, lo = [], 0
+    for w in widths:
+        views.append(whole[:, lo : lo + w])
+        lo += w
+    return views
+
+
+def _last_compute_op(graph: TensorGraph, capability: str) -> Optional[int]:
+    """op_id of the graph's final compute op if its operator can write into a given tensor."""
+    ops = graph.get_compute_ops()
+    if ops and getattr(ops[-1].operator, capability, False):
+        return ops[-1].op_id
+    return None
+
+
 def _seed_forward(ctxs, hs, rotary, mask, seed: SeedConfig) -> None:
     for ctx, h in zip(ctxs, hs):
         ctx.tensor_store.set(seed.h_tid, h)
@@ -139,6 +165,16 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         ctxs = [NanoBatchContext(batch_idx=i, stream=streams[i]) for i in range(n)]
         _seed_forward(ctxs, hs, rotary, mask, seed)
 
+        # The nanobatch outputs are written side by side into one [s, b, h] tensor, so the
+        # caller can put them together without a copy; likewise the input gradients in backward.
+        in_place = n > 1 and bool(getattr(config, "join_nanobatches_in_place", False))
+        if in_place:
+            last = _last_compute_op(fwd_graph, "forward_accepts_out_sink")
+            sinks = _batch_slices(hs) if last is not None else None
+            if sinks is not None:
+                for c, sink in zip(ctxs, sinks):
+                    c.output_sinks[last] = sink
+
         schedule = scheduler.current_schedule if scheduler is not None else None
         _fork(streams)
         _run_forward(fwd_parts, ctxs, schedule, is_grad_enabled)
@@ -158,6 +194,7 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         func_ctx.attention_mask = mask
         func_ctx.checkpoint_activations = checkpoint_activations
         func_ctx.fuse_wgrad_accumulation = bool(getattr(config, "fuse_wgrad_accumulation", False))
+        func_ctx.join_in_place = in_place
 
         if checkpoint_activations:
             func_ctx.forward_partitions = fwd_parts
@@ -217,6 +254,14 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             for c in ctxs:
                 for op_id, op_ctx in c.op_contexts.items():
                     op_ctx.wgrad_sink = sinks.setdefault(op_id, {})
+
+        if func_ctx.join_in_place:
+            last = _last_compute_op(func_ctx.backward_tensor_graph, "backward_accepts_out_sink")
+            sinks = _batch_slices(grad_outs) if last is not None else None
+            if sinks is not None:
+                for c, sink in zip(ctxs, sinks):
+                    if last in c.op_contexts:
+                        c.op_contexts[last].out_sink = sink
 
         protected = {id(t) for t in (rotary, mask) if t is not None}
         per_nb: List[Dict[int, List]] = [{} for _ in range(n)]

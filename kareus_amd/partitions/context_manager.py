@@ -75,6 +75,8 @@ class NanoBatchContext:
     tensor_store: TensorStore = field(default_factory=TensorStore)
     op_contexts: Dict[int, OperationContext] = field(default_factory=dict)
     stream: Optional[Any] = None  # torch.cuda.Stream this nanobatch runs on (None: caller's)
+    # op_id -> tensor that op's forward output is to be written into (consumed when the op runs)
+    output_sinks: Dict[int, torch.Tensor] = field(default_factory=dict)
     _saved_tensors: List[Optional[torch.Tensor]] = field(default_factory=list)
     _saved_ranges: Dict[int, Tuple[int, int]] = field(default_factory=dict)
 

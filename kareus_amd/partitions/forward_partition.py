@@ -38,6 +38,8 @@ class ForwardPartition(PartitionBase):
                 or any(p.requires_grad for p in op.operator.parameters())
             )
             op_ctx.requires_grad = needs_grad
+            if ctx.output_sinks and op.op_id in ctx.output_sinks:
+                op_ctx.out_sink = ctx.output_sinks.pop(op.op_id)
 
             if start == idx:
                 comm_out, comm_extra = self._launch_comm(pre_ctx, sm_num, block_size)

@@ -78,6 +78,36 @@ def test_fused_weight_gradient_accumulation_equals_autograd_sum(recompute):
         assert (a - b).abs().max() <= 1e-5 * b.abs().max()
 
 
+@pytest.mark.parametrize("b,nnb", [(4, 4), (8, 4), (4, 2)])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_nanobatches_joined_in_place_equal_concatenation(b, nnb, recompute, monkeypatch):
+    """The last op of every nanobatch writes into its slice of one [s, b, h] tensor (and the first
+    fork's backward into its slice of the input gradient): same numbers as concatenating, and
+    no concatenation is run."""
+    x, go, ref = _oracle(layers=2, s=64, b=b)
+    results = {}
+    for in_place in (False, True):
+        cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32,
+                          backend="eager", checkpoint_activations=recompute,
+                          join_nanobatches_in_place=in_place)
+        model = LayerStack(cfg, seed=1234)
+        calls = []
+        real_cat = torch.cat
+        monkeypatch.setattr(torch, "cat", lambda *a, **k: (calls.append(1), real_cat(*a, **k))[1])
+        y, dx = _run(model, x, go)
+        monkeypatch.setattr(torch, "cat", real_cat)
+        results[in_place] = (y, dx, [p.grad.clone() for p in model.parameters()], len(calls))
+        assert y.is_contiguous() and dx.is_contiguous() and y.shape == x.shape
+    (y0, dx0, g0, cats0), (y1, dx1, g1, cats1) = results[False], results[True]
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1)
+    assert all(torch.equal(a, c) for a, c in zip(g0, g1))
+    # joining costs two concatenations (outputs, input gradients); the QKV merge in the attention
+    # backward concatenates too and is there either way
+    assert cats0 - cats1 == 2
+    ry, rdx, _ = ref
+    assert (y1 - ry).abs().max() <= 2e-4 * ry.abs().max() and (dx1 - rdx).abs().max() <= 2e-4 * rdx.abs().max()
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
