@@ -75,6 +75,14 @@ size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols);
 int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
                    void* dx, void* dgamma, void* workspace, int rows, int cols,
                    int64_t dy_ld, int64_t x_ld, void* stream);
+/* RMSNorm backward followed by the backward of the residual fork in front of the norm
+ * (rmsnorm.py:256-263 then kareus/megatron/core/extensions/ops/residual_fork.py:104-106) in one
+ * pass: dx = bf16(dx_norm) + dres, bit-identical to kr_rmsnorm_bwd followed by kr_add.  dres:
+ * [rows, cols] bf16 with row stride dres_ld, or NULL for the plain backward; dx may be a slice of
+ * a larger tensor (row stride dx_ld).  */
+int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd, const void* gamma,
+                       const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
+                       int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
 
 /* ---- Rotary position embedding ---------------------------------------------------------
  * Replaces fused_rotary_positional_embedding.forward / backward (Apex), called from

@@ -46,13 +46,20 @@ class EagerBackend:
 
     # dx = rs * (g - xhat * mean(g * xhat)), g = gamma * dy ; dgamma = sum_rows dy * xhat
     # (rmsnorm_bwd_kernels.cuh:95-128)
-    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor) -> Tuple[Tensor, Tensor]:
+    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor,
+                    residual_grad: Tensor = None, out: Tensor = None) -> Tuple[Tensor, Tensor]:
         xhat = x.float() * rstd[:, None]
         dyf = dy.float()
         g = dyf * gamma.float()
         dx = rstd[:, None] * (g - xhat * (g * xhat).mean(dim=-1, keepdim=True))
         dgamma = (dyf * xhat).sum(dim=0)
-        return dx.to(x.dtype), dgamma.to(gamma.dtype)
+        dx = dx.to(x.dtype)
+        if residual_grad is not None:
+            dx = dx + residual_grad        # rounded first, then added: as the two separate ops do
+        if out is not None:
+            out.copy_(dx)
+            dx = out
+        return dx, dgamma.to(gamma.dtype)
 
     # y = t cos f + rotate_half(t) sin f, rotate_half([a, b]) = [-b, a]; trig in fp32
     # (kareus/megatron/core/models/common/embedding/rope_utils.py:147-182)

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
+    "kr_rmsnorm_bwd_add": (_c_int, [_c_void_p] * 8 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
     "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
                 + [_c_int, _c_int, _c_int, _c_void_p]),
     "kr_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
@@ -155,18 +156,37 @@ class HipBackend:
         self._check(rc, "kr_rmsnorm_fwd")
         return y, rstd
 
-    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor) -> Tuple[Tensor, Tensor]:
+    def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor,
+                    residual_grad: Tensor = None, out: Tensor = None) -> Tuple[Tensor, Tensor]:
+        """``residual_grad`` (same shape as ``x``): the gradient of the residual branch forked off
+        in front of the norm is added to the norm's input gradient in the same pass.  ``out``: the
+        [rows, cols] tensor (possibly a row-strided slice) the input gradient is written into."""
         self._dev(dy, x, rstd, gamma)
         self._bf16(dy, x, gamma)
         x, dy = self._rows(x), self._rows(dy)
         rows, cols = x.shape
-        dx = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
+        if out is None:
+            dx = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
+        else:
+            self._dev(out)
+            self._bf16(out)
+            dx = out
+            if dx.shape != x.shape or dx.stride(1) != 1 or dx.stride(0) % 8 or dx.stride(0) < cols:
+                raise RuntimeError("rmsnorm_bwd: out must be [rows, cols] with a single row stride")
+        res_ptr, res_ld = None, 0
+        if residual_grad is not None:
+            self._dev(residual_grad)
+            self._bf16(residual_grad)
+            if residual_grad.shape != x.shape:
+                raise RuntimeError("rmsnorm_bwd: residual_grad must have the shape of x")
+            residual_grad = self._rows(residual_grad)
+            res_ptr, res_ld = residual_grad.data_ptr(), residual_grad.stride(0)
         dgamma = torch.empty_like(gamma)
         ws = torch.empty(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), dtype=torch.uint8, device=x.device)
-        rc = self.lib.kr_rmsnorm_bwd(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-                                     dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols,
-                                     dy.stride(0), x.stride(0), self._stream())
-        self._check(rc, "kr_rmsnorm_bwd")
+        rc = self.lib.kr_rmsnorm_bwd_add(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+                                         res_ptr, dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols,
+                                         dy.stride(0), x.stride(0), res_ld, dx.stride(0), self._stream())
+        self._check(rc, "kr_rmsnorm_bwd_add")
         return dx, dgamma
 
     # -- RoPE -------------------------------------------------------------------------

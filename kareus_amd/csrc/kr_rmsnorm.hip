@@ -63,11 +63,16 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
   }
 }
 
-template <int NCHUNK>
+// ADD: the residual fork that follows the norm in the backward pass is folded in: the input
+// gradient of the norm is rounded to bf16 exactly as the stand-alone kernel rounds it and then
+// the gradient of the residual branch is added, so the fused result is bit-identical to the
+// two kernels run one after the other while one write and one read of the tensor disappear.
+template <int NCHUNK, bool ADD>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
-    const bf16* __restrict__ gamma, bf16* __restrict__ dx, float* __restrict__ partial, int rows,
-    int cols, int64_t dy_ld, int64_t x_ld) {
+    const bf16* __restrict__ gamma, const bf16* __restrict__ dres, bf16* __restrict__ dx,
+    float* __restrict__ partial, int rows, int cols, int64_t dy_ld, int64_t x_ld, int64_t dres_ld,
+    int64_t dx_ld) {
   __shared__ float red[kWaves - 1][64 * 8];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nvec = cols / 8;
@@ -103,16 +108,19 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
         dg[c][e] += d * xh;
       }
     dot = wave_sum(dot) * inv_cols;
-    bf16* oxr = dx + (int64_t)row * cols;
+    bf16* oxr = dx + (int64_t)row * dx_ld;
+    const bf16* rr = ADD ? dres + (int64_t)row * dres_ld : nullptr;
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int v = lane + c * 64;
       if (v < nvec) {
-        bf16x8 o;
+        bf16x8 o, r;
+        if (ADD) r = ldg8(rr + v * 8);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float xh = (float)xv[c][e] * rs;
           o[e] = (bf16)(rs * ((float)dv[c][e] * (float)g[c][e] - xh * dot));
+          if (ADD) o[e] = (bf16)((float)o[e] + (float)r[e]);
         }
         stg8(oxr + v * 8, o);
       }
@@ -215,24 +223,42 @@ extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
   return (size_t)bwd_blocks(rows) * (size_t)cols * sizeof(float);
 }
 
-extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
-                              void* dx, void* dgamma, void* workspace, int rows, int cols,
-                              int64_t dy_ld, int64_t x_ld, void* stream) {
+extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd,
+                                  const void* gamma, const void* dres, void* dx, void* dgamma,
+                                  void* workspace, int rows, int cols, int64_t dy_ld, int64_t x_ld,
+                                  int64_t dres_ld, int64_t dx_ld, void* stream) {
   if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0 ||
-      dy_ld < cols || x_ld < cols)
+      dy_ld < cols || x_ld < cols || dx_ld < cols || (dres && dres_ld < cols))
     return KR_EINVAL;
-  if (cols % 8 || dy_ld % 8 || x_ld % 8 || cols > 8192) return KR_EUNSUPPORTED;
+  if (cols % 8 || dy_ld % 8 || x_ld % 8 || dx_ld % 8 || (dres && dres_ld % 8) || cols > 8192)
+    return KR_EUNSUPPORTED;
   if (!kr_aligned16(x) || !kr_aligned16(dy) || !kr_aligned16(dx) || !kr_aligned16(gamma) ||
-      !kr_aligned16(workspace))
+      !kr_aligned16(workspace) || (dres && !kr_aligned16(dres)))
     return KR_EINVAL;
   const int blocks = bwd_blocks(rows);
   const int nc = chunks_for(cols);
-  KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_bwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
-                                           (hipStream_t)stream, (const bf16*)dy, (const bf16*)x,
-                                           rstd, (const bf16*)gamma, (bf16*)dx, (float*)workspace,
-                                           rows, cols, dy_ld, x_ld));
+  if (dres) {
+    KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, true>), dim3(blocks),
+                                             dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy,
+                                             (const bf16*)x, rstd, (const bf16*)gamma,
+                                             (const bf16*)dres, (bf16*)dx, (float*)workspace, rows,
+                                             cols, dy_ld, x_ld, dres_ld, dx_ld));
+  } else {
+    KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, false>), dim3(blocks),
+                                             dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy,
+                                             (const bf16*)x, rstd, (const bf16*)gamma,
+                                             (const bf16*)nullptr, (bf16*)dx, (float*)workspace, rows,
+                                             cols, dy_ld, x_ld, (int64_t)0, dx_ld));
+  }
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 31) / 32), dim3(kDgammaThreads), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
   return kr_launch_status();
+}
+
+extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
+                              void* dx, void* dgamma, void* workspace, int rows, int cols,
+                              int64_t dy_ld, int64_t x_ld, void* stream) {
+  return kr_rmsnorm_bwd_add(dy, x, rstd, gamma, nullptr, dx, dgamma, workspace, rows, cols, dy_ld,
+                            x_ld, 0, cols, stream);
 }

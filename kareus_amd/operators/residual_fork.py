@@ -14,6 +14,7 @@ from ..partitions.tensor_graph import Channel, PartitionableOperator
 class ResidualForkOp(BasicOperation, PartitionableOperator):
     num_extra_outputs = 1
     backward_accepts_out_sink = True
+    backward_is_residual_add = True   # backward = grad_main + grad_residual, nothing else
 
     def __init__(self, backend="hip") -> None:
         super().__init__()

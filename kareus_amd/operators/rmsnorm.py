@@ -38,5 +38,37 @@ class RMSNorm(BasicOperation):
         return dx.view(grad_output.shape), (dgamma,)
 
 
+    # -- fused backward with the residual fork that precedes the norm in the layer ------------
+    def can_fuse_backward_with(self, next_operator) -> bool:
+        return bool(getattr(next_operator, "backward_is_residual_add", False))
+
+    def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):
+        if len(basic_op_ctxs) == 1:
+            return super().fuser_backward(basic_op_ctxs, grad_output,
+                                          basic_op_grad_extra_outputs=basic_op_grad_extra_outputs)
+        # [norm, fork]: dx = norm_backward(dy) + grad_residual in one pass over the tensor
+        # (kareus/megatron/core/extensions/ops/residual_fork.py:104-106 after rmsnorm.py:256-263)
+        norm_ctx, fork_ctx = basic_op_ctxs
+        (grad_residual,) = basic_op_grad_extra_outputs[1]
+        sink = fork_ctx.__dict__.pop("out_sink", None)
+        x2d, rstd = norm_ctx.saved_tensors
+        dy = grad_output.reshape(x2d.shape)
+        out2d = None
+        if sink is not None:
+            try:
+                out2d = sink.view(x2d.shape)   # a one-sequence slice is a row-strided matrix
+            except RuntimeError:
+                out2d = None
+        dx, dgamma = get_backend(self._backend_name).rmsnorm_bwd(
+            dy, x2d, rstd, self.weight.detach(), residual_grad=grad_residual.reshape(x2d.shape), out=out2d)
+        if sink is not None:
+            if out2d is None:
+                sink.copy_(dx.view(sink.shape))
+            dx = sink
+        else:
+            dx = dx.view(grad_output.shape)
+        return dx, [(dgamma,), ()], [(), ()]
+
+
 class PartitionableRMSNorm(RMSNorm, PartitionableOperator):
     """RMSNorm that can be placed in a partition graph."""

@@ -21,6 +21,10 @@ from .partition_base import PartitionBase, _current_stream
 
 @dataclass
 class BackwardPartition(PartitionBase):
+    # adjacent ops that offer a fused backward (RMSNorm + the residual fork in front of it) run
+    # as one call; the numbers are those of the separate calls
+    fuse_backward_ops: bool = True
+
     def execute(
         self,
         ctx: NanoBatchContext,
@@ -30,6 +34,25 @@ class BackwardPartition(PartitionBase):
         with self._on_stream(ctx), self._timed():
             return self._execute(ctx, pre_ctx, protected_tensor_ids or set())
 
+    def _fusable_follower(self, idx: int, start: int, ctx: NanoBatchContext):
+        """The op after ``idx`` when the two can run as one fused backward: the first op offers it
+        (``can_fuse_backward_with``), the second consumes the first's only output and needs a
+        gradient, and the scheduled launch point does not fall between them."""
+        if not self.fuse_backward_ops or idx + 1 >= len(self.comp_ops) or start == idx + 1:
+            return None
+        op, nxt = self.comp_ops[idx], self.comp_ops[idx + 1]
+        offer = getattr(op.operator, "can_fuse_backward_with", None)
+        if offer is None or not offer(nxt.operator):
+            return None
+        outs, nxt_ins = op.get_output_tensor_ids(), nxt.get_input_tensor_ids()
+        if len(outs) != 1 or not nxt_ins or nxt_ins[0] != outs[0]:
+            return None
+        if not ctx.get_op_context(nxt.op_id).requires_grad:
+            return None
+        if any(t not in ctx.tensor_store for t in nxt_ins[1:]):
+            return None
+        return nxt
+
     def _execute(self, ctx, pre_ctx, protected: set) -> Dict[int, List]:
         start, _end, sm_num, block_size = self._setup_comm()
         store = ctx.tensor_store
@@ -37,42 +60,54 @@ class BackwardPartition(PartitionBase):
         launched = False
         grad_params: Dict[int, List] = {}
 
-        for idx, op in enumerate(self.comp_ops):
+        idx, num_ops = 0, len(self.comp_ops)
+        while idx < num_ops:
+            op = self.comp_ops[idx]
             op_ctx = ctx.get_op_context(op.op_id)
             if not op_ctx.requires_grad:
                 break
 
             in_ids = op.get_input_tensor_ids()
             dy = store.get(in_ids[0])
+            group, group_ctxs = [op], [op_ctx]
             grad_extra_out = [tuple(store.get(t) for t in in_ids[1:])] if len(in_ids) > 1 else []
+            follower = self._fusable_follower(idx, start, ctx)
+            if follower is not None:
+                group.append(follower)
+                group_ctxs.append(ctx.get_op_context(follower.op_id))
+                grad_extra_out = [tuple(store.get(t) for t in in_ids[1:]),
+                                  tuple(store.get(t) for t in follower.get_input_tensor_ids()[1:])]
+            last = idx + len(group) - 1
 
             if start == idx:
                 comm_out, comm_extra = self._launch_comm(pre_ctx, sm_num, block_size, backward=True)
                 launched = True
 
             dx, op_param_grads, grad_extra_in = op.operator.fuser_backward(
-                [op_ctx], dy, basic_op_grad_extra_outputs=grad_extra_out
+                group_ctxs, dy, basic_op_grad_extra_outputs=grad_extra_out
             )
 
-            grad_params[op.op_id] = [g for group in op_param_grads for g in group]
-            if not self.profiling_mode:
-                if op_ctx.saved_tensors is not None:
-                    clear_tensor_data(
-                        *[t for t in op_ctx.saved_tensors if t is not None and id(t) not in protected]
-                    )
-                op_ctx.saved_tensors = None
-
-            self._op_done(idx)
-            if idx == start - 1:
+            for k, (member, member_ctx) in enumerate(zip(group, group_ctxs)):
+                grad_params[member.op_id] = list(op_param_grads[k]) if len(group) > 1 else [
+                    g for grads in op_param_grads for g in grads]
+                if not self.profiling_mode:
+                    if member_ctx.saved_tensors is not None:
+                        clear_tensor_data(
+                            *[t for t in member_ctx.saved_tensors if t is not None and id(t) not in protected]
+                        )
+                    member_ctx.saved_tensors = None
+                self._op_done(idx + k)
+            if last == start - 1:
                 self.comm_op.event_record(_current_stream())
 
-            out_ids = op.get_output_tensor_ids()
+            out_ids = group[-1].get_output_tensor_ids()
             store.set(out_ids[0], dx)
-            if grad_extra_in and grad_extra_in[0]:
+            if grad_extra_in and grad_extra_in[-1]:
                 for k, tid in enumerate(out_ids[1:]):
-                    g = grad_extra_in[0][k]
+                    g = grad_extra_in[-1][k]
                     if g is not None:
                         store.set(tid, g)
+            idx = last + 1
 
         if self.comm_op is not None:
             if not launched:  # no slot given, or the op loop stopped before reaching it

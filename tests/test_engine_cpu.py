@@ -108,6 +108,41 @@ def test_nanobatches_joined_in_place_equal_concatenation(b, nnb, recompute, monk
     assert (y1 - ry).abs().max() <= 2e-4 * ry.abs().max() and (dx1 - rdx).abs().max() <= 2e-4 * rdx.abs().max()
 
 
+@pytest.mark.parametrize("nnb", [1, 4])
+def test_fused_norm_and_fork_backward_changes_nothing(nnb, monkeypatch):
+    """RMSNorm backward and the residual fork's backward run as one call when adjacent (two pairs
+    per layer); switching the fusion off, or putting the schedule's launch point between the
+    two, gives the same bits."""
+    from kareus_amd.operators.rmsnorm import RMSNorm
+    from kareus_amd.partitions.backward_partition import BackwardPartition
+
+    x, go, ref = _oracle(layers=2, s=64, b=4)
+    fused_calls = []
+    real = RMSNorm.fuser_backward
+
+    def spy(self, ctxs, dy, **kw):
+        fused_calls.append(len(ctxs))
+        return real(self, ctxs, dy, **kw)
+
+    monkeypatch.setattr(RMSNorm, "fuser_backward", spy)
+    results = {}
+    for fuse in (True, False):
+        cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager")
+        model = LayerStack(cfg, seed=1234)
+        for part in model.backward_partitions:
+            assert isinstance(part, BackwardPartition)
+            part.fuse_backward_ops = fuse
+        fused_calls.clear()
+        y, dx = _run(model, x, go)
+        results[fuse] = (y, dx, [p.grad.clone() for p in model.parameters()])
+        assert fused_calls == [2 if fuse else 1] * (4 * nnb)   # 2 layers x 2 norms per nanobatch
+    assert torch.equal(results[True][1], results[False][1])
+    assert all(torch.equal(a, c) for a, c in zip(results[True][2], results[False][2]))
+    for p in model.parameters():
+        p.grad = None
+    _check(model, x, go, ref)
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")

@@ -92,6 +92,44 @@ def test_rmsnorm(be, rows, cols):
     assert (yc.float() - 3.0 / math.sqrt(9.0 + 1e-5)).abs().max() < 1e-2
 
 
+@pytest.mark.parametrize("cols", [512, 3072, 4096, 8192])
+def test_rmsnorm_backward_fused_with_residual_add_is_bit_identical(be, cols):
+    """RMSNorm backward + the residual fork's gradient sum in one kernel: same bits as the two
+    kernels one after the other, also when the residual gradient is a row-strided slice and the
+    result goes into a slice of a larger tensor; the weight gradient is untouched."""
+    rows, batch = 300, 3
+    x, dy = rnd(rows, cols, seed=40), rnd(rows, cols, seed=41)
+    res_full = rnd(rows, batch, cols, seed=42)
+    g = (1 + 0.1 * torch.randn(cols, generator=torch.Generator().manual_seed(43))).to(DEV, torch.bfloat16)
+    _, rstd = be.rmsnorm_fwd(x, g, 1e-5)
+    dx_plain, dg_plain = be.rmsnorm_bwd(dy, x, rstd, g)
+    res = res_full[:, 1, :]
+    want = be.add(dx_plain, res)
+    got, dg = be.rmsnorm_bwd(dy, x, rstd, g, residual_grad=res)
+    assert torch.equal(got, want) and torch.equal(dg, dg_plain)
+    whole = torch.zeros(rows, batch, cols, device=DEV, dtype=torch.bfloat16)
+    sink = whole[:, 2, :]
+    back, _ = be.rmsnorm_bwd(dy, x, rstd, g, residual_grad=res.contiguous(), out=sink)
+    assert back.data_ptr() == sink.data_ptr() and torch.equal(whole[:, 2, :], want)
+    assert not whole[:, :2, :].any()
+    oracle = R.rmsnorm_bwd_formula(dy.float(), x.float(), g.float(), 1e-5)[0] + res.float()
+    assert rel(got, oracle) <= TOL
+
+
+def test_add_writes_into_a_batch_slice(be):
+    """The residual add can put its sum into a [seq, nb, hidden] slice of a [seq, batch, hidden]
+    tensor (one row stride addresses seq rows of nb*hidden elements)."""
+    seq, batch, hidden = 96, 4, 512
+    for nb in (1, 2):
+        a, b = rnd(seq, nb, hidden, seed=50 + nb), rnd(seq, nb, hidden, seed=60 + nb)
+        whole = torch.zeros(seq, batch, hidden, device=DEV, dtype=torch.bfloat16)
+        out = be.add(a, b, out=whole[:, nb:2 * nb])
+        assert out.data_ptr() == whole[:, nb:2 * nb].data_ptr()
+        assert torch.equal(whole[:, nb:2 * nb], a + b) and not whole[:, :nb].any() and not whole[:, 2 * nb:].any()
+    with pytest.raises(RuntimeError):
+        be.add(a, b, out=torch.zeros(seq, hidden, 2 * nb, device=DEV, dtype=torch.bfloat16).transpose(1, 2)[:, :nb])
+
+
 def test_row_strided_nanobatch_slices_need_no_copy(be):
     """One sequence out of a [seq, batch, hidden] tensor is a matrix with row stride batch*hidden:
     RMSNorm (forward and backward) and the residual add must read it in place and give exactly
