@@ -390,6 +390,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     }
   };
 
+  // Two barriers per K-step delimit the half-periods.  The one in the middle of a K-step (after
+  // it, group 1 computes and group 0 moves) orders every LDS hazard: data of the next K-step
+  // visible, slots of the current one free.  The one at the start of a K-step only keeps the two
+  // groups' MFMA bursts apart; every slot a group overwrites after it was last read before the
+  // previous middle barrier.  With a transposed B operand the kernel is a little faster when the
+  // hand-over at the start is left to the hardware (the next burst may begin while the last one
+  // drains); with both operands K-major it is clearly slower, so there the barrier stays.
+  constexpr bool kFreeHandoff = B_T;
   const int total_items = ntiles * (split_k ? splits : 1);
   int item = blockIdx.x;
   select_item(item);
@@ -412,7 +420,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   if (group == 0) {
     read_frags(0);
     for (int ks = 0; ks < nk; ++ks) {
-      lds_barrier();  // half-period 2ks: this group computes, the other moves data
+      // half-period 2ks: this group computes, the other moves data
+      if (!kFreeHandoff) lds_barrier();
       compute();
       if (ks + 1 < nk) {
         // B of step ks+1 was requested one K-step ago
@@ -428,7 +437,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     }
   } else {
     for (int ks = 0; ks < nk; ++ks) {
-      lds_barrier();
+      if (!kFreeHandoff) lds_barrier();
       // A(ks+2) replaces B(ks-1), dead since the previous K-step
       if (ks + 2 < nk)
         move_data(ks, ks + 2);
