@@ -153,40 +153,48 @@ __global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void att
           sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sacc[t], 0, 0, 0);
         }
       }
-      // scores -> log2 domain, causal mask, online softmax
-      const bool need_mask = key0 + BKV - 1 > qw0;
+      // Online softmax in the log2 domain.  The running maximum is kept on the raw scores and
+      // the scale folded into the exponent's multiply-add; only the tile on the diagonal pays
+      // for the causal mask (the branch is wave-uniform); the output accumulators are rescaled
+      // only when some row of the wave saw a new maximum.
+      if (key0 + BKV - 1 > qw0) {
+        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+            if (key > qrow) sacc[t][e] = -INFINITY;
+          }
+      }
       float mx = -INFINITY;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          float sv = sacc[t][e] * scale_log2;
-          if (need_mask) {
-            const int key = key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-            if (key > qrow) sv = -INFINITY;
-          }
-          sacc[t][e] = sv;
-          mx = fmaxf(mx, sv);
-        }
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+      const bool moved = m_new != m_run;
       m_run = m_new;
+      const float neg_m = -m_new * scale_log2;
       float psum = 0.f;
       bf16x8 pb[2][2];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const float p = __builtin_amdgcn_exp2f(sacc[t][e] - m_new);
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][e], scale_log2, neg_m));
           psum += p;
           pb[t][e >> 3][e & 7] = (bf16)p;
         }
       l_run = l_run * alpha + psum;
+      if (__any(moved)) {
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt)
+        for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
+          for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
+      }
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -218,7 +226,8 @@ __global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void att
     if (half == 1) return;
     const float m_b = xch[slot], l_b = xch[256 + slot];
     const float m_new = fmaxf(m_run, m_b);
-    const float a_a = __builtin_amdgcn_exp2f(m_run - m_new), a_b = __builtin_amdgcn_exp2f(m_b - m_new);
+    const float a_a = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+    const float a_b = __builtin_amdgcn_exp2f((m_b - m_new) * scale_log2);
     m_run = m_new;
     l_run = l_run * a_a + l_b * a_b;
 #pragma unroll
@@ -241,7 +250,8 @@ __global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void att
       *reinterpret_cast<bf16x4*>(op + dt * 32 + g * 8 + h * 4) = ov;
     }
   if (h == 0)
-    lse[((int64_t)bi * nq + head) * s + qrow] = (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2;
+    lse[((int64_t)bi * nq + head) * s + qrow] =
+        (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
 #define KR_ATTN_FWD_ARGS                                                                        \
@@ -461,7 +471,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     const int qt = qt_first + it * qsplit + part;
     sq.load(qb, ql.s_, qt * 64, tid);
     sdo.load(dob, dol.s_, qt * 64, tid);
-    if (tid < 64) st_stat = lse[stat0 + qt * 64 + tid] * kLog2e;
+    if (tid < 64) st_stat = -lse[stat0 + qt * 64 + tid] * kLog2e;  // negated: the exponent is one fma
     else if (tid < 128) st_stat = delta[stat0 + qt * 64 + tid - 64];
   };
   auto stage_store = [&](int buf) {
@@ -500,8 +510,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
         const bf16x8 dof = read_rows_swz(dotile, sub * 32, kk, lane);
         dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dof, vf[kk], dpacc, 0, 0, 0);
       }
-      // lane: key column krow, query rows qs0 + 8g + 4h + e
-      const bool need_mask = qs0 < kw0 + 31;
+      // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that straddle the
+      // diagonal pay for the causal mask (wave-uniform branch)
+      if (qs0 < kw0 + 31) {
+        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (qs0 + 8 * (e >> 2) + 4 * h + (e & 3) < krow) sacc[e] = -INFINITY;
+      }
       bf16x8 pb[2], dsb[2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -509,8 +525,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float p = __builtin_amdgcn_exp2f(sacc[g * 4 + e] * scale_log2 - l4[e]);
-          if (need_mask && (qs0 + 8 * g + 4 * h + e < krow)) p = 0.f;
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
           const float ds = p * (dpacc[g * 4 + e] - d4[e]);
           pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
           dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
@@ -641,7 +656,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     dof[kk] = ldg8(dop + kk * 16 + h * 8);
   }
   const int64_t stat = ((int64_t)bi * nq + head) * s + qrow;
-  const float my_lse = lse[stat] * kLog2e;
+  const float neg_lse = -lse[stat] * kLog2e;
   const float my_delta = delta[stat];
 
   f32x16 dqacc[HD / 32];
@@ -669,7 +684,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     if (key0 <= qw0 + 31) {
       const bf16* ktile = area + cur * STAGE;
       const bf16* vtile = ktile + TILE_ELEMS;
-      const bool need_mask = key0 + BKV - 1 > qw0;
+      const bool need_mask = key0 + BKV - 1 > qw0;  // wave-uniform: the tile on the diagonal
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         f32x16 sacc, dpacc;
@@ -687,10 +702,15 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
         }
         // lane: query row qrow, keys key0 + 32t + 8g + 4h + e
         bf16x8 dsb[2];
+        if (need_mask) {
+          asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            if (key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3) > qrow) sacc[e] = -INFINITY;
+        }
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          float p = __builtin_amdgcn_exp2f(sacc[e] * scale_log2 - my_lse);
-          if (need_mask && (key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3) > qrow)) p = 0.f;
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], scale_log2, neg_lse));
           dsb[e >> 3][e & 7] = (bf16)(p * (dpacc[e] - my_delta));
         }
 #pragma unroll
