@@ -79,6 +79,99 @@ __device__ __forceinline__ bf16x8 read_vt_frag(const bf16* vt, int key0, int d0,
   return u.v;
 }
 
+// Output staging.  After the MFMAs a lane holds, for its row (lane % 32), groups of four
+// consecutive channels; stored from there an instruction scatters 64 small pieces over 32 rows
+// and the texture-address path takes them one at a time.  Each wave therefore passes its
+// results through 4 KB of LDS of its own (32 rows of 128 bytes, 16-byte chunks XOR-swizzled
+// against bank conflicts) and reads them back as whole rows, 8 lanes per row, so an
+// instruction writes 8 contiguous 128-byte segments.  Only lanes of one wave exchange data:
+// the program order of its LDS instructions is all the ordering needed.
+struct RowStage {
+  char* base;
+  int wr, wsw, h, rrow, rch;
+  __device__ __forceinline__ void init(void* lds4k, int lane) {
+    base = reinterpret_cast<char*>(lds4k);
+    const int r = lane & 31;
+    h = lane >> 5;
+    wr = r * 128;
+    wsw = (r >> 1) & 7;
+    rrow = lane >> 3;
+    rch = lane & 7;
+  }
+  static __device__ __forceinline__ void sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+  }
+  // bf16 pass = 32 rows x 64 channels: block j (0/1) of 32 channels, group g of the MFMA layout
+  __device__ __forceinline__ void put_bf16(int j, int g, bf16x4 v) const {
+    *reinterpret_cast<bf16x4*>(base + wr + (((4 * j + g) ^ wsw) << 4) + 8 * h) = v;
+  }
+  // read q (0..3): row 8q + lane/8 of the pass, channels 8*(lane%8) .. +7
+  __device__ __forceinline__ bf16x8 get_bf16(int q, int& row, int& col) const {
+    row = 8 * q + rrow;
+    col = 8 * rch;
+    return *reinterpret_cast<const bf16x8*>(base + row * 128 + ((rch ^ ((row >> 1) & 7)) << 4));
+  }
+  // fp32 pass = 32 rows x 32 channels
+  __device__ __forceinline__ void put_f32(int g, f32x4 v) const {
+    *reinterpret_cast<f32x4*>(base + wr + (((2 * g + h) ^ wsw) << 4)) = v;
+  }
+  __device__ __forceinline__ f32x4 get_f32(int q, int& row, int& col) const {
+    row = 8 * q + rrow;
+    col = 4 * rch;
+    return *reinterpret_cast<const f32x4*>(base + row * 128 + ((rch ^ ((row >> 1) & 7)) << 4));
+  }
+};
+
+// 32 rows x 128 channels of fp32 accumulators (scaled) -> bf16 rows at dst + row * row_stride
+__device__ __forceinline__ void store_rows_bf16(const RowStage& st, const f32x16 (&acc)[HD / 32],
+                                                float mul, bf16* dst, int64_t row_stride) {
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (bf16)(acc[2 * pass + j][g * 4 + e] * mul);
+        st.put_bf16(j, g, v);
+      }
+    RowStage::sync();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int row, col;
+      const bf16x8 v = st.get_bf16(q, row, col);
+      stg8(dst + (int64_t)row * row_stride + pass * 64 + col, v);
+    }
+    RowStage::sync();
+  }
+}
+
+// the same as fp32 rows (partial results for a later reduction)
+__device__ __forceinline__ void store_rows_f32(const RowStage& st, const f32x16 (&acc)[HD / 32],
+                                               float mul, float* dst, int64_t row_stride) {
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      f32x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = acc[dt][g * 4 + e] * mul;
+      st.put_f32(g, v);
+    }
+    RowStage::sync();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int row, col;
+      const f32x4 v = st.get_f32(q, row, col);
+      *reinterpret_cast<f32x4*>(dst + (int64_t)row * row_stride + dt * 32 + col) = v;
+    }
+    RowStage::sync();
+  }
+}
+
 // A workgroup owns 128 queries of one (batch, head).  Its eight waves form two halves of four;
 // both halves hold the same queries (wave w and wave w+4 the same 32 rows) and walk the key
 // tiles alternately — half 0 the even 64-key tiles, half 1 the odd ones — each with its own
@@ -239,16 +332,20 @@ __global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void att
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
   const float inv_l = 1.0f / l_tot;
-  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qrow * o_ss;
+  // rows of the wave: qw0 .. qw0+31.  The staging areas are idle by now; with two halves the
+  // hand-over buffer occupies the first (2 + 64) * 1 KiB, so the output staging sits behind it.
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + (HALVES == 2 ? 68 * 1024 : 0) + wave * 4096, lane);
+  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qw0 * o_ss;
+  {
+    // normalise by the row sum (a per-lane factor: the lane's row) while staging
+    f32x16 on[HD / 32];
 #pragma unroll
-  for (int dt = 0; dt < HD / 32; ++dt)
+    for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      bf16x4 ov;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) ov[e] = (bf16)(oacc[dt][g * 4 + e] * inv_l);
-      *reinterpret_cast<bf16x4*>(op + dt * 32 + g * 8 + h * 4) = ov;
-    }
+      for (int e = 0; e < 16; ++e) on[dt][e] = oacc[dt][e] * inv_l;
+    store_rows_bf16(rs, on, 1.0f, op, o_ss);
+  }
   if (h == 0)
     lse[((int64_t)bi * nq + head) * s + qrow] =
         (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
@@ -545,39 +642,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     __syncthreads();
   }
 
+  // the loop ended with a barrier: the staging buffers are free for the output transposition
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + wave * 4096, lane);
   if (PARTIAL) {
-    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + krow;
-    float* pk = part_k + prow * HD;
-    float* pv = part_v + prow * HD;
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 a, b;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          a[e] = dkacc[dt][g * 4 + e] * scale;
-          b[e] = dvacc[dt][g * 4 + e];
-        }
-        *reinterpret_cast<f32x4*>(pk + dt * 32 + g * 8 + h * 4) = a;
-        *reinterpret_cast<f32x4*>(pv + dt * 32 + g * 8 + h * 4) = b;
-      }
+    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + kw0;
+    store_rows_f32(rs, dkacc, scale, part_k + prow * HD, HD);
+    store_rows_f32(rs, dvacc, 1.0f, part_v + prow * HD, HD);
   } else {
-    bf16* dkp = dk + dkl.at(bi, kvh) + (int64_t)krow * dkl.s_;
-    bf16* dvp = dv + dvl.at(bi, kvh) + (int64_t)krow * dvl.s_;
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        bf16x4 a, b;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          a[e] = (bf16)(dkacc[dt][g * 4 + e] * scale);
-          b[e] = (bf16)dvacc[dt][g * 4 + e];
-        }
-        *reinterpret_cast<bf16x4*>(dkp + dt * 32 + g * 8 + h * 4) = a;
-        *reinterpret_cast<bf16x4*>(dvp + dt * 32 + g * 8 + h * 4) = b;
-      }
+    store_rows_bf16(rs, dkacc, scale, dk + dkl.at(bi, kvh) + (int64_t)kw0 * dkl.s_, dkl.s_);
+    store_rows_bf16(rs, dvacc, 1.0f, dv + dvl.at(bi, kvh) + (int64_t)kw0 * dvl.s_, dvl.s_);
   }
 }
 
@@ -746,16 +820,10 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
       for (int e = 0; e < 16; ++e) dqacc[dt][e] += xch[(dt * 16 + e) * 256 + slot];
   }
 
-  bf16* dqp = dq + dql.at(bi, head, per) + (int64_t)qrow * dql.s_;
-#pragma unroll
-  for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      bf16x4 a;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) a[e] = (bf16)(dqacc[dt][g * 4 + e] * scale);
-      *reinterpret_cast<bf16x4*>(dqp + dt * 32 + g * 8 + h * 4) = a;
-    }
+  // output transposition through LDS (behind the 64 KiB hand-over buffer when there are two halves)
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + (HALVES == 2 ? 64 * 1024 : 0) + wave * 4096, lane);
+  store_rows_bf16(rs, dqacc, scale, dq + dql.at(bi, head, per) + (int64_t)qw0 * dql.s_, dql.s_);
 }
 
 #define KR_ATTN_DQ_ARGS                                                                          \
