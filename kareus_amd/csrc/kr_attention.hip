@@ -3,10 +3,9 @@
 // Roofline: MFMA.  Algorithmic work: forward 2*b*nq*s^2*hd FLOP (causal half of 4*s^2*hd),
 // backward 2.5x that.
 //
-// Forward.  A workgroup of 4 waves owns 128 consecutive queries of one (batch, query head);
-// each wave owns 32 of them and never exchanges data with the others — they only share the
-// K/V tiles (64 keys at a time) that the workgroup stages in LDS, double-buffered with the
-// next tile's global loads in flight during the current tile's math.
+// Forward (attn_fwd_pp_kernel below).  A workgroup of 8 waves owns 128 consecutive queries of
+// one (batch, query head); wave w and wave w + 4 own the same 32 of them and walk the even /
+// odd 64-key tiles, in antiphase, merging their softmax partials at the end.
 //   S^T = K . Q^T is computed with K rows on the MFMA A port and the wave's Q fragment (held
 //   in registers for the whole kernel) on the B port, so a lane ends up with 16 scores per
 //   32-key tile *of a single query row* (row = lane % 32; lanes l and l+32 split the keys).
@@ -23,13 +22,8 @@
 namespace {
 
 constexpr int HD = 128;
-constexpr int BQ = 128;       // queries per workgroup (4 waves x 32)
+constexpr int BQ = 128;       // queries per workgroup (4 waves x 32, twice over)
 constexpr int BKV = 64;       // keys per staged tile
-constexpr int LDKT = HD + 8;  // K tile row length in LDS (elements)
-constexpr int LDVT = HD + 32; // V tile row length in LDS (elements)
-constexpr int K_ELEMS = BKV * LDKT;
-constexpr int V_ELEMS = BKV * LDVT;
-constexpr int FWD_THREADS = 256;   // threads of one half of a workgroup (4 waves x 32 queries)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr int kXcds = 8;
@@ -38,45 +32,6 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nblocks) {
   const int q = nblocks / kXcds, r = nblocks % kXcds;
   const int xcd = pid % kXcds;
   return xcd * q + (xcd < r ? xcd : r) + pid / kXcds;
-}
-
-struct KVStager {
-  bf16x8 kreg[4], vreg[4];
-  __device__ __forceinline__ void load(const bf16* __restrict__ kb, const bf16* __restrict__ vb,
-                                       int64_t k_ss, int64_t v_ss, int key0, int tid) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * FWD_THREADS;
-      const int row = c >> 4, col = (c & 15) * 8;
-      kreg[i] = ldg8(kb + (int64_t)(key0 + row) * k_ss + col);
-      vreg[i] = ldg8(vb + (int64_t)(key0 + row) * v_ss + col);
-    }
-  }
-  __device__ __forceinline__ void store(bf16* kt, bf16* vt, int tid) const {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * FWD_THREADS;
-      const int row = c >> 4, col = (c & 15) * 8;
-      *reinterpret_cast<bf16x8*>(kt + row * LDKT + col) = kreg[i];
-      *reinterpret_cast<bf16x8*>(vt + row * LDVT + col) = vreg[i];
-    }
-  }
-};
-
-// V^T fragment for one MFMA: rows-of-output d = d0 + lane%32, contraction slots
-// {key0 + 4h + 0..3, key0 + 8 + 4h + 0..3}, h = lane/32 (matches how P sits in registers).
-__device__ __forceinline__ bf16x8 read_vt_frag(const bf16* vt, int key0, int d0, int lane) {
-  const int p = lane & 15;
-  const int row = key0 + 4 * (lane >> 5) + (p >> 2);
-  const int col = d0 + ((lane >> 4) & 1) * 16 + (p & 3) * 4;
-  const bf16* a0 = vt + row * LDVT + col;
-  union {
-    struct { s16x4 lo, hi; } s;
-    bf16x8 v;
-  } u;
-  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
-  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 8 * LDVT));
-  return u.v;
 }
 
 // Output staging.  After the MFMAs a lane holds, for its row (lane % 32), groups of four
@@ -172,236 +127,12 @@ __device__ __forceinline__ void store_rows_f32(const RowStage& st, const f32x16 
   }
 }
 
-// A workgroup owns 128 queries of one (batch, head).  Its eight waves form two halves of four;
-// both halves hold the same queries (wave w and wave w+4 the same 32 rows) and walk the key
-// tiles alternately — half 0 the even 64-key tiles, half 1 the odd ones — each with its own
-// double-buffered K/V staging area and its own running (max, sum, output).  At the end half 1
-// hands its state to half 0 through LDS and half 0 merges the two softmax partials.  The longest
-// rows of a causal problem thus take half as many steps, which is what bounds the kernel when
-// there are only as many workgroups as CUs (a nanobatch of one sequence).  With plenty of
-// workgroups (HALVES = 1: four waves, every key tile, two workgroups per CU) the coupling of the
-// halves at every barrier costs more than the shorter tail gains, so the host picks per launch.
-template <int HALVES>
-__global__ __launch_bounds__(FWD_THREADS * HALVES, HALVES == 1 ? 2 : 1) void attn_fwd_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
-    bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
-    int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
-    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
-    int64_t o_sg, int64_t o_sh) {
-  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  constexpr int STAGE = K_ELEMS + V_ELEMS;
-
-  const int half = HALVES == 1 ? 0 : (int)(threadIdx.x >> 8);  // which key tiles this wave walks
-  const int tid = threadIdx.x & (FWD_THREADS - 1);   // thread index inside the half
-  const int lane = tid & 63, wave = tid >> 6, h = lane >> 5;
-  const int nqt = s / BQ;
-  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int qt = nqt - 1 - (lid % nqt);  // longest rows first inside each (batch, head)
-  const int head = (lid / nqt) % nq;
-  const int bi = lid / (nqt * nq);
-  const int per = nq / nkv;
-  const int kvh = head / per, hj = head % per;  // KV group and position inside the group
-
-  const int q0 = qt * BQ;
-  const int qw0 = q0 + wave * 32;
-  const int qrow = qw0 + (lane & 31);
-  const bf16* qp = q + (int64_t)bi * q_sb + kvh * q_sg + hj * q_sh + (int64_t)qrow * q_ss;
-  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
-  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
-
-  bf16x8 qf[HD / 16];
-#pragma unroll
-  for (int kk = 0; kk < HD / 16; ++kk) qf[kk] = ldg8(qp + kk * 16 + h * 8);
-
-  f32x16 oacc[HD / 32];
-#pragma unroll
-  for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) oacc[dt][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-
-  const int nsteps = (q0 + BQ) / (HALVES * BKV);  // key tiles per half (the tile count is even)
-  bf16* const area = smem + half * 2 * STAGE;  // this half's two staging buffers
-  KVStager st;
-  st.load(kb, vb, k_ss, v_ss, half * BKV, tid);
-  st.store(area, area + K_ELEMS, tid);
-  __syncthreads();
-
-  for (int j = 0; j < nsteps; ++j) {
-    const int cur = j & 1;
-    if (j + 1 < nsteps) st.load(kb, vb, k_ss, v_ss, (HALVES * (j + 1) + half) * BKV, tid);
-    const int key0 = (HALVES * j + half) * BKV;
-    if (key0 <= qw0 + 31) {  // wave-uniform: this tile has keys some of the wave's rows may see
-      const bf16* kt = area + cur * STAGE;
-      const bf16* vt = kt + K_ELEMS;
-      f32x16 sacc[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < HD / 16; ++kk) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
-              kt + (t * 32 + (lane & 31)) * LDKT + kk * 16 + h * 8);
-          sacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sacc[t], 0, 0, 0);
-        }
-      }
-      // Online softmax in the log2 domain.  The running maximum is kept on the raw scores and
-      // the scale folded into the exponent's multiply-add; only the tile on the diagonal pays
-      // for the causal mask (the branch is wave-uniform); the output accumulators are rescaled
-      // only when some row of the wave saw a new maximum.
-      if (key0 + BKV - 1 > qw0) {
-        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int key = key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-            if (key > qrow) sacc[t][e] = -INFINITY;
-          }
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
-      const bool moved = m_new != m_run;
-      m_run = m_new;
-      const float neg_m = -m_new * scale_log2;
-      float psum = 0.f;
-      bf16x8 pb[2][2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][e], scale_log2, neg_m));
-          psum += p;
-          pb[t][e >> 3][e & 7] = (bf16)p;
-        }
-      l_run = l_run * alpha + psum;
-      if (__any(moved)) {
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-          for (int dt = 0; dt < HD / 32; ++dt) {
-            const bf16x8 vf = read_vt_frag(vt, t * 32 + k2 * 16, dt * 32, lane);
-            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[t][k2], oacc[dt], 0, 0, 0);
-          }
-    }
-    if (j + 1 < nsteps) st.store(area + (cur ^ 1) * STAGE, area + (cur ^ 1) * STAGE + K_ELEMS, tid);
-    __syncthreads();
-  }
-
-  // merge the two halves' partial softmax: half 1 -> LDS -> half 0 (the staging areas are free:
-  // the loop ended with a barrier).  Layout [value][wave][lane] so that lanes read consecutively.
-  if (HALVES == 2) {
-    float* xch = reinterpret_cast<float*>(smem);
-    const int slot = wave * 64 + lane;
-    if (half == 1) {
-      xch[slot] = m_run;
-      xch[256 + slot] = l_run;
-#pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) xch[(2 + dt * 16 + e) * 256 + slot] = oacc[dt][e];
-    }
-    __syncthreads();
-    if (half == 1) return;
-    const float m_b = xch[slot], l_b = xch[256 + slot];
-    const float m_new = fmaxf(m_run, m_b);
-    const float a_a = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
-    const float a_b = __builtin_amdgcn_exp2f((m_b - m_new) * scale_log2);
-    m_run = m_new;
-    l_run = l_run * a_a + l_b * a_b;
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e)
-        oacc[dt][e] = oacc[dt][e] * a_a + xch[(2 + dt * 16 + e) * 256 + slot] * a_b;
-  }
-
-  const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
-  const float inv_l = 1.0f / l_tot;
-  // rows of the wave: qw0 .. qw0+31.  The staging areas are idle by now; with two halves the
-  // hand-over buffer occupies the first (2 + 64) * 1 KiB, so the output staging sits behind it.
-  RowStage rs;
-  rs.init(reinterpret_cast<char*>(smem) + (HALVES == 2 ? 68 * 1024 : 0) + wave * 4096, lane);
-  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qw0 * o_ss;
-  {
-    // normalise by the row sum (a per-lane factor: the lane's row) while staging
-    f32x16 on[HD / 32];
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) on[dt][e] = oacc[dt][e] * inv_l;
-    store_rows_bf16(rs, on, 1.0f, op, o_ss);
-  }
-  if (h == 0)
-    lse[((int64_t)bi * nq + head) * s + qrow] =
-        (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
-}
-
-#define KR_ATTN_FWD_ARGS                                                                        \
-  const bf16*, const bf16*, const bf16*, bf16*, float*, int, int, int, float, int64_t, int64_t,  \
-      int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,  \
-      int64_t, int64_t
-template __global__ void attn_fwd_kernel<1>(KR_ATTN_FWD_ARGS);
-template __global__ void attn_fwd_kernel<2>(KR_ATTN_FWD_ARGS);
-#undef KR_ATTN_FWD_ARGS
-
 }  // namespace
 
 static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
   if (s <= 0 || b <= 0 || nq <= 0 || nkv <= 0) return KR_EINVAL;
   if (hd != HD || s % BQ || nq % nkv) return KR_EUNSUPPORTED;
   return KR_OK;
-}
-
-extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
-                           int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
-                           int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
-                           int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
-                           int64_t o_sg, int64_t o_sh, void* stream) {
-  if (!q || !k || !v || !o || !lse) return KR_EINVAL;
-  const int rc = check_attn_common(s, b, nq, nkv, hd);
-  if (rc != KR_OK) return rc;
-  if (!kr_aligned16(q) || !kr_aligned16(k) || !kr_aligned16(v) || !kr_aligned16(o)) return KR_EINVAL;
-  if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
-       o_sh) % 8)
-    return KR_EINVAL;
-  constexpr size_t lds_one = 2 * (K_ELEMS + V_ELEMS) * sizeof(bf16);  // two buffers per half
-  static const hipError_t attr_status = [] {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<1>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_one);
-    if (e != hipSuccess) return e;
-    return hipFuncSetAttribute((const void*)attn_fwd_kernel<2>,
-                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds_one));
-  }();
-  if (attr_status != hipSuccess) return KR_ELAUNCH;
-  const int blocks = (s / BQ) * nq * b;
-  // few workgroups (at most four per CU): the longest causal rows set the time -> split the keys
-  if (blocks <= 4 * 256) {
-    hipLaunchKernelGGL(attn_fwd_kernel<2>, dim3(blocks), dim3(2 * FWD_THREADS), 2 * lds_one,
-                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
-                       lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
-                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
-  } else {
-    hipLaunchKernelGGL(attn_fwd_kernel<1>, dim3(blocks), dim3(FWD_THREADS), lds_one,
-                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
-                       lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
-                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
-  }
-  return kr_launch_status();
 }
 
 // =============================================================================================
@@ -486,6 +217,276 @@ __device__ __forceinline__ bf16x8 read_cols_swz(const bf16* tile, int r0, int d0
   u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row, col)));
   u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row + 8, col)));
   return u.v;
+}
+
+// ---- direct global -> LDS loads (see the GEMM for why they are written as inline assembly:
+// the compiler must not know of them, or it drains them in front of every barrier).  The 64
+// lanes of one load land contiguously: lane p at lds_byte + 16 p.
+__device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, uint32_t lds_byte) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_byte), "v"(byte_off), "s"(base)
+               : "memory", "m0");
+}
+
+// Ping-pong forward.  Two halves of four waves own the same 128 queries and walk the even / odd
+// key tiles (merged at the end like HALVES = 2 of attn_fwd_kernel), but the halves run in
+// antiphase.  Time is cut into periods by workgroup barriers; in every period one half only
+// feeds the matrix pipe — P.V of its previous tile, then S = Q.K^T of its next one, 32 MFMAs —
+// while the other half does everything else for its own tile: the softmax (exponentials, row
+// statistics, rounding to bf16, the occasional rescale of the output accumulators) and the
+// requests for the K / V tiles two steps ahead, which go straight from global memory into LDS
+// (swizzled [64][128] tiles, the swizzle applied on the global side).  A SIMD hosts one wave of
+// each half, so its matrix pipe and its vector ALU are busy at the same time instead of taking
+// turns, which is what happens when co-resident waves are in the same phase.
+__global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
+    int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+    int64_t o_sg, int64_t o_sh) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+
+  const int half = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+  const int tid = threadIdx.x & 255;
+  const int lane = tid & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nqt = s / BQ;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int qt = nqt - 1 - (lid % nqt);  // longest rows first inside each (batch, head)
+  const int head = (lid / nqt) % nq;
+  const int bi = lid / (nqt * nq);
+  const int per = nq / nkv;
+  const int kvh = head / per, hj = head % per;
+
+  const int q0 = qt * BQ;
+  const int qw0 = q0 + wave * 32;
+  const int qrow = qw0 + (lane & 31);
+  const bf16* qp = q + (int64_t)bi * q_sb + kvh * q_sg + hj * q_sh + (int64_t)qrow * q_ss;
+  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
+  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
+
+  bf16x8 qf[HD / 16];
+#pragma unroll
+  for (int kk = 0; kk < HD / 16; ++kk) qf[kk] = ldg8(qp + kk * 16 + h * 8);
+
+  f32x16 oacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int nsteps = (q0 + BQ) / (2 * BKV);  // key tiles per half
+  // LDS tile = 16 blocks; block b holds rows b, b+16, b+32, b+48 of the tile, 256 bytes each, in
+  // the order one wave-wide request delivers them (lane p at +16 p: row b + 16 (p / 16), chunk
+  // p % 16 — 16 consecutive lanes fetch one contiguous row), followed by a little padding.  With
+  // the padding chosen per operand (K: 16 bytes, V: 64) both kinds of fragment reads are free of
+  // bank conflicts, and every fragment address is one per-lane base plus an instruction
+  // immediate.  Per half: K tile j in kbuf + (j & 1) tiles, V tile j in vbuf + (j & 1) tiles.
+  constexpr uint32_t KBLK = 1024 + 16, VBLK = 1024 + 64, KTILE = 16 * KBLK, VTILE = 16 * VBLK;
+  const uint32_t kbuf = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + half * 2 * (KTILE + VTILE);
+  const uint32_t vbuf = kbuf + 2 * KTILE;
+  auto key_of = [&](int j) { return (2 * j + half) * BKV; };
+  // row-major fragment (K): row 32 t + lane%32, chunk 2 kk + h  ->  + 512 t + 32 kk
+  const uint32_t kfrag_lane = (uint32_t)((lane & 15) * KBLK + ((lane >> 4) & 1) * 256 + h * 16);
+  // transposed fragment (V): rows 16 g + 4 h + p/4 (+8), channels 32 dt + 16 (lane/16 % 2) +
+  // 4 (p % 4)  ->  + 256 g + 64 dt (+ 8 blocks)
+  const uint32_t vfrag_lane = (uint32_t)((4 * h + ((lane & 15) >> 2)) * VBLK + ((lane >> 4) & 1) * 32 +
+                                         ((lane & 3) >> 1) * 16 + (lane & 1) * 8);
+
+  // one wave requests 4 KiB of a tile: blocks wave + 4 i
+  auto request = [&](const bf16* base, int64_t ss, int j, uint32_t tile, uint32_t blk_bytes) {
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
+    const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int blk = wave + 4 * i;
+      dma_b128(base + (int64_t)(key_of(j) + blk) * ss, lane_off, tile + blk * blk_bytes);
+    }
+  };
+
+  request(kb, k_ss, 0, kbuf, KBLK);
+  if (nsteps > 1) request(kb, k_ss, 1, kbuf + KTILE, KBLK);
+  request(vb, v_ss, 0, vbuf, VBLK);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  if (half == 1) __syncthreads();  // half 1 starts one period late
+
+  // a tile is live for this wave if some of its rows can see some of its keys (wave-uniform)
+  auto live = [&](int j) { return key_of(j) <= qw0 + 31; };
+  bf16x8 pb[2][2];
+
+  // O^T += V^T . P^T for tile jj of this half (pb holds its probabilities)
+  auto pv_step = [&](int jj) {
+      uint32_t va = vbuf + (jj & 1) * VTILE + vfrag_lane;
+      asm volatile("" : "+v"(va));  // one base register; everything else is an immediate
+      auto vfrag = [&](int g, int dt) {  // keys 16 g .. 16 g + 15 of the tile, channels 32 dt ..
+        union {
+          struct { s16x4 lo, hi; } s;
+          bf16x8 v;
+        } u;
+        const uint32_t a = va + g * 256 + dt * 64;
+        u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a));
+        u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a + 8 * VBLK));
+        return u.v;
+      };
+      // fragments are fetched one group of four MFMAs ahead, by hand: left to itself the
+      // scheduler hoists every read of the period to its start and runs out of registers
+      bf16x8 fr[2][HD / 32];
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt) fr[0][dt] = vfrag(0, dt);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g + 1 < 4) {
+#pragma unroll
+          for (int dt = 0; dt < HD / 32; ++dt) fr[(g + 1) & 1][dt] = vfrag(g + 1, dt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[g & 1][dt], pb[g >> 1][g & 1],
+                                                             oacc[dt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      };
+
+  for (int j = 0; j < nsteps; ++j) {
+    // ---- matrix period: O^T += V^T . P^T of tile j-1, then S^T = K . Q^T of tile j
+    f32x16 sacc[2];
+    __builtin_amdgcn_s_setprio(1);
+    if (j > 0) pv_step(j - 1);
+    {
+      uint32_t ka = kbuf + (j & 1) * KTILE + kfrag_lane;
+      asm volatile("" : "+v"(ka));
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
+      auto kfrag = [&](int t, int kk) { return *(KR_LDS const bf16x8*)(ka + t * 512 + kk * 32); };
+      bf16x8 fr[2][4];  // group g: contraction steps 2g, 2g+1 for both 32-key blocks
+#pragma unroll
+      for (int u = 0; u < 4; ++u) fr[0][u] = kfrag(u & 1, u >> 1);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g + 1 < 4) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) fr[(g + 1) & 1][u] = kfrag(u & 1, 2 * (g + 1) + (u >> 1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[g & 1][u], qf[2 * g + (u >> 1)],
+                                                                sacc[u & 1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();
+
+    // ---- vector period of tile j: request K(j+2) and V(j+1) (their buffers were last read in
+    // the matrix period that just ended), then the softmax
+    if (j + 2 < nsteps) request(kb, k_ss, j + 2, kbuf + (j & 1) * KTILE, KBLK);
+    if (j + 1 < nsteps) request(vb, v_ss, j + 1, vbuf + ((j + 1) & 1) * VTILE, VBLK);
+    {
+      const int key0 = key_of(j);
+      if (key0 + BKV - 1 > qw0) {
+        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+        const int lim = qrow - key0 - 4 * h;  // element offsets beyond it are keys after the query
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            if (t * 32 + 8 * (e >> 2) + (e & 3) > lim) sacc[t][e] = -INFINITY;
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // nothing seen yet: any finite reference
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);
+      const bool moved = m_new != m_run;
+      m_run = m_new;
+      const float neg_m = -m_ref * scale_log2;
+      float psum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][e], scale_log2, neg_m));
+          psum += pe;
+          pb[t][e >> 3][e & 7] = (bf16)pe;
+          // eight elements at a time: scheduled freely, all 32 exponent arguments and results
+          // would be alive together
+          if ((e & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+        }
+      l_run = l_run * alpha + psum;
+      if (__any(moved)) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
+      }
+    }
+    // what was requested one step ago (K(j+1), V(j)) is read in the next matrix period; the
+    // requests of this period (at most 8 per wave, retired in order) may stay in flight
+    if (j + 1 < nsteps)
+      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing is requested any more
+    __syncthreads();
+  }
+  // last matrix period: the product of the final tile
+  __builtin_amdgcn_s_setprio(1);
+  pv_step(nsteps - 1);
+  __builtin_amdgcn_s_setprio(0);
+  __syncthreads();
+  if (half == 0) __syncthreads();  // the period half 1 is behind by
+
+  // merge the two halves' partial softmax: half 1 -> LDS -> half 0 (every buffer is idle: the
+  // loop ended with a barrier and no request is in flight).  [value][wave][lane] layout.
+  float* xch = reinterpret_cast<float*>(smem);
+  const int slot = wave * 64 + lane;
+  if (half == 1) {
+    xch[slot] = m_run;
+    xch[256 + slot] = l_run;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) xch[(2 + dt * 16 + e) * 256 + slot] = oacc[dt][e];
+  }
+  __syncthreads();
+  if (half == 1) return;
+  {
+    const float m_b = xch[slot], l_b = xch[256 + slot];
+    const float m_new = fmaxf(m_run, m_b);
+    const float a_a = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2);
+    const float a_b = __builtin_amdgcn_exp2f((m_b - m_new) * scale_log2);
+    m_run = m_new;
+    l_run = l_run * a_a + l_b * a_b;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        oacc[dt][e] = oacc[dt][e] * a_a + xch[(2 + dt * 16 + e) * 256 + slot] * a_b;
+  }
+  const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
+  const float inv_l = 1.0f / l_tot;
+  RowStage rs;  // behind the (2 + 64) KiB hand-over buffer
+  rs.init(reinterpret_cast<char*>(smem) + 68 * 1024 + wave * 4096, lane);
+  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qw0 * o_ss;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[dt][e] *= inv_l;
+  store_rows_bf16(rs, oacc, 1.0f, op, o_ss);
+  if (h == 0)
+    lse[((int64_t)bi * nq + head) * s + qrow] =
+        (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ dout,
@@ -611,9 +612,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
       // diagonal pay for the causal mask (wave-uniform branch)
       if (qs0 < kw0 + 31) {
         asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+        const int lim = krow - qs0 - 4 * h;  // element offsets below it are queries before the key
 #pragma unroll
         for (int e = 0; e < 16; ++e)
-          if (qs0 + 8 * (e >> 2) + 4 * h + (e & 3) < krow) sacc[e] = -INFINITY;
+          if (8 * (e >> 2) + (e & 3) < lim) sacc[e] = -INFINITY;
       }
       bf16x8 pb[2], dsb[2];
 #pragma unroll
@@ -778,9 +780,10 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
         bf16x8 dsb[2];
         if (need_mask) {
           asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+          const int lim = qrow - key0 - t * 32 - 4 * h;
 #pragma unroll
           for (int e = 0; e < 16; ++e)
-            if (key0 + t * 32 + 8 * (e >> 2) + 4 * h + (e & 3) > qrow) sacc[e] = -INFINITY;
+            if (8 * (e >> 2) + (e & 3) > lim) sacc[e] = -INFINITY;
         }
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -942,3 +945,31 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   }
   return kr_launch_status();
 }
+
+extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
+                           int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
+                           int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
+                           int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+                           int64_t o_sg, int64_t o_sh, void* stream) {
+  if (!q || !k || !v || !o || !lse) return KR_EINVAL;
+  const int rc = check_attn_common(s, b, nq, nkv, hd);
+  if (rc != KR_OK) return rc;
+  if (!kr_aligned16(q) || !kr_aligned16(k) || !kr_aligned16(v) || !kr_aligned16(o)) return KR_EINVAL;
+  if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
+       o_sh) % 8)
+    return KR_EINVAL;
+  // two K and two V tiles of 17 KiB (padded blocks) per half; afterwards the same memory holds
+  // the hand-over of half 1 (66 KiB) and, from 68 KiB on, 4 KiB of output staging per wave
+  constexpr size_t lds_pp = 2 * 2 * 16 * ((1024 + 16) + (1024 + 64));  // 133 KiB
+  static_assert(lds_pp >= 84 * 1024, "hand-over and output staging must fit");
+  static const hipError_t attr_status = hipFuncSetAttribute(
+      (const void*)attn_fwd_pp_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_pp);
+  if (attr_status != hipSuccess) return KR_ELAUNCH;
+  const int blocks = (s / BQ) * nq * b;
+  hipLaunchKernelGGL(attn_fwd_pp_kernel, dim3(blocks), dim3(512), lds_pp, (hipStream_t)stream,
+                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o, lse, s, nq, nkv,
+                     scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, o_ss,
+                     o_sb, o_sg, o_sh);
+  return kr_launch_status();
+}
+
