@@ -229,6 +229,51 @@ __device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, ui
                : "memory", "m0");
 }
 
+// ---- blocked LDS tile: [64 rows][128 channels] bf16, filled straight from global memory ------
+// A tile is 16 blocks; block B holds rows r, r+16, r+32, r+48 (r = 4 (B % 4) + B / 4), 256 bytes
+// each, in the order one wave-wide request delivers them (lane p at +16 p: row r + 16 (p / 16),
+// 16-byte chunk p % 16 — 16 consecutive lanes fetch one contiguous row), then 16 bytes of
+// padding.  Both ways of reading fragments out of it are free of bank conflicts, and every
+// fragment address is one per-lane base plus an instruction immediate.
+constexpr uint32_t BT_BLK = 1024 + 16, BT_BYTES = 16 * BT_BLK;
+
+// the four waves of a group bring in one tile (rows = its first row in global memory)
+__device__ __forceinline__ void bt_request(const bf16* rows, int64_t ss, uint32_t tile, int wave,
+                                           int lane) {
+  int l2 = lane;
+  asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
+  const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int blk = wave + 4 * i;
+    dma_b128(rows + (int64_t)(4 * (blk & 3) + (blk >> 2)) * ss, lane_off, tile + blk * BT_BLK);
+  }
+}
+// row-major fragments: lane gets row 32 t + lane % 32, channels 16 kk + 8 (lane / 32) + 0..7
+__device__ __forceinline__ uint32_t bt_rows_lane(int lane) {
+  const int r = lane & 31;
+  return (uint32_t)((4 * (r & 3) + ((r >> 2) & 3)) * BT_BLK + (r >> 4) * 256 + (lane >> 5) * 16);
+}
+__device__ __forceinline__ bf16x8 bt_rows(uint32_t base, int t, int kk) {
+  return *(KR_LDS const bf16x8*)(base + t * 512 + kk * 32);
+}
+// transposed fragments: lane gets channel 32 dt + lane % 32, rows 16 g + {4 h + 0..3, 8 + 4 h + 0..3}
+__device__ __forceinline__ uint32_t bt_cols_lane(int lane) {
+  const int p = lane & 15;
+  return (uint32_t)((4 * (p >> 2) + (lane >> 5)) * BT_BLK + ((lane >> 4) & 1) * 32 +
+                    ((p & 3) >> 1) * 16 + (p & 1) * 8);
+}
+__device__ __forceinline__ bf16x8 bt_cols(uint32_t base, int g, int dt) {
+  union {
+    struct { s16x4 lo, hi; } s;
+    bf16x8 v;
+  } u;
+  const uint32_t a = base + g * 256 + dt * 64;
+  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a));
+  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a + 2 * BT_BLK));
+  return u.v;
+}
+
 // Ping-pong forward.  Two halves of four waves own the same 128 queries and walk the even / odd
 // key tiles (merged at the end like HALVES = 2 of attn_fwd_kernel), but the halves run in
 // antiphase.  Time is cut into periods by workgroup barriers; in every period one half only
@@ -521,10 +566,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     QLayout ql,
     KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  // stage layout: Q tile | dO tile | lse[64] fp32 | delta[64] fp32
-  constexpr int STAGE = 2 * TILE_ELEMS + 256;  // in bf16 units (256 bf16 = 128 floats)
+  // stage layout: Q tile | dO tile (blocked tiles) | lse[64] fp32 | delta[64] fp32
+  constexpr uint32_t STAGE = 2 * BT_BYTES + 512;  // bytes
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nkt = s / 128;
   // qsplit workgroups share a key tile and take every qsplit-th query tile (fp32 partials, summed
   // by the group-reduce kernel): with few workgroups the first key tiles, which see all queries,
@@ -562,35 +608,39 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   const bf16* qb = q + ql.at(bi, head, per);
   const bf16* dob = dout + dol.at(bi, head, per);
   const int64_t stat0 = ((int64_t)bi * nq + head) * s;
-  TileStager sq, sdo;
   float st_stat = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
 
-  auto stage_load = [&](int it) {
+  // Q and dO tiles go straight from global memory into LDS; the row statistics pass through a
+  // register of the first 128 threads
+  auto stage_request = [&](int it, int buf) {
     const int qt = qt_first + it * qsplit + part;
-    sq.load(qb, ql.s_, qt * 64, tid);
-    sdo.load(dob, dol.s_, qt * 64, tid);
+    bt_request(qb + (int64_t)qt * 64 * ql.s_, ql.s_, lds0 + buf * STAGE, wave, lane);
+    bt_request(dob + (int64_t)qt * 64 * dol.s_, dol.s_, lds0 + buf * STAGE + BT_BYTES, wave, lane);
     if (tid < 64) st_stat = -lse[stat0 + qt * 64 + tid] * kLog2e;  // negated: the exponent is one fma
     else if (tid < 128) st_stat = delta[stat0 + qt * 64 + tid - 64];
   };
-  auto stage_store = [&](int buf) {
-    bf16* base = smem + buf * STAGE;
-    sq.store(base, tid);
-    sdo.store(base + TILE_ELEMS, tid);
-    float* stats = reinterpret_cast<float*>(base + 2 * TILE_ELEMS);
+  auto stage_publish = [&](int buf) {
+    float* stats = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + buf * STAGE + 2 * BT_BYTES);
     if (tid < 128) stats[tid] = st_stat;
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of both tiles has landed
   };
 
-  stage_load(0);
-  stage_store(0);
+  stage_request(0, 0);
+  stage_publish(0);
   __syncthreads();
 
   for (int it = 0; it < niter; ++it) {
     const int cur = it & 1;
-    if (it + 1 < niter) stage_load(it + 1);
+    if (it + 1 < niter) stage_request(it + 1, cur ^ 1);
     const int q0 = (qt_first + it * qsplit + part) * 64;
-    const bf16* qtile = smem + cur * STAGE;
-    const bf16* dotile = qtile + TILE_ELEMS;
-    const float* stats = reinterpret_cast<const float*>(qtile + 2 * TILE_ELEMS);
+    const uint32_t qtile = lds0 + cur * STAGE, dotile = qtile + BT_BYTES;
+    const float* stats =
+        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + cur * STAGE + 2 * BT_BYTES);
+    // one base register per tile and read direction; everything else is an immediate
+    uint32_t q_rows = qtile + bt_rows_lane(lane), do_rows = dotile + bt_rows_lane(lane);
+    uint32_t q_cols = qtile + bt_cols_lane(lane), do_cols = dotile + bt_cols_lane(lane);
+    asm volatile("" : "+v"(q_rows), "+v"(do_rows), "+v"(q_cols), "+v"(do_cols));
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int qs0 = q0 + sub * 32;
@@ -603,10 +653,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
       }
 #pragma unroll
       for (int kk = 0; kk < HD / 16; ++kk) {
-        const bf16x8 qfr = read_rows_swz(qtile, sub * 32, kk, lane);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr, kf[kk], sacc, 0, 0, 0);
-        const bf16x8 dof = read_rows_swz(dotile, sub * 32, kk, lane);
-        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dof, vf[kk], dpacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(q_rows, sub, kk), kf[kk], sacc, 0, 0, 0);
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(do_rows, sub, kk), vf[kk], dpacc, 0, 0, 0);
       }
       // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that straddle the
       // diagonal pay for the causal mask (wave-uniform branch)
@@ -634,13 +682,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
       for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
-          const bf16x8 dot = read_cols_swz(dotile, sub * 32 + k2 * 16, dt * 32, lane);
-          dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot, pb[k2], dvacc[dt], 0, 0, 0);
-          const bf16x8 qtr = read_cols_swz(qtile, sub * 32 + k2 * 16, dt * 32, lane);
-          dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr, dsb[k2], dkacc[dt], 0, 0, 0);
+          dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(do_cols, 2 * sub + k2, dt), pb[k2],
+                                                              dvacc[dt], 0, 0, 0);
+          dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(q_cols, 2 * sub + k2, dt), dsb[k2],
+                                                              dkacc[dt], 0, 0, 0);
         }
     }
-    if (it + 1 < niter) stage_store(cur ^ 1);
+    if (it + 1 < niter) stage_publish(cur ^ 1);
     __syncthreads();
   }
 
@@ -890,7 +938,7 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   const int qsplit = dkdv_query_split(s, b, nq);
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
-  constexpr size_t lds_dkdv = 2 * (2 * TILE_ELEMS + 256) * sizeof(bf16);
+  constexpr size_t lds_dkdv = 2 * (2 * BT_BYTES + 512);  // two stages: Q tile, dO tile, statistics
   constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
