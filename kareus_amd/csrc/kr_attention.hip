@@ -626,70 +626,91 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of both tiles has landed
   };
 
+  // Three stages: while tile `it` is consumed, tile it+1 is already complete (its first score
+  // block is computed one step ahead, see below) and tile it+2 is on its way.
   stage_request(0, 0);
   stage_publish(0);
+  if (niter > 1) {
+    stage_request(1, 1);
+    stage_publish(1);
+  }
   __syncthreads();
 
-  for (int it = 0; it < niter; ++it) {
-    const int cur = it & 1;
-    if (it + 1 < niter) stage_request(it + 1, cur ^ 1);
-    const int q0 = (qt_first + it * qsplit + part) * 64;
-    const uint32_t qtile = lds0 + cur * STAGE, dotile = qtile + BT_BYTES;
-    const float* stats =
-        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + cur * STAGE + 2 * BT_BYTES);
-    // one base register per tile and read direction; everything else is an immediate
-    uint32_t q_rows = qtile + bt_rows_lane(lane), do_rows = dotile + bt_rows_lane(lane);
-    uint32_t q_cols = qtile + bt_cols_lane(lane), do_cols = dotile + bt_cols_lane(lane);
-    asm volatile("" : "+v"(q_rows), "+v"(do_rows), "+v"(q_cols), "+v"(do_cols));
+  // The wave runs alone on its SIMD, so the overlap of matrix and vector work has to come from
+  // inside it: the two score products of a 32-query block (S = Q.K^T, dP = dO.V^T) are issued
+  // one block ahead of the exponentials that consume them, and execute while the vector ALU
+  // works on the previous block.  Blocks that lie wholly before the wave's keys are not
+  // skipped but masked to zero (there are at most three per wave): the loop body stays
+  // straight-line code and the accumulators stay where they are.
+  auto scores = [&](int buf, int sub, f32x16& sacc, f32x16& dpacc) {
+    uint32_t q_rows = lds0 + buf * STAGE + bt_rows_lane(lane);
+    uint32_t do_rows = q_rows + BT_BYTES;
+    asm volatile("" : "+v"(q_rows), "+v"(do_rows));  // one base register each; the rest are immediates
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      const int qs0 = q0 + sub * 32;
-      if (qs0 + 31 < kw0) continue;  // wave-uniform: every query of the block precedes the keys
-      f32x16 sacc, dpacc;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        sacc[e] = 0.f;
-        dpacc[e] = 0.f;
-      }
-#pragma unroll
-      for (int kk = 0; kk < HD / 16; ++kk) {
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(q_rows, sub, kk), kf[kk], sacc, 0, 0, 0);
-        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(do_rows, sub, kk), vf[kk], dpacc, 0, 0, 0);
-      }
-      // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that straddle the
-      // diagonal pay for the causal mask (wave-uniform branch)
-      if (qs0 < kw0 + 31) {
-        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
-        const int lim = krow - qs0 - 4 * h;  // element offsets below it are queries before the key
-#pragma unroll
-        for (int e = 0; e < 16; ++e)
-          if (8 * (e >> 2) + (e & 3) < lim) sacc[e] = -INFINITY;
-      }
-      bf16x8 pb[2], dsb[2];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
-          const float ds = p * (dpacc[g * 4 + e] - d4[e]);
-          pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
-          dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
-        }
-      }
-#pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt) {
-          dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(do_cols, 2 * sub + k2, dt), pb[k2],
-                                                              dvacc[dt], 0, 0, 0);
-          dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(q_cols, 2 * sub + k2, dt), dsb[k2],
-                                                              dkacc[dt], 0, 0, 0);
-        }
+    for (int e = 0; e < 16; ++e) {
+      sacc[e] = 0.f;
+      dpacc[e] = 0.f;
     }
-    if (it + 1 < niter) stage_publish(cur ^ 1);
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(q_rows, sub, kk), kf[kk], sacc, 0, 0, 0);
+      dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(do_rows, sub, kk), vf[kk], dpacc, 0, 0, 0);
+    }
+  };
+  // P = exp2(S c - lse), dS = P (dP - delta); then dV^T += dO^T . P and dK^T += Q^T . dS
+  auto consume = [&](int buf, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
+    const float* stats =
+        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + buf * STAGE + 2 * BT_BYTES);
+    // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that reach the diagonal
+    // pay for the causal mask (wave-uniform branch)
+    if (qs0 < kw0 + 31) {
+      asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+      const int lim = krow - qs0 - 4 * h;  // element offsets below it are queries before the key
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        if (8 * (e >> 2) + (e & 3) < lim) sacc[e] = -INFINITY;
+    }
+    bf16x8 pb[2], dsb[2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
+        const float ds = p * (dpacc[g * 4 + e] - d4[e]);
+        pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
+        dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
+      }
+    }
+    uint32_t q_cols = lds0 + buf * STAGE + bt_cols_lane(lane);
+    uint32_t do_cols = q_cols + BT_BYTES;
+    asm volatile("" : "+v"(q_cols), "+v"(do_cols));
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt) {
+        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(do_cols, 2 * sub + k2, dt), pb[k2],
+                                                            dvacc[dt], 0, 0, 0);
+        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(q_cols, 2 * sub + k2, dt), dsb[k2],
+                                                            dkacc[dt], 0, 0, 0);
+      }
+  };
+
+  f32x16 s0, dp0, s1, dp1;
+  scores(0, 0, s0, dp0);
+  int buf = 0;  // it % 3
+  for (int it = 0; it < niter; ++it) {
+    const int nxt = buf == 2 ? 0 : buf + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
+    if (it + 2 < niter) stage_request(it + 2, nxt2);
+    const int q0 = (qt_first + it * qsplit + part) * 64;
+    scores(buf, 1, s1, dp1);
+    consume(buf, 0, q0, s0, dp0);
+    scores(nxt, 0, s0, dp0);  // first block of the next tile (after the last tile: unused)
+    consume(buf, 1, q0 + 32, s1, dp1);
+    if (it + 2 < niter) stage_publish(nxt2);
     __syncthreads();
+    buf = nxt;
   }
 
   // the loop ended with a barrier: the staging buffers are free for the output transposition
@@ -938,7 +959,7 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   const int qsplit = dkdv_query_split(s, b, nq);
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
-  constexpr size_t lds_dkdv = 2 * (2 * BT_BYTES + 512);  // two stages: Q tile, dO tile, statistics
+  constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512);  // three stages: Q tile, dO tile, statistics
   constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
