@@ -155,14 +155,11 @@ static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
 //      dQ^T += K^T.dS^T with the K tile read back transposed.
 //   Recomputing S and dP in both passes costs 7 instead of 5 tile products but keeps every
 //   accumulator in registers and every output written exactly once.
-// LDS tiles that are read both ways ([rows][128] bf16, 256-byte rows, no padding) use an XOR
-// swizzle of the 16-byte chunk index, chunk ^= ((row & 7) << 1) | ((row >> 3) & 1): 8
-// consecutive rows land in 8 different 32-byte bank groups for the vector reads, and the 4x64-
-// byte footprint of a transposing read spreads over all banks as well.
+// Every K / V / Q / dO tile is staged straight from global memory into a blocked LDS tile that
+// can be read both ways (as rows and transposed) without bank conflicts; see bt_request below.
 // =============================================================================================
 namespace {
 
-constexpr int TILE_ELEMS = 64 * HD;  // one swizzled [64][128] tile
 
 // query-like tensors: head h of KV group g = h / per sits at g*g_ + (h % per)*h_
 struct QLayout {
@@ -175,49 +172,6 @@ struct KLayout {
   int64_t s_, b_, h_;
   __device__ __forceinline__ int64_t at(int bi, int kvh) const { return (int64_t)bi * b_ + kvh * h_; }
 };
-
-__device__ __forceinline__ int swz_off(int row, int col) {
-  const int f = ((row & 7) << 1) | ((row >> 3) & 1);
-  return row * HD + ((((col >> 3) ^ f)) << 3) + (col & 7);
-}
-
-// [64][128] tile, global rows row0.. -> swizzled LDS; 256 threads, 4 chunks each
-struct TileStager {
-  bf16x8 r[4];
-  __device__ __forceinline__ void load(const bf16* __restrict__ base, int64_t ss, int row0, int tid) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * 256;
-      r[i] = ldg8(base + (int64_t)(row0 + (c >> 4)) * ss + (c & 15) * 8);
-    }
-  }
-  __device__ __forceinline__ void store(bf16* tile, int tid) const {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + i * 256;
-      *reinterpret_cast<bf16x8*>(tile + swz_off(c >> 4, (c & 15) * 8)) = r[i];
-    }
-  }
-};
-
-// row-major fragment: lane gets tile row (row0 + lane%32), columns 16*kk + 8*(lane/32) + 0..7
-__device__ __forceinline__ bf16x8 read_rows_swz(const bf16* tile, int row0, int kk, int lane) {
-  return *reinterpret_cast<const bf16x8*>(tile + swz_off(row0 + (lane & 31), kk * 16 + (lane >> 5) * 8));
-}
-
-// transposed fragment: lane gets tile column (d0 + lane%32), rows {r0+4h+0..3, r0+8+4h+0..3}
-__device__ __forceinline__ bf16x8 read_cols_swz(const bf16* tile, int r0, int d0, int lane) {
-  const int p = lane & 15;
-  const int row = r0 + 4 * (lane >> 5) + (p >> 2);
-  const int col = d0 + ((lane >> 4) & 1) * 16 + (p & 3) * 4;
-  union {
-    struct { s16x4 lo, hi; } s;
-    bf16x8 v;
-  } u;
-  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row, col)));
-  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(tile + swz_off(row + 8, col)));
-  return u.v;
-}
 
 // ---- direct global -> LDS loads (see the GEMM for why they are written as inline assembly:
 // the compiler must not know of them, or it drains them in front of every barrier).  The 64
@@ -775,10 +729,11 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
     KLayout kl, KLayout vl, QLayout dol, QLayout dql) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  constexpr int STAGE = 2 * TILE_ELEMS;  // K tile | V tile, both swizzled [64][128]
+  constexpr uint32_t STAGE = 2 * BT_BYTES;  // K tile | V tile (blocked tiles), bytes
 
-  const int half = HALVES == 1 ? 0 : (int)(threadIdx.x >> 8);
-  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+  const int half = HALVES == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+  const int tid = threadIdx.x & 255, lane = tid & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nqt = s / BQ;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int qt = nqt - 1 - (lid % nqt);
@@ -811,24 +766,27 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     for (int e = 0; e < 16; ++e) dqacc[dt][e] = 0.f;
 
   const int ntiles = (q0 + BQ) / (HALVES * BKV);  // key tiles per half (the tile count is even)
-  bf16* const area = smem + half * 2 * STAGE;
-  TileStager sk, sv;
-  sk.load(kb, kl.s_, half * BKV, tid);
-  sv.load(vb, vl.s_, half * BKV, tid);
-  sk.store(area, tid);
-  sv.store(area + TILE_ELEMS, tid);
+  // K and V tiles go straight from global memory into this half's two LDS stages
+  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + half * 2 * STAGE;
+  auto stage_request = [&](int j, int buf) {
+    const int key0 = (HALVES * j + half) * BKV;
+    bt_request(kb + (int64_t)key0 * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
+    bt_request(vb + (int64_t)key0 * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
+  };
+  stage_request(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
   for (int j = 0; j < ntiles; ++j) {
     const int cur = j & 1;
-    if (j + 1 < ntiles) {
-      sk.load(kb, kl.s_, (HALVES * (j + 1) + half) * BKV, tid);
-      sv.load(vb, vl.s_, (HALVES * (j + 1) + half) * BKV, tid);
-    }
+    if (j + 1 < ntiles) stage_request(j + 1, cur ^ 1);
     const int key0 = (HALVES * j + half) * BKV;
     if (key0 <= qw0 + 31) {
-      const bf16* ktile = area + cur * STAGE;
-      const bf16* vtile = ktile + TILE_ELEMS;
+      // one base register per tile and read direction; everything else is an immediate
+      uint32_t k_rows = area + cur * STAGE + bt_rows_lane(lane);
+      uint32_t v_rows = k_rows + BT_BYTES;
+      uint32_t k_cols = area + cur * STAGE + bt_cols_lane(lane);
+      asm volatile("" : "+v"(k_rows), "+v"(v_rows), "+v"(k_cols));
       const bool need_mask = key0 + BKV - 1 > qw0;  // wave-uniform: the tile on the diagonal
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -840,10 +798,8 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
         }
 #pragma unroll
         for (int kk = 0; kk < HD / 16; ++kk) {
-          const bf16x8 kfr = read_rows_swz(ktile, t * 32, kk, lane);
-          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[kk], sacc, 0, 0, 0);
-          const bf16x8 vfr = read_rows_swz(vtile, t * 32, kk, lane);
-          dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dpacc, 0, 0, 0);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(k_rows, t, kk), qf[kk], sacc, 0, 0, 0);
+          dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(v_rows, t, kk), dof[kk], dpacc, 0, 0, 0);
         }
         // lane: query row qrow, keys key0 + 32t + 8g + 4h + e
         bf16x8 dsb[2];
@@ -863,15 +819,12 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
         for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
           for (int dt = 0; dt < HD / 32; ++dt) {
-            const bf16x8 ktr = read_cols_swz(ktile, t * 32 + k2 * 16, dt * 32, lane);
-            dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktr, dsb[k2], dqacc[dt], 0, 0, 0);
+            dqacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(k_cols, 2 * t + k2, dt), dsb[k2],
+                                                                dqacc[dt], 0, 0, 0);
           }
       }
     }
-    if (j + 1 < ntiles) {
-      sk.store(area + (cur ^ 1) * STAGE, tid);
-      sv.store(area + (cur ^ 1) * STAGE + TILE_ELEMS, tid);
-    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of the next tiles has landed
     __syncthreads();
   }
 
@@ -960,7 +913,7 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
   constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512);  // three stages: Q tile, dO tile, statistics
-  constexpr size_t lds_dq = 2 * (2 * TILE_ELEMS) * sizeof(bf16);
+  constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
