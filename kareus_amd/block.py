@@ -300,7 +300,14 @@ class LayerStack(torch.nn.Module):
         return params
 
     def rotary_pos_emb(self, seq_len: int, device=None) -> torch.Tensor:
-        return rotary_frequencies(seq_len, self.config.kv_channels, self.config.rotary_base, device=device)
+        """The fp32 rotary table [s, 1, 1, hd]; built once per (length, device) and kept."""
+        key = (seq_len, str(device))
+        cache = self.__dict__.setdefault("_rotary_cache", {})
+        if key not in cache:
+            cache.clear()  # one table at a time is enough: the sequence length rarely changes
+            cache[key] = rotary_frequencies(seq_len, self.config.kv_channels, self.config.rotary_base,
+                                            device=device)
+        return cache[key]
 
     # -- execution ----------------------------------------------------------------
     def forward(self, hidden_states: torch.Tensor, attention_mask=None, rotary_pos_emb=None,
