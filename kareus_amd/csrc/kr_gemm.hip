@@ -493,7 +493,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
     };
+    // Global addresses are a wave-uniform block base plus a 32-bit lane offset (row 8q + rrow
+    // of the block, this lane's chunk): four offset registers serve every access of the tile.
+    const bool rows_in = m_wave + TM * 32 <= M;  // wave-uniform: no row of the wave tile is cut off
     if (out_partial == nullptr && !accumulate) {
+      uint32_t lo[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * ldc + 8 * rch);
+      const bool cols_in = n_wave + 8 * rch < N;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -506,49 +513,86 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
             *reinterpret_cast<bf16x4*>(stage + wr + (((4 * j + g) ^ wsw) << 4) + 8 * h) = o;
           }
         wave_sync();
+        bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int rr = 8 * q + rrow;
           const bf16x8 v =
               *reinterpret_cast<const bf16x8*>(stage + rr * 128 + ((rch ^ ((rr >> 1) & 7)) << 4));
-          const int m = m_wave + i * 32 + rr, n = n_wave + 8 * rch;
-          if (m < M && n < N) stg8(C + (int64_t)m * ldc + n, v);
+          if (cols_in && (rows_in || m_wave + i * 32 + rr < M)) stg8(cb + lo[q], v);
         }
         wave_sync();
       }
     } else {
+      // fp32 staging, one 32 x 32 block per pass; `emit(i, j, q, v)` gets four consecutive
+      // columns of row 8q + rrow of block (i, j)
+      auto fp32_passes = [&](auto&& before_block_row, auto&& emit) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+          before_block_row(i);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+          for (int j = 0; j < TN; ++j) {
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            f32x4 pv;
+            for (int g = 0; g < 4; ++g) {
+              f32x4 pv;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
-            *reinterpret_cast<f32x4*>(stage + wr + (((2 * g + h) ^ wsw) << 4)) = pv;
+              for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
+              *reinterpret_cast<f32x4*>(stage + wr + (((2 * g + h) ^ wsw) << 4)) = pv;
+            }
+            wave_sync();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int rr = 8 * q + rrow;
+              const f32x4 v = *reinterpret_cast<const f32x4*>(stage + rr * 128 +
+                                                              ((rch ^ ((rr >> 1) & 7)) << 4));
+              emit(i, j, q, v);
+            }
+            wave_sync();
           }
-          wave_sync();
+        }
+      };
+      if (out_partial != nullptr) {
+        uint32_t lo[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int rr = 8 * q + rrow;
-            const f32x4 v =
-                *reinterpret_cast<const f32x4*>(stage + rr * 128 + ((rch ^ ((rr >> 1) & 7)) << 4));
-            const int m = m_wave + i * 32 + rr, n = n_wave + j * 32 + 4 * rch;
-            if (m >= M || n >= N) continue;
-            if (out_partial != nullptr) {
-              *reinterpret_cast<f32x4*>(out_partial + (int64_t)m * N + n) = v;
-            } else {
-              bf16* dst = C + (int64_t)m * ldc + n;
-              const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
-              bf16x4 o;
+        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * N + 4 * rch);
+        fp32_passes([](int) {},
+                    [&](int i, int j, int q, const f32x4& v) {
+                      float* const pb = out_partial + ((int64_t)(m_wave + i * 32) * N + n_wave + j * 32);
+                      if (n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M))
+                        *reinterpret_cast<f32x4*>(pb + lo[q]) = v;
+                    });
+      } else {
+        // accumulation into C: the old values of a 32-row block (the same row segments the
+        // results go to) are requested one block ahead of the passes that use them, so their
+        // memory latency is paid once per tile, not once per pass.  Positions beyond the matrix
+        // read a valid neighbour instead and are never stored back.
+        uint32_t lo[4];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)old[e]);
-              *reinterpret_cast<bf16x4*>(dst) = o;
+        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * ldc + 4 * rch);
+        bf16x4 oldc[2][TN][4];
+        auto fetch_old = [&](int i) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave + j * 32);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const bool in = n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M);
+              oldc[i & 1][j][q] = *reinterpret_cast<const bf16x4*>(in ? cb + lo[q] : C);
             }
           }
-          wave_sync();
-        }
+        };
+        fetch_old(0);
+        fp32_passes([&](int i) { if (i + 1 < TM) fetch_old(i + 1); },
+                    [&](int i, int j, int q, const f32x4& v) {
+                      bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave + j * 32);
+                      if (n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M)) {
+                        bf16x4 o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[i & 1][j][q][e]);
+                        *reinterpret_cast<bf16x4*>(cb + lo[q]) = o;
+                      }
+                    });
+      }
     }
   }
   if (!more) break;
@@ -708,7 +752,9 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   if ((M | N | K) % 8 || (lda | ldb | ldc) % 8) return KR_EUNSUPPORTED;
   // chunk offsets inside an operand are kept in 32 bits
   const int64_t a_rows = layout == KR_GEMM_NT ? 64 : M, b_rows = layout == KR_GEMM_TN ? N : 64;
-  if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31 || ldc >= (int64_t)1 << 31)
+  // ... and so are the offsets of the 32 rows of an output block from the block's first element
+  if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31 || ldc >= (int64_t)1 << 26 ||
+      N >= 1 << 26)
     return KR_EUNSUPPORTED;
   const bf16* a = (const bf16*)A;
   const bf16* b = (const bf16*)B;
