@@ -431,12 +431,14 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
           for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
       }
     }
-    // what was requested one step ago (K(j+1), V(j)) is read in the next matrix period; the
-    // requests of this period (at most 8 per wave, retired in order) may stay in flight
-    if (j + 1 < nsteps)
-      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+    // what was requested one step ago (K(j+1), V(j)) is read in the next matrix period; exactly
+    // the requests of this period (4 per tile and wave, retired in order) may stay in flight
+    if (j + 2 < nsteps)
+      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): K(j+2) and V(j+1) were requested
+    else if (j + 1 < nsteps)
+      __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only V(j+1)
     else
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing is requested any more
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing was requested
     __syncthreads();
   }
   // last matrix period: the product of the final tile
