@@ -183,6 +183,14 @@ __device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, ui
                : "memory", "m0");
 }
 
+// 4 bytes per lane: lane p lands at lds_byte + 4 p
+__device__ __forceinline__ void dma_b32(const void* base, uint32_t byte_off, uint32_t lds_byte) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_byte), "v"(byte_off), "s"(base)
+               : "memory", "m0");
+}
+
 // ---- blocked LDS tile: [64 rows][128 channels] bf16, filled straight from global memory ------
 // A tile is 16 blocks; block B holds rows r, r+16, r+32, r+48 (r = 4 (B % 4) + B / 4), 256 bytes
 // each, in the order one wave-wide request delivers them (lane p at +16 p: row r + 16 (p / 16),
@@ -492,7 +500,9 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
 
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ dout,
                                                          const bf16* __restrict__ o,
-                                                         float* __restrict__ delta, int s, int nq,
+                                                         const float* __restrict__ lse,
+                                                         float* __restrict__ delta,
+                                                         float* __restrict__ neg_lse2, int s, int nq,
                                                          int per, int64_t total_rows, QLayout dol,
                                                          QLayout ol) {
   // 16 lanes per (batch, head, position) row of 128 channels
@@ -509,14 +519,19 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
   for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) acc += __shfl_xor(acc, off, KR_WAVE);
-  if (sub == 0) delta[row] = acc;
+  if (sub == 0) {
+    delta[row] = acc;
+    // -lse in the log2 domain, so that the dK/dV kernel's exponent is one multiply-add and its
+    // row statistics can go straight from global memory into LDS
+    neg_lse2[row] = -lse[row] * kLog2e;
+  }
 }
 
 // PARTIAL = true: fp32 results for this query head go to part_k / part_v [b, nq, s, 128]
 template <bool PARTIAL>
 __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
-    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    const bf16* __restrict__ dout, const float* __restrict__ neg_lse2, const float* __restrict__ delta,
     bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
     float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, float scale, float scale_log2,
     QLayout ql,
@@ -564,42 +579,55 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   const bf16* qb = q + ql.at(bi, head, per);
   const bf16* dob = dout + dol.at(bi, head, per);
   const int64_t stat0 = ((int64_t)bi * nq + head) * s;
-  float st_stat = 0.f;  // threads 0..63 carry lse, 64..127 carry delta of the tile being staged
   const uint32_t lds0 = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
 
   // Q and dO tiles go straight from global memory into LDS; the row statistics pass through a
-  // register of the first 128 threads
-  auto stage_request = [&](int it, int buf) {
-    const int qt = qt_first + it * qsplit + part;
-    bt_request(qb + (int64_t)qt * 64 * ql.s_, ql.s_, lds0 + buf * STAGE, wave, lane);
-    bt_request(dob + (int64_t)qt * 64 * dol.s_, dol.s_, lds0 + buf * STAGE + BT_BYTES, wave, lane);
-    if (tid < 64) st_stat = -lse[stat0 + qt * 64 + tid] * kLog2e;  // negated: the exponent is one fma
-    else if (tid < 128) st_stat = delta[stat0 + qt * 64 + tid - 64];
+  // register of the first 128 threads.  A wave's share of a stage is eight 1-KiB requests
+  // (blocks wave + 4 i of the Q tile, then of the dO tile); request_one(i) issues one of them.
+  int req_qt = 0;
+  uint32_t req_tile = 0;
+  auto request_begin = [&](int it, int stage) {
+    req_qt = qt_first + it * qsplit + part;
+    req_tile = lds0 + stage * STAGE;
+    // the tile's 64 + 64 row statistics: one 4-byte-per-lane request each, by waves 0 and 1
+    if (wave < 2) {
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));
+      dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + req_qt * 64, (uint32_t)l2 * 4u,
+              req_tile + 2 * BT_BYTES + wave * 256);
+    }
   };
-  auto stage_publish = [&](int buf) {
-    float* stats = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + buf * STAGE + 2 * BT_BYTES);
-    if (tid < 128) stats[tid] = st_stat;
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of both tiles has landed
+  auto request_one = [&](int i) {
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
+    const bool second = i >= 4;
+    const bf16* rows = second ? dob + (int64_t)req_qt * 64 * dol.s_ : qb + (int64_t)req_qt * 64 * ql.s_;
+    const int64_t ss = second ? dol.s_ : ql.s_;
+    const int blk = wave + 4 * (i & 3);
+    const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+    dma_b128(rows + (int64_t)(4 * (blk & 3) + (blk >> 2)) * ss, lane_off,
+             req_tile + (second ? BT_BYTES : 0) + blk * BT_BLK);
   };
-
-  // Three stages: while tile `it` is consumed, tile it+1 is already complete (its first score
-  // block is computed one step ahead, see below) and tile it+2 is on its way.
-  stage_request(0, 0);
-  stage_publish(0);
-  if (niter > 1) {
-    stage_request(1, 1);
-    stage_publish(1);
+  // Four stages: while tile `it` is consumed, tile it+1 is already complete (its first score
+  // block is computed one step ahead, see below), tiles it+2 and it+3 are on their way.
+  for (int p = 0; p < 3 && p < niter; ++p) {
+    request_begin(p, p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) request_one(i);
   }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
   // The wave runs alone on its SIMD, so the overlap of matrix and vector work has to come from
   // inside it: the two score products of a 32-query block (S = Q.K^T, dP = dO.V^T) are issued
   // one block ahead of the exponentials that consume them, and execute while the vector ALU
-  // works on the previous block.  Blocks that lie wholly before the wave's keys are not
-  // skipped but masked to zero (there are at most three per wave): the loop body stays
-  // straight-line code and the accumulators stay where they are.
-  auto scores = [&](int buf, int sub, f32x16& sacc, f32x16& dpacc) {
-    uint32_t q_rows = lds0 + buf * STAGE + bt_rows_lane(lane);
+  // works on the previous block; the requests for a later tile are issued one at a time between
+  // those MFMAs (the texture-address path takes ~64 cycles per request and would otherwise
+  // stall the wave for 500 cycles with the matrix pipe idle).  Blocks that lie wholly before
+  // the wave's keys are not skipped but masked to zero (there are at most three per wave): the
+  // loop body stays straight-line code and the accumulators stay where they are.
+  auto scores = [&](int stage, int sub, f32x16& sacc, f32x16& dpacc, bool with_requests) {
+    uint32_t q_rows = lds0 + stage * STAGE + bt_rows_lane(lane);
     uint32_t do_rows = q_rows + BT_BYTES;
     asm volatile("" : "+v"(q_rows), "+v"(do_rows));  // one base register each; the rest are immediates
 #pragma unroll
@@ -607,16 +635,43 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
       sacc[e] = 0.f;
       dpacc[e] = 0.f;
     }
+    // all sixteen fragments are requested before the first MFMA (registers are plentiful at one
+    // wave per SIMD)
+    bf16x8 qfr[HD / 16], dofr[HD / 16];
 #pragma unroll
     for (int kk = 0; kk < HD / 16; ++kk) {
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(q_rows, sub, kk), kf[kk], sacc, 0, 0, 0);
-      dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_rows(do_rows, sub, kk), vf[kk], dpacc, 0, 0, 0);
+      qfr[kk] = bt_rows(q_rows, sub, kk);
+      dofr[kk] = bt_rows(do_rows, sub, kk);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], sacc, 0, 0, 0);
+      dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[kk], vf[kk], dpacc, 0, 0, 0);
+      if (with_requests) {
+        request_one(kk);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
   // P = exp2(S c - lse), dS = P (dP - delta); then dV^T += dO^T . P and dK^T += Q^T . dS
-  auto consume = [&](int buf, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
+  auto consume = [&](int stage, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
     const float* stats =
-        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + buf * STAGE + 2 * BT_BYTES);
+        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + stage * STAGE + 2 * BT_BYTES);
+    // the transposed fragments of the two products at the end are requested first and arrive
+    // while the vector ALU does the exponentials
+    uint32_t q_cols = lds0 + stage * STAGE + bt_cols_lane(lane);
+    uint32_t do_cols = q_cols + BT_BYTES;
+    asm volatile("" : "+v"(q_cols), "+v"(do_cols));
+    bf16x8 dot[2][HD / 32], qtr[2][HD / 32];
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt) {
+        dot[k2][dt] = bt_cols(do_cols, 2 * sub + k2, dt);
+        qtr[k2][dt] = bt_cols(q_cols, 2 * sub + k2, dt);
+      }
+    __builtin_amdgcn_sched_barrier(0);
     // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that reach the diagonal
     // pay for the causal mask (wave-uniform branch)
     if (qs0 < kw0 + 31) {
@@ -639,34 +694,35 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
         dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
       }
     }
-    uint32_t q_cols = lds0 + buf * STAGE + bt_cols_lane(lane);
-    uint32_t do_cols = q_cols + BT_BYTES;
-    asm volatile("" : "+v"(q_cols), "+v"(do_cols));
+    __builtin_amdgcn_sched_barrier(0);  // the vector work first, then the MFMAs back to back
 #pragma unroll
     for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
       for (int dt = 0; dt < HD / 32; ++dt) {
-        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(do_cols, 2 * sub + k2, dt), pb[k2],
-                                                            dvacc[dt], 0, 0, 0);
-        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bt_cols(q_cols, 2 * sub + k2, dt), dsb[k2],
-                                                            dkacc[dt], 0, 0, 0);
+        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[k2][dt], pb[k2], dvacc[dt], 0, 0, 0);
+        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[k2][dt], dsb[k2], dkacc[dt], 0, 0, 0);
       }
   };
 
   f32x16 s0, dp0, s1, dp1;
-  scores(0, 0, s0, dp0);
-  int buf = 0;  // it % 3
+  scores(0, 0, s0, dp0, false);
   for (int it = 0; it < niter; ++it) {
-    const int nxt = buf == 2 ? 0 : buf + 1, nxt2 = nxt == 2 ? 0 : nxt + 1;
-    if (it + 2 < niter) stage_request(it + 2, nxt2);
+    const int cur = it & 3, nxt = (it + 1) & 3, far = (it + 3) & 3;
+    const bool more = it + 3 < niter;  // tile it+3 goes where tile it-1 was read last
+    if (more) request_begin(it + 3, far);
     const int q0 = (qt_first + it * qsplit + part) * 64;
-    scores(buf, 1, s1, dp1);
-    consume(buf, 0, q0, s0, dp0);
-    scores(nxt, 0, s0, dp0);  // first block of the next tile (after the last tile: unused)
-    consume(buf, 1, q0 + 32, s1, dp1);
-    if (it + 2 < niter) stage_publish(nxt2);
+    scores(cur, 1, s1, dp1, more);
+    consume(cur, 0, q0, s0, dp0);
+    scores(nxt, 0, s0, dp0, false);  // first block of the next tile (after the last tile: unused)
+    consume(cur, 1, q0 + 32, s1, dp1);
+    // tile it+2 (requested an iteration ago) must have landed before the barrier that makes it
+    // readable as `nxt` of the next iteration; this iteration's eight tile requests, issued
+    // after its statistics request, may fly on
+    if (more)
+      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     __syncthreads();
-    buf = nxt;
   }
 
   // the loop ended with a barrier: the staging buffers are free for the output transposition
@@ -877,7 +933,7 @@ static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <=
 
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
   if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
-  size_t bytes = (size_t)b * nq * s * sizeof(float);  // delta
+  size_t bytes = 2 * (size_t)b * nq * s * sizeof(float);  // delta, and -lse in the log2 domain
   const int qsplit = dkdv_query_split(s, b, nq);
   if (nq != nkv || qsplit > 1)  // fp32 dK, dV partials per (query head, query-tile part)
     bytes += 2 * (size_t)b * nq * qsplit * s * hd * sizeof(float);
@@ -910,11 +966,12 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
       dvl{dv_ss, dv_sb, dv_sh};
   float* delta = (float*)workspace;
   const int64_t rows = (int64_t)b * nq * s;
-  float* part_k = delta + rows;
+  float* neg_lse2 = delta + rows;
+  float* part_k = neg_lse2 + rows;
   const int qsplit = dkdv_query_split(s, b, nq);
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
-  constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512);  // three stages: Q tile, dO tile, statistics
+  constexpr size_t lds_dkdv = 4 * (2 * BT_BYTES + 512);  // four stages: Q tile, dO tile, statistics
   constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
@@ -934,14 +991,15 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
 
   const int per = nq / nkv;
   hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
-                     (const bf16*)dout, (const bf16*)o, delta, s, nq, per, rows, dol, ol);
+                     (const bf16*)dout, (const bf16*)o, lse, delta, neg_lse2, s, nq, per, rows, dol, ol);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
   const dim3 grid_kv((s / 128) * nq * b * qsplit);
   if (partial) {
     hipLaunchKernelGGL(attn_bwd_dkdv_kernel<true>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
-                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
-                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, qsplit, scale, scale_log2, ql,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,
+                       (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, qsplit, scale,
+                       scale_log2, ql,
                        kl, vl, dol, dkl, dvl);
     if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
     const int64_t total = (int64_t)b * nkv * s * 16;
@@ -950,8 +1008,8 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
                        nkv, qsplit, total, dkl, dvl);
   } else {
     hipLaunchKernelGGL(attn_bwd_dkdv_kernel<false>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
-                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
-                       (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, 1, scale, scale_log2, ql, kl,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,
+                       (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, 1, scale, scale_log2, ql, kl,
                        vl, dol, dkl, dvl);
   }
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;

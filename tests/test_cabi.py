@@ -46,11 +46,11 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1
     assert lib.kr_gemm_bf16(0, 8, 8, 8, 16, 8, 16, 8, 18, 8, 0, None, 0, None) == -1   # misaligned C
     assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 64) == 0  # head_dim 64 unsupported
-    # delta, plus fp32 dK/dV partials per query head when heads share KV heads ...
-    assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 32, 128) == 4 * 32 * 4096 * 4
-    assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 8, 128) == 4 * 32 * 4096 * 4 + 2 * 4 * 32 * 4096 * 128 * 4
+    # delta and the rescaled lse, plus fp32 dK/dV partials per query head when heads share KV heads ...
+    assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 32, 128) == 2 * 4 * 32 * 4096 * 4
+    assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 8, 128) == 2 * 4 * 32 * 4096 * 4 + 2 * 4 * 32 * 4096 * 128 * 4
     # ... and per (query head, half of the query tiles) when the launch has few workgroups
-    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 4, 128) == 256 * 4 * 4 + 2 * 256 * 4 * 2 * 128 * 4
-    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 128) == 256 * 4 * 4 + 2 * 256 * 4 * 2 * 128 * 4
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 4, 128) == 2 * 256 * 4 * 4 + 2 * 256 * 4 * 2 * 128 * 4
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 128) == 2 * 256 * 4 * 4 + 2 * 256 * 4 * 2 * 128 * 4
     assert lib.kr_gemm_workspace_bytes(2, 1536, 4096, 16384) > 0 and lib.kr_gemm_workspace_bytes(0, 4096, 7168, 4096) == 0
     assert lib.kr_rmsnorm_bwd_workspace_bytes(8192, 4096) == 512 * 4096 * 4
