@@ -108,9 +108,11 @@ def available_frequencies_mhz(device_index: int = 0) -> List[int]:
     return out
 
 
-def set_gpu_frequency(target_freq_mhz: int, device_index: int = 0) -> bool:
+def set_gpu_frequency(target_freq_mhz: int, device_index: int = 0, settle_s: float = 0.5) -> bool:
     """Pin the shader clock to the listed level closest to ``target_freq_mhz``.  Returns False
-    (and changes nothing) when the files are missing or not writable by this user."""
+    (and changes nothing) when the files are missing or not writable by this user.  ``settle_s``:
+    pause after the write (a measurement wants the clock settled, a per-instruction switch in
+    a training loop passes 0)."""
     d = _device_dir(device_index)
     levels = available_frequencies_mhz(device_index)
     if d is None or not levels:
@@ -123,7 +125,8 @@ def set_gpu_frequency(target_freq_mhz: int, device_index: int = 0) -> bool:
             f.write(str(level))
     except OSError:
         return False
-    time.sleep(0.5)
+    if settle_s > 0:
+        time.sleep(settle_s)
     return True
 
 

@@ -6,6 +6,7 @@ from .parser import (
     parse_schedule_file,
 )
 from .pipeline_comm_scheduler import PipelineCommScheduler
+from .pipeline_frequency_scheduler import PipelineFrequencyScheduler
 
 __all__ = [
     "CommConfig",
@@ -14,4 +15,5 @@ __all__ = [
     "parse_schedule_file",
     "parse_frequency_file",
     "PipelineCommScheduler",
+    "PipelineFrequencyScheduler",
 ]

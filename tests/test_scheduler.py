@@ -60,6 +60,59 @@ def test_shipped_frequency_plan(fixtures_dir):
         assert [n for n, _ in st_f] == ["backward" if it.bwd_mlp is not None else "forward" for it in st_s]
 
 
+def test_frequency_plan_is_stepped_and_applied(fixtures_dir):
+    """The frequency plan of a stage drives the same four hooks as the communication schedule:
+    one (instruction, MHz) per instruction, the clock switched only when the value changes, the
+    instruction kind checked, the plan drained at step end."""
+    from kareus_amd.scheduler import PipelineFrequencyScheduler
+
+    path = os.path.join(fixtures_dir, "freqs_pipeline_02328.py")
+    plan = parse_frequency_file(path)[0]
+    calls = []
+    sch = PipelineFrequencyScheduler(path, pp_rank=0, num_instructions=16,
+                                     set_frequency=lambda mhz: (calls.append(mhz), True)[1],
+                                     reset_frequency=lambda: True)
+    for _ in range(2):                       # two steps: the plan restarts, the clock is remembered
+        sch.on_step_begin()
+        for name, _mhz in plan:
+            sch.on_instruction_begin(name)
+            sch.on_instruction_end(name)
+        sch.on_step_end()
+        assert [(n, f) for n, f, _ in sch.history] == plan and all(a for _, _, a in sch.history)
+    changes = [mhz for i, (_, mhz) in enumerate(plan + plan) if i == 0 or mhz != (plan + plan)[i - 1][1]]
+    assert calls == changes and sch.current_frequency == plan[-1][1]
+    assert sch.release() and sch.current_frequency is None
+    # a setter that is refused (an ordinary user may not write the clock files) is recorded, not fatal
+    denied = PipelineFrequencyScheduler(path, pp_rank=1, set_frequency=lambda mhz: False, reset_frequency=lambda: False)
+    denied.on_step_begin()
+    denied.on_instruction_begin("forward")
+    assert denied.history == [("forward", parse_frequency_file(path)[1][0][1], False)] and not denied.applied
+    # wrong instruction kind, plan overrun, plan not drained, bad arguments
+    with pytest.raises(RuntimeError, match="mismatch"):
+        denied.on_instruction_begin("forward" if parse_frequency_file(path)[1][1][0] == "backward" else "backward")
+    sch.on_step_begin()
+    sch.on_instruction_begin("forward")
+    with pytest.raises(RuntimeError, match="more entries"):
+        sch.on_step_end()
+    sch.on_step_begin()
+    for name, _ in plan:
+        sch.on_instruction_begin(name)
+    with pytest.raises(RuntimeError, match="No more planned"):
+        sch.on_instruction_begin("forward")
+    with pytest.raises(IndexError):
+        PipelineFrequencyScheduler(path, pp_rank=2)
+    with pytest.raises(ValueError, match="does not match"):
+        PipelineFrequencyScheduler(path, pp_rank=0, num_instructions=8)
+    with pytest.raises(FileNotFoundError):
+        PipelineFrequencyScheduler(os.path.join(fixtures_dir, "missing.py"), pp_rank=0)
+    # the default setter goes through sysfs; without a GPU (or without write access) it reports False
+    default = PipelineFrequencyScheduler(path, pp_rank=0)
+    default.on_step_begin()
+    default.on_instruction_begin("forward")
+    assert default.history[0][:2] == plan[0] and default.history[0][2] in (False, True)
+    default.release()   # hands the clock back if the write was allowed
+
+
 def test_other_grammars(fixtures_dir, tmp_path):
     ac = parse_schedule_file(os.path.join(fixtures_dir, "single_stage_ac.py"), True, False)
     assert len(ac) == 1 and len(ac[0]) == 4
