@@ -199,16 +199,19 @@ __device__ __forceinline__ void dma_b32(const void* base, uint32_t byte_off, uin
 // fragment address is one per-lane base plus an instruction immediate.
 constexpr uint32_t BT_BLK = 1024 + 16, BT_BYTES = 16 * BT_BLK;
 
-// the four waves of a group bring in one tile (rows = its first row in global memory)
+// The four waves (wave = 0..3) of a group bring in one tile; `rows` = its first row in global
+// memory.  Wave w fills blocks w, w + 4, w + 8, w + 12, which hold the tile rows 4 w + 0..3
+// (+ 16, 32, 48): four consecutive rows, so a request costs one pointer increment.
 __device__ __forceinline__ void bt_request(const bf16* rows, int64_t ss, uint32_t tile, int wave,
                                            int lane) {
   int l2 = lane;
   asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
   const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+  const bf16* row = rows + (int64_t)(4 * wave) * ss;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int blk = wave + 4 * i;
-    dma_b128(rows + (int64_t)(4 * (blk & 3) + (blk >> 2)) * ss, lane_off, tile + blk * BT_BLK);
+    dma_b128(row, lane_off, tile + (wave + 4 * i) * BT_BLK);
+    row += ss;
   }
 }
 // row-major fragments: lane gets row 32 t + lane % 32, channels 16 kk + 8 (lane / 32) + 0..7
@@ -302,21 +305,36 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
   const uint32_t vfrag_lane = (uint32_t)((4 * h + ((lane & 15) >> 2)) * VBLK + ((lane >> 4) & 1) * 32 +
                                          ((lane & 3) >> 1) * 16 + (lane & 1) * 8);
 
-  // one wave requests 4 KiB of a tile: blocks wave + 4 i
-  auto request = [&](const bf16* base, int64_t ss, int j, uint32_t tile, uint32_t blk_bytes) {
-    int l2 = lane;
-    asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
-    const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+  // One wave requests 4 KiB of a tile: blocks wave + 4 i, i.e. tile rows wave + 4 i (+ 16, 32,
+  // 48).  Everything a request needs is kept ready — a pointer to row `wave` of the next tile to
+  // ask for, advanced by two tiles per step, the distance of four rows, the lane's byte offset —
+  // so that a request costs a handful of scalar instructions: the vector period is bound by the
+  // number of instructions the wave has to issue.
+  const bf16* kreq = kb + (int64_t)(key_of(0) + wave) * k_ss;
+  const bf16* vreq = vb + (int64_t)(key_of(0) + wave) * v_ss;
+  const int64_t k_tiles2 = (int64_t)2 * BKV * k_ss, v_tiles2 = (int64_t)2 * BKV * v_ss;
+  const int64_t k_rows4 = 4 * k_ss, v_rows4 = 4 * v_ss;
+  const uint32_t k_lane_off = (uint32_t)((lane >> 4) * 16 * (int)k_ss + (lane & 15) * 8) * 2u;
+  const uint32_t v_lane_off = (uint32_t)((lane >> 4) * 16 * (int)v_ss + (lane & 15) * 8) * 2u;
+  auto request = [&](const bf16* row, int64_t rows4, uint32_t lane_off, uint32_t tile, uint32_t blk_bytes) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int blk = wave + 4 * i;
-      dma_b128(base + (int64_t)(key_of(j) + blk) * ss, lane_off, tile + blk * blk_bytes);
+      dma_b128(row, lane_off, tile + (wave + 4 * i) * blk_bytes);
+      row += rows4;
     }
   };
+  auto request_k = [&](uint32_t tile) {
+    request(kreq, k_rows4, k_lane_off, tile, KBLK);
+    kreq += k_tiles2;
+  };
+  auto request_v = [&](uint32_t tile) {
+    request(vreq, v_rows4, v_lane_off, tile, VBLK);
+    vreq += v_tiles2;
+  };
 
-  request(kb, k_ss, 0, kbuf, KBLK);
-  if (nsteps > 1) request(kb, k_ss, 1, kbuf + KTILE, KBLK);
-  request(vb, v_ss, 0, vbuf, VBLK);
+  request_k(kbuf);
+  if (nsteps > 1) request_k(kbuf + KTILE);
+  request_v(vbuf);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
   if (half == 1) __syncthreads();  // half 1 starts one period late
@@ -394,8 +412,8 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
 
     // ---- vector period of tile j: request K(j+2) and V(j+1) (their buffers were last read in
     // the matrix period that just ended), then the softmax
-    if (j + 2 < nsteps) request(kb, k_ss, j + 2, kbuf + (j & 1) * KTILE, KBLK);
-    if (j + 1 < nsteps) request(vb, v_ss, j + 1, vbuf + ((j + 1) & 1) * VTILE, VBLK);
+    if (j + 2 < nsteps) request_k(kbuf + (j & 1) * KTILE);
+    if (j + 1 < nsteps) request_v(vbuf + ((j + 1) & 1) * VTILE);
     {
       const int key0 = key_of(j);
       if (key0 + BKV - 1 > qw0) {
@@ -584,11 +602,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   // Q and dO tiles go straight from global memory into LDS; the row statistics pass through a
   // register of the first 128 threads.  A wave's share of a stage is eight 1-KiB requests
   // (blocks wave + 4 i of the Q tile, then of the dO tile); request_one(i) issues one of them.
-  int req_qt = 0;
-  uint32_t req_tile = 0;
+  // request_begin(it, stage) prepares tile `it`: pointers to the four consecutive rows this wave
+  // fetches of the Q and of the dO tile (rows 4 wave + 0..3, + 16, 32, 48 through the lanes).
+  uint32_t req_tile = 0, req_lane_off = 0;
+  const bf16* req_q = nullptr;
+  const bf16* req_do = nullptr;
+  const bf16* req_row = nullptr;
   auto request_begin = [&](int it, int stage) {
-    req_qt = qt_first + it * qsplit + part;
+    const int req_qt = qt_first + it * qsplit + part;
     req_tile = lds0 + stage * STAGE;
+    req_q = qb + ((int64_t)req_qt * 64 + 4 * wave) * ql.s_;
+    req_do = dob + ((int64_t)req_qt * 64 + 4 * wave) * dol.s_;
     // the tile's 64 + 64 row statistics: one 4-byte-per-lane request each, by waves 0 and 1
     if (wave < 2) {
       int l2 = lane;
@@ -597,16 +621,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
               req_tile + 2 * BT_BYTES + wave * 256);
     }
   };
+  // requests 0..3: the Q tile, 4..7: the dO tile; issued in this order
   auto request_one = [&](int i) {
-    int l2 = lane;
-    asm volatile("" : "+v"(l2));  // nothing derived from it is kept alive between requests
     const bool second = i >= 4;
-    const bf16* rows = second ? dob + (int64_t)req_qt * 64 * dol.s_ : qb + (int64_t)req_qt * 64 * ql.s_;
-    const int64_t ss = second ? dol.s_ : ql.s_;
-    const int blk = wave + 4 * (i & 3);
-    const uint32_t lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
-    dma_b128(rows + (int64_t)(4 * (blk & 3) + (blk >> 2)) * ss, lane_off,
-             req_tile + (second ? BT_BYTES : 0) + blk * BT_BLK);
+    if ((i & 3) == 0) {
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));  // the lane offset lives only across the four requests of a tile
+      const int ss = (int)(second ? dol.s_ : ql.s_);
+      req_lane_off = (uint32_t)((l2 >> 4) * 16 * ss + (l2 & 15) * 8) * 2u;
+      req_row = second ? req_do : req_q;
+    }
+    dma_b128(req_row, req_lane_off, req_tile + (second ? BT_BYTES : 0) + (wave + 4 * (i & 3)) * BT_BLK);
+    req_row += second ? dol.s_ : ql.s_;
   };
   // Four stages: while tile `it` is consumed, tile it+1 is already complete (its first score
   // block is computed one step ahead, see below), tiles it+2 and it+3 are on their way.
