@@ -179,6 +179,58 @@ def copy_calibration(device, n=1 << 29, launches=10):
             "avg_launch_us": sec * 1e6, "achieved_GBps": 6 * n / sec / 1e9}
 
 
+def hbm_kernels(w, nnb, device, launches=50):
+    """Every HBM-bound kernel of the layer alone on the GPU, at the nanobatch shape and at the
+    whole-microbatch shape: average launch time (HIP events on the launch stream) and
+    algorithmic bytes (operands read once, results written once) per second against 8 TB/s."""
+    from kareus_amd.backend import get_backend
+    from kareus_amd.operators.rotary_embedding import rotary_frequencies
+
+    be = get_backend("hip")
+    bf = torch.bfloat16
+    rows_out = []
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / launches
+
+    def report(name, tokens, nbytes, fn):
+        sec = timed(fn)
+        rows_out.append({"kernel": name, "tokens": tokens, "bytes": nbytes, "avg_launch_us": sec * 1e6,
+                         "achieved_TBps": nbytes / sec / 1e12, "frac_of_8TBps": nbytes / sec / HBM_PEAK})
+
+    h, f, hd = w["h"], w["ffn"], w["hd"]
+    heads = w["nq"] + w["nkv"]
+    for t in sorted({(w["b"] // nnb) * w["s"], w["b"] * w["s"]}):
+        x = torch.randn(t, h, device=device, dtype=bf)
+        y = torch.randn(t, h, device=device, dtype=bf)
+        gamma = torch.ones(h, device=device, dtype=bf)
+        report("add_kernel (residual add)", t, 3 * t * h * 2, lambda: be.add(x, y))
+        report("rmsnorm_fwd_kernel", t, 2 * t * h * 2, lambda: be.rmsnorm_fwd(x, gamma, 1e-5))
+        normed, rstd = be.rmsnorm_fwd(x, gamma, 1e-5)
+        report("rmsnorm_bwd_kernel + rmsnorm_dgamma_kernel", t, 3 * t * h * 2,
+               lambda: be.rmsnorm_bwd(y, x, rstd, gamma))
+        report("rmsnorm_bwd_kernel<ADD> (+ residual gradient) + dgamma", t, 4 * t * h * 2,
+               lambda: be.rmsnorm_bwd(y, x, rstd, gamma, residual_grad=normed))
+        u = torch.randn(t, 2 * f, device=device, dtype=bf)
+        dy = torch.randn(t, f, device=device, dtype=bf)
+        report("swiglu_fwd_kernel", t, 3 * t * f * 2, lambda: be.swiglu_fwd(u))
+        report("swiglu_bwd_kernel", t, 5 * t * f * 2, lambda: be.swiglu_bwd(dy, u))
+        s_len = w["s"]
+        qk = torch.randn(s_len, t // s_len, heads, hd, device=device, dtype=bf)
+        freqs = rotary_frequencies(s_len, hd, 500000.0, device=device)
+        report("rope_kernel (q and k heads)", t, 2 * t * heads * hd * 2, lambda: be.rope_fwd(qk, freqs))
+    return rows_out
+
+
 def cpu_baseline(w, budget_s=25.0):
     """The CPU oracle (fp32 PyTorch, autograd backward) on a bounded sample: same layer widths,
     one sequence of at most 1024 tokens, as many iterations as fit the time budget."""
@@ -222,6 +274,8 @@ def main():
                     help="run only the dominant-kernel leg (the command profiled under profiles/)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a residual-add kernel of known size (calibrates FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--hbm-kernels", action="store_true",
+                    help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs one GPU's shard of the layer; --gpus must be 1 "
@@ -239,6 +293,9 @@ def main():
         return
     if args.copy_calibration:
         print(json.dumps({"copy_calibration": copy_calibration(device)}))
+        return
+    if args.hbm_kernels:
+        print(json.dumps({"hbm_kernels": hbm_kernels(w, w["nnb"], device)}))
         return
     gen = torch.Generator().manual_seed(42)
     x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)

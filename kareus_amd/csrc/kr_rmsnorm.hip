@@ -67,7 +67,11 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
 // gradient of the norm is rounded to bf16 exactly as the stand-alone kernel rounds it and then
 // the gradient of the residual branch is added, so the fused result is bit-identical to the
 // two kernels run one after the other while one write and one read of the tensor disappear.
-template <int NCHUNK, bool ADD>
+// FULL: the row is exactly NCHUNK * 64 vectors long (hidden sizes 512 * k).  No lane is ever
+// idle, so the loop body is straight-line code and every load of a row — x, dy and the residual
+// gradient — is issued before the first wait; with per-chunk bounds checks each chunk of the
+// output pass paid its own round trip to memory.
+template <int NCHUNK, bool ADD, bool FULL>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
     const bf16* __restrict__ gamma, const bf16* __restrict__ dres, bf16* __restrict__ dx,
@@ -82,20 +86,25 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
     const int v = lane + c * 64;
-    g[c] = v < nvec ? ldg8(gamma + v * 8) : zero8();
+    g[c] = (FULL || v < nvec) ? ldg8(gamma + v * 8) : zero8();
 #pragma unroll
     for (int e = 0; e < 8; ++e) dg[c][e] = 0.f;
   }
   for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
     const bf16* xr = x + (int64_t)row * x_ld;
     const bf16* dr = dy + (int64_t)row * dy_ld;
+    const bf16* rr = ADD ? dres + (int64_t)row * dres_ld : nullptr;
     const float rs = rstd[row];
-    bf16x8 xv[NCHUNK], dv[NCHUNK];
+    bf16x8 xv[NCHUNK], dv[NCHUNK], rv[ADD && FULL ? NCHUNK : 1];
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int v = lane + c * 64;
-      xv[c] = v < nvec ? ldg8(xr + v * 8) : zero8();
-      dv[c] = v < nvec ? ldg8(dr + v * 8) : zero8();
+      xv[c] = (FULL || v < nvec) ? ldg8(xr + v * 8) : zero8();
+      dv[c] = (FULL || v < nvec) ? ldg8(dr + v * 8) : zero8();
+    }
+    if (ADD && FULL) {
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) rv[c] = ldg8(rr + (lane + c * 64) * 8);
     }
     float dot = 0.f;
 #pragma unroll
@@ -109,13 +118,12 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
       }
     dot = wave_sum(dot) * inv_cols;
     bf16* oxr = dx + (int64_t)row * dx_ld;
-    const bf16* rr = ADD ? dres + (int64_t)row * dres_ld : nullptr;
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int v = lane + c * 64;
-      if (v < nvec) {
+      if (FULL || v < nvec) {
         bf16x8 o, r;
-        if (ADD) r = ldg8(rr + v * 8);
+        if (ADD) r = FULL ? rv[c] : ldg8(rr + v * 8);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float xh = (float)xv[c][e] * rs;
@@ -237,19 +245,20 @@ extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rs
     return KR_EINVAL;
   const int blocks = bwd_blocks(rows);
   const int nc = chunks_for(cols);
+#define KR_RMS_BWD(ADDV, FULLV)                                                                     \
+  KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, ADDV, FULLV>), dim3(blocks),    \
+                                           dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy, \
+                                           (const bf16*)x, rstd, (const bf16*)gamma,                \
+                                           (const bf16*)dres, (bf16*)dx, (float*)workspace, rows,   \
+                                           cols, dy_ld, x_ld, dres ? dres_ld : (int64_t)0, dx_ld))
+  // rows of exactly 1, 2, 3, 4, 6 or 8 times 512 elements take the straight-line kernel
+  const bool full = cols % 512 == 0 && cols / 512 == nc && nc <= 8 && nc != 5 && nc != 7;
   if (dres) {
-    KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, true>), dim3(blocks),
-                                             dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy,
-                                             (const bf16*)x, rstd, (const bf16*)gamma,
-                                             (const bf16*)dres, (bf16*)dx, (float*)workspace, rows,
-                                             cols, dy_ld, x_ld, dres_ld, dx_ld));
+    if (full) { KR_RMS_BWD(true, true); } else { KR_RMS_BWD(true, false); }
   } else {
-    KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, false>), dim3(blocks),
-                                             dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy,
-                                             (const bf16*)x, rstd, (const bf16*)gamma,
-                                             (const bf16*)nullptr, (bf16*)dx, (float*)workspace, rows,
-                                             cols, dy_ld, x_ld, (int64_t)0, dx_ld));
+    if (full) { KR_RMS_BWD(false, true); } else { KR_RMS_BWD(false, false); }
   }
+#undef KR_RMS_BWD
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 31) / 32), dim3(kDgammaThreads), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
