@@ -73,10 +73,18 @@ class HipBackend:
 
     def __init__(self) -> None:
         self.lib = load_library()
+        self._gemm_ws_bytes: dict = {}  # (layout, m, n, k, split_k) -> workspace bytes
 
     # -- plumbing -------------------------------------------------------------------
-    @staticmethod
-    def _stream() -> int:
+    # the raw handle of the current stream without building a torch.cuda.Stream object: this is
+    # asked once per kernel launch
+    _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    _raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+    @classmethod
+    def _stream(cls) -> int:
+        if cls._raw_stream is not None and cls._raw_device is not None:
+            return cls._raw_stream(cls._raw_device())
         return torch.cuda.current_stream().cuda_stream
 
     def _check(self, rc: int, what: str) -> None:
@@ -115,8 +123,12 @@ class HipBackend:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
             out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-        ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
-                    self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
+        key = (layout, m, n, k, split_k)
+        ws_bytes = self._gemm_ws_bytes.get(key)
+        if ws_bytes is None:
+            ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
+                        self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
+            self._gemm_ws_bytes[key] = ws_bytes
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
         rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
                                    out.data_ptr(), out.stride(0), int(accumulate),

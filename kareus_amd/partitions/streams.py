@@ -10,19 +10,53 @@ whole forward/backward on the host to check the ordering rules without a GPU.
 from __future__ import annotations
 
 import contextlib
+import threading
 
 import torch
 
 
+class _StreamScope:
+    """``with`` block that makes a stream current.  Unlike ``torch.cuda.stream`` it also tells the
+    owning ``TorchStreams`` which stream that is, so that the engine's many questions about the
+    current stream inside the block cost a thread-local lookup instead of a new stream object."""
+
+    __slots__ = ("api", "stream", "prev_known", "prev")
+
+    def __init__(self, api, stream) -> None:
+        self.api, self.stream = api, stream
+
+    def __enter__(self):
+        tls = self.api._tls
+        self.prev_known = getattr(tls, "current", None)
+        self.prev = self.prev_known if self.prev_known is not None else torch.cuda.current_stream()
+        torch.cuda.set_stream(self.stream)
+        tls.current = self.stream
+        return self.stream
+
+    def __exit__(self, *exc):
+        torch.cuda.set_stream(self.prev)
+        self.api._tls.current = self.prev_known
+        return False
+
+
 class TorchStreams:
+    def __init__(self) -> None:
+        self._available = None
+        self._tls = threading.local()  # .current: the stream set by the innermost stream() block
+
     def available(self) -> bool:
-        return torch.cuda.is_available()
+        if self._available is None:
+            self._available = torch.cuda.is_available()
+        return self._available
 
     def current_stream(self):
-        return torch.cuda.current_stream() if torch.cuda.is_available() else None
+        known = getattr(self._tls, "current", None)
+        if known is not None:
+            return known
+        return torch.cuda.current_stream() if self.available() else None
 
     def stream(self, s):
-        return contextlib.nullcontext() if s is None else torch.cuda.stream(s)
+        return contextlib.nullcontext() if s is None else _StreamScope(self, s)
 
     def new_stream(self):
         return torch.cuda.Stream()
