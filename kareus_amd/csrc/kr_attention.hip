@@ -240,14 +240,14 @@ __device__ __forceinline__ bf16x8 bt_cols(uint32_t base, int g, int dt) {
 }
 
 // Ping-pong forward.  Two halves of four waves own the same 128 queries and walk the even / odd
-// key tiles (merged at the end like HALVES = 2 of attn_fwd_kernel), but the halves run in
-// antiphase.  Time is cut into periods by workgroup barriers; in every period one half only
-// feeds the matrix pipe — P.V of its previous tile, then S = Q.K^T of its next one, 32 MFMAs —
-// while the other half does everything else for its own tile: the softmax (exponentials, row
-// statistics, rounding to bf16, the occasional rescale of the output accumulators) and the
-// requests for the K / V tiles two steps ahead, which go straight from global memory into LDS
-// (swizzled [64][128] tiles, the swizzle applied on the global side).  A SIMD hosts one wave of
-// each half, so its matrix pipe and its vector ALU are busy at the same time instead of taking
+// key tiles (their partial softmax results are merged at the end, half 1 handing its state to
+// half 0 through LDS), but the halves run in antiphase.  Time is cut into periods by workgroup
+// barriers; in every period one half only feeds the matrix pipe — P.V of its previous tile, then
+// S = Q.K^T of its next one, 32 MFMAs — while the other half does everything else for its own
+// tile: the softmax (exponentials, row statistics, rounding to bf16, the occasional rescale of
+// the output accumulators) and the requests for the K / V tiles two steps ahead, which go
+// straight from global memory into blocked [64][128] LDS tiles.  A SIMD hosts one wave of each
+// half, so its matrix pipe and its vector ALU are busy at the same time instead of taking
 // turns, which is what happens when co-resident waves are in the same phase.
 __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
