@@ -92,7 +92,7 @@ def test_rmsnorm(be, rows, cols):
     assert (yc.float() - 3.0 / math.sqrt(9.0 + 1e-5)).abs().max() < 1e-2
 
 
-@pytest.mark.parametrize("cols", [512, 3072, 4096, 8192])
+@pytest.mark.parametrize("cols", [512, 1376, 2560, 3072, 4096, 8192])
 def test_rmsnorm_backward_fused_with_residual_add_is_bit_identical(be, cols):
     """RMSNorm backward + the residual fork's gradient sum in one kernel: same bits as the two
     kernels one after the other, also when the residual gradient is a row-strided slice and the
