@@ -888,11 +888,16 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
         // lane: query row qrow, keys key0 + 32t + 8g + 4h + e
         bf16x8 dsb[2];
         if (need_mask) {
-          asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+          // Off the diagonal no mask code must run.  Left alone the compiler turns the branch
+          // into 16 unconditional selects; values that pass through an (empty) volatile asm can
+          // only be produced where the asm executes, i.e. inside the branch.
           const int lim = qrow - key0 - t * 32 - 4 * h;
 #pragma unroll
-          for (int e = 0; e < 16; ++e)
-            if (8 * (e >> 2) + (e & 3) > lim) sacc[e] = -INFINITY;
+          for (int e = 0; e < 16; ++e) {
+            float v = 8 * (e >> 2) + (e & 3) > lim ? -INFINITY : sacc[e];
+            asm volatile("" : "+v"(v));
+            sacc[e] = v;
+          }
         }
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
