@@ -231,6 +231,47 @@ def hbm_kernels(w, nnb, device, launches=50):
     return rows_out
 
 
+def attention_kernels(w, nnb, device, launches=20):
+    """Causal attention forward and backward alone on the GPU, at the nanobatch batch and at the
+    whole-microbatch batch: average time of one forward / one backward call (HIP events on the
+    launch stream) and causal FLOPs (2*b*nq*s^2*hd forward, 2.5x backward) per second."""
+    from kareus_amd.backend import get_backend
+
+    be = get_backend("hip")
+    bf = torch.bfloat16
+    s_len, nq, nkv, hd = w["s"], w["nq"], w["nkv"], w["hd"]
+    scale = hd ** -0.5
+    out = []
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / launches
+
+    for b in sorted({w["b"] // nnb, w["b"]}):
+        q = torch.randn(s_len, b, nq, hd, device=device, dtype=bf)
+        k = torch.randn(s_len, b, nkv, hd, device=device, dtype=bf)
+        v = torch.randn(s_len, b, nkv, hd, device=device, dtype=bf)
+        o, lse = be.attn_fwd(q, k, v, scale)
+        do = torch.randn_like(o)
+        flops = 2.0 * b * nq * s_len * s_len * hd
+        t_f = timed(lambda: be.attn_fwd(q, k, v, scale))
+        t_b = timed(lambda: be.attn_bwd(do, q, k, v, o, lse, scale))
+        out.append({"batch": b, "seq": s_len, "q_heads": nq, "kv_heads": nkv, "head_dim": hd,
+                    "fwd_us": t_f * 1e6, "fwd_TFLOPs": flops / t_f / 1e12,
+                    "fwd_frac_of_peak": flops / t_f / MFMA_PEAK_BF16,
+                    "bwd_us": t_b * 1e6, "bwd_TFLOPs": 2.5 * flops / t_b / 1e12,
+                    "bwd_frac_of_peak": 2.5 * flops / t_b / MFMA_PEAK_BF16})
+    return out
+
+
 def cpu_baseline(w, budget_s=25.0):
     """The CPU oracle (fp32 PyTorch, autograd backward) on a bounded sample: same layer widths,
     one sequence of at most 1024 tokens, as many iterations as fit the time budget."""
@@ -274,6 +315,8 @@ def main():
                     help="run only the dominant-kernel leg (the command profiled under profiles/)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a residual-add kernel of known size (calibrates FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--attention-kernels", action="store_true",
+                    help="run only the attention forward/backward stand-alone (TFLOP/s against the MFMA peak)")
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
     args = ap.parse_args()
@@ -293,6 +336,9 @@ def main():
         return
     if args.copy_calibration:
         print(json.dumps({"copy_calibration": copy_calibration(device)}))
+        return
+    if args.attention_kernels:
+        print(json.dumps({"attention_kernels": attention_kernels(w, w["nnb"], device)}))
         return
     if args.hbm_kernels:
         print(json.dumps({"hbm_kernels": hbm_kernels(w, w["nnb"], device)}))
