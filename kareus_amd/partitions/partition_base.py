@@ -21,8 +21,6 @@ import contextlib
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Tuple, Union
 
-import torch
-
 from .context_manager import NanoBatchContext
 from .streams import stream_api
 from .tensor_graph import CommunicationOp, ComputeOp

@@ -27,7 +27,7 @@ import itertools
 import json
 import os
 import warnings
-from typing import Dict, Iterable, List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 Config = Tuple[object, object, int, int]          # (overlap_start, overlap_end, sm, block)
 Measured = Tuple[float, float]                    # (time_s, energy_j)
