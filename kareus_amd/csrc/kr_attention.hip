@@ -339,8 +339,6 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
   __syncthreads();
   if (half == 1) __syncthreads();  // half 1 starts one period late
 
-  // a tile is live for this wave if some of its rows can see some of its keys (wave-uniform)
-  auto live = [&](int j) { return key_of(j) <= qw0 + 31; };
   bf16x8 pb[2][2];
 
   // O^T += V^T . P^T for tile jj of this half (pb holds its probabilities)
