@@ -77,7 +77,8 @@ def test_rope_fused_in_place_leaves_value_heads(be):
 
 
 # ------------------------------------------------------------------ rmsnorm
-@pytest.mark.parametrize("rows,cols", [(1024, 512), (4096, 3072), (1000, 4096), (3, 8), (70, 8192), (257, 1376)])
+@pytest.mark.parametrize("rows,cols", [(1024, 512), (130, 1024), (67, 1536), (129, 2048), (4096, 3072), (1000, 4096),
+                                       (3, 8), (70, 8192), (257, 1376), (33, 2560), (40, 3584)])
 def test_rmsnorm(be, rows, cols):
     x, dy = rnd(rows, cols, seed=8), rnd(rows, cols, seed=9)
     g = (1 + 0.1 * torch.randn(cols, generator=torch.Generator().manual_seed(10))).to(DEV, torch.bfloat16)
