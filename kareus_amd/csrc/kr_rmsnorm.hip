@@ -67,44 +67,59 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
 // gradient of the norm is rounded to bf16 exactly as the stand-alone kernel rounds it and then
 // the gradient of the residual branch is added, so the fused result is bit-identical to the
 // two kernels run one after the other while one write and one read of the tensor disappear.
-// FULL: the row is exactly NCHUNK * 64 vectors long (hidden sizes 512 * k).  No lane is ever
-// idle, so the loop body is straight-line code and every load of a row — x, dy and the residual
-// gradient — is issued before the first wait; with per-chunk bounds checks each chunk of the
-// output pass paid its own round trip to memory.
-template <int NCHUNK, bool ADD, bool FULL>
+// FULL: the row is exactly SPLIT * NCHUNK * 64 vectors long (hidden sizes 512 * k).  No lane is
+// ever idle, so the loop body is straight-line code and every load of a row — x, dy and the
+// residual gradient — is issued before the first wait; with per-chunk bounds checks each chunk of
+// the output pass paid its own round trip to memory.
+// SPLIT = 2: two waves share a row (rows of more than 4096 elements), each holding half of it, so
+// that a wave's registers still hold its part; the halves of the row's dot product meet in LDS.
+template <int NCHUNK, bool ADD, bool FULL, int SPLIT>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
     const bf16* __restrict__ gamma, const bf16* __restrict__ dres, bf16* __restrict__ dx,
     float* __restrict__ partial, int rows, int cols, int64_t dy_ld, int64_t x_ld, int64_t dres_ld,
     int64_t dx_ld) {
+  constexpr int kRowsPerBlock = kWaves / SPLIT;
   __shared__ float red[kWaves - 1][64 * 8];
+  __shared__ float halves[2][kRowsPerBlock][2];  // [iteration parity][row of the block][half]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int part = SPLIT == 2 ? (wave & 1) : 0;      // which half of the row this wave holds
+  const int slot = SPLIT == 2 ? (wave >> 1) : wave;  // which of the block's rows
   const int nvec = cols / 8;
   const float inv_cols = 1.0f / (float)cols;
+  // this lane's vectors of a row: v0, v0 + 64, ...
+  const int v0 = part * NCHUNK * 64 + lane;
   bf16x8 g[NCHUNK];
   float dg[NCHUNK][8];
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    const int v = lane + c * 64;
+    const int v = v0 + c * 64;
     g[c] = (FULL || v < nvec) ? ldg8(gamma + v * 8) : zero8();
 #pragma unroll
     for (int e = 0; e < 8; ++e) dg[c][e] = 0.f;
   }
-  for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
-    const bf16* xr = x + (int64_t)row * x_ld;
-    const bf16* dr = dy + (int64_t)row * dy_ld;
-    const bf16* rr = ADD ? dres + (int64_t)row * dres_ld : nullptr;
-    const float rs = rstd[row];
+  int parity = 0;
+  // (with two waves per row every wave of the block makes the same number of trips: the loop
+  // holds a workgroup barrier)
+  for (int base = blockIdx.x * kRowsPerBlock; base < rows; base += gridDim.x * kRowsPerBlock) {
+    const int row = base + slot;
+    const bool active = SPLIT == 1 || row < rows;  // SPLIT == 1: the loop bound is the wave's own
+    if (SPLIT == 1 && row >= rows) break;
+    const int64_t r64 = active ? row : 0;
+    const bf16* xr = x + r64 * x_ld;
+    const bf16* dr = dy + r64 * dy_ld;
+    const bf16* rr = ADD ? dres + r64 * dres_ld : nullptr;
+    const float rs = active ? rstd[r64] : 0.f;
     bf16x8 xv[NCHUNK], dv[NCHUNK], rv[ADD && FULL ? NCHUNK : 1];
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
-      const int v = lane + c * 64;
-      xv[c] = (FULL || v < nvec) ? ldg8(xr + v * 8) : zero8();
-      dv[c] = (FULL || v < nvec) ? ldg8(dr + v * 8) : zero8();
+      const int v = v0 + c * 64;
+      xv[c] = (active && (FULL || v < nvec)) ? ldg8(xr + v * 8) : zero8();
+      dv[c] = (active && (FULL || v < nvec)) ? ldg8(dr + v * 8) : zero8();
     }
     if (ADD && FULL) {
 #pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) rv[c] = ldg8(rr + (lane + c * 64) * 8);
+      for (int c = 0; c < NCHUNK; ++c) rv[c] = active ? ldg8(rr + (v0 + c * 64) * 8) : zero8();
     }
     float dot = 0.f;
 #pragma unroll
@@ -116,12 +131,19 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
         dot += d * (float)g[c][e] * xh;
         dg[c][e] += d * xh;
       }
-    dot = wave_sum(dot) * inv_cols;
-    bf16* oxr = dx + (int64_t)row * dx_ld;
+    dot = wave_sum(dot);
+    if (SPLIT == 2) {
+      if (lane == 0) halves[parity][slot][part] = dot;
+      __syncthreads();
+      dot = halves[parity][slot][0] + halves[parity][slot][1];
+      parity ^= 1;  // the next row uses the other buffer: one barrier per row is enough
+    }
+    dot *= inv_cols;
+    bf16* oxr = dx + r64 * dx_ld;
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
-      const int v = lane + c * 64;
-      if (FULL || v < nvec) {
+      const int v = v0 + c * 64;
+      if (active && (FULL || v < nvec)) {
         bf16x8 o, r;
         if (ADD) r = FULL ? rv[c] : ldg8(rr + v * 8);
 #pragma unroll
@@ -134,23 +156,24 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
       }
     }
   }
-  // combine the block's waves chunk by chunk, then publish the block's partial row
+  // combine the waves that hold the same columns chunk by chunk, then publish the block's
+  // partial row
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    if (wave > 0) {
+    if (slot > 0) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) red[wave - 1][e * 64 + lane] = dg[c][e];
+      for (int e = 0; e < 8; ++e) red[(slot - 1) * SPLIT + part][e * 64 + lane] = dg[c][e];
     }
     __syncthreads();
-    if (wave == 0) {
-      const int v = lane + c * 64;
+    if (slot == 0) {
+      const int v = v0 + c * 64;
       if (v < nvec) {
         float* pr = partial + (int64_t)blockIdx.x * cols + v * 8;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           float sum = dg[c][e];
 #pragma unroll
-          for (int w = 0; w < kWaves - 1; ++w) sum += red[w][e * 64 + lane];
+          for (int w = 1; w < kRowsPerBlock; ++w) sum += red[(w - 1) * SPLIT + part][e * 64 + lane];
           pr[e] = sum;
         }
       }
@@ -192,14 +215,30 @@ __global__ __launch_bounds__(kDgammaThreads) void rmsnorm_dgamma_kernel(const fl
   }
 }
 
-inline int bwd_blocks(int rows) {
-  int blocks = (rows + kWaves - 1) / kWaves;
+// rows wider than 4096 elements are shared by two waves
+inline int bwd_split(int cols) { return cols > 4096 ? 2 : 1; }
+
+inline int bwd_blocks(int rows, int cols) {
+  const int rows_per_block = kWaves / bwd_split(cols);
+  int blocks = (rows + rows_per_block - 1) / rows_per_block;
   return blocks > kMaxBwdBlocks ? kMaxBwdBlocks : blocks;
 }
 
 inline int chunks_for(int cols) { return (cols / 8 + 63) / 64; }
 
 }  // namespace
+
+// at most 8 vectors per lane (backward: wider rows are shared by two waves)
+#define KR_DISPATCH_CHUNKS8(NC, CALL) \
+  switch (NC) {                       \
+    case 1: { constexpr int C_ = 1; CALL; } break;   \
+    case 2: { constexpr int C_ = 2; CALL; } break;   \
+    case 3: { constexpr int C_ = 3; CALL; } break;   \
+    case 4: { constexpr int C_ = 4; CALL; } break;   \
+    case 5: case 6: { constexpr int C_ = 6; CALL; } break;   \
+    case 7: case 8: { constexpr int C_ = 8; CALL; } break;   \
+    default: return KR_EUNSUPPORTED;  \
+  }
 
 #define KR_DISPATCH_CHUNKS(NC, CALL) \
   switch (NC) {                      \
@@ -228,7 +267,7 @@ extern "C" int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* 
 
 extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
   if (rows <= 0 || cols <= 0) return 0;
-  return (size_t)bwd_blocks(rows) * (size_t)cols * sizeof(float);
+  return (size_t)bwd_blocks(rows, cols) * (size_t)cols * sizeof(float);
 }
 
 extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd,
@@ -243,20 +282,28 @@ extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rs
   if (!kr_aligned16(x) || !kr_aligned16(dy) || !kr_aligned16(dx) || !kr_aligned16(gamma) ||
       !kr_aligned16(workspace) || (dres && !kr_aligned16(dres)))
     return KR_EINVAL;
-  const int blocks = bwd_blocks(rows);
-  const int nc = chunks_for(cols);
-#define KR_RMS_BWD(ADDV, FULLV)                                                                     \
-  KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, ADDV, FULLV>), dim3(blocks),    \
-                                           dim3(kThreads), 0, (hipStream_t)stream, (const bf16*)dy, \
-                                           (const bf16*)x, rstd, (const bf16*)gamma,                \
-                                           (const bf16*)dres, (bf16*)dx, (float*)workspace, rows,   \
-                                           cols, dy_ld, x_ld, dres ? dres_ld : (int64_t)0, dx_ld))
-  // rows of exactly 1, 2, 3, 4, 6 or 8 times 512 elements take the straight-line kernel
-  const bool full = cols % 512 == 0 && cols / 512 == nc && nc <= 8 && nc != 5 && nc != 7;
-  if (dres) {
-    if (full) { KR_RMS_BWD(true, true); } else { KR_RMS_BWD(true, false); }
+  const int blocks = bwd_blocks(rows, cols);
+  const int split = bwd_split(cols);
+  const int nc = (cols / 8 + 64 * split - 1) / (64 * split);  // 16-byte vectors per lane
+#define KR_RMS_BWD(ADDV, FULLV, SPLITV)                                                             \
+  KR_DISPATCH_CHUNKS8(nc, hipLaunchKernelGGL((rmsnorm_bwd_kernel<C_, ADDV, FULLV, SPLITV>),         \
+                                           dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream,    \
+                                           (const bf16*)dy, (const bf16*)x, rstd,                   \
+                                           (const bf16*)gamma, (const bf16*)dres, (bf16*)dx,        \
+                                           (float*)workspace, rows, cols, dy_ld, x_ld,              \
+                                           dres ? dres_ld : (int64_t)0, dx_ld))
+  // rows of exactly 1, 2, 3, 4, 6 or 8 times 512 elements per wave take the straight-line kernel
+  const bool full = cols % (512 * split) == 0 && cols / (512 * split) == nc && nc <= 8 && nc != 5 && nc != 7;
+  if (split == 2) {
+    if (dres) {
+      if (full) { KR_RMS_BWD(true, true, 2); } else { KR_RMS_BWD(true, false, 2); }
+    } else {
+      if (full) { KR_RMS_BWD(false, true, 2); } else { KR_RMS_BWD(false, false, 2); }
+    }
+  } else if (dres) {
+    if (full) { KR_RMS_BWD(true, true, 1); } else { KR_RMS_BWD(true, false, 1); }
   } else {
-    if (full) { KR_RMS_BWD(false, true); } else { KR_RMS_BWD(false, false); }
+    if (full) { KR_RMS_BWD(false, true, 1); } else { KR_RMS_BWD(false, false, 1); }
   }
 #undef KR_RMS_BWD
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;

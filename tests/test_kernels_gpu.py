@@ -78,7 +78,7 @@ def test_rope_fused_in_place_leaves_value_heads(be):
 
 # ------------------------------------------------------------------ rmsnorm
 @pytest.mark.parametrize("rows,cols", [(1024, 512), (130, 1024), (67, 1536), (129, 2048), (4096, 3072), (1000, 4096),
-                                       (3, 8), (70, 8192), (257, 1376), (33, 2560), (40, 3584)])
+                                       (3, 8), (70, 8192), (257, 1376), (33, 2560), (40, 3584), (45, 5120), (31, 6144), (9, 4104)])
 def test_rmsnorm(be, rows, cols):
     x, dy = rnd(rows, cols, seed=8), rnd(rows, cols, seed=9)
     g = (1 + 0.1 * torch.randn(cols, generator=torch.Generator().manual_seed(10))).to(DEV, torch.bfloat16)
@@ -93,7 +93,7 @@ def test_rmsnorm(be, rows, cols):
     assert (yc.float() - 3.0 / math.sqrt(9.0 + 1e-5)).abs().max() < 1e-2
 
 
-@pytest.mark.parametrize("cols", [512, 1376, 2560, 3072, 4096, 8192])
+@pytest.mark.parametrize("cols", [512, 1376, 2560, 3072, 4096, 5000, 6144, 8192])
 def test_rmsnorm_backward_fused_with_residual_add_is_bit_identical(be, cols):
     """RMSNorm backward + the residual fork's gradient sum in one kernel: same bits as the two
     kernels one after the other, also when the residual gradient is a row-strided slice and the
