@@ -17,6 +17,8 @@
 //   P nor V is ever transposed through memory.
 // Tensors are addressed through (seq, batch, head) strides, so sequence-major [s, b, h, d]
 // views of the fused QKV projection are consumed in place.
+#include <stdlib.h>
+
 #include "kr_common.h"
 
 namespace {
@@ -762,6 +764,227 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
   }
 }
 
+// dK/dV with the waves of a SIMD specialised.  The kernel above runs one wave per SIMD and is
+// bound by the number of instructions that wave has to issue (one every 4-5 cycles): scores,
+// exponentials and the two accumulating products all queue in one instruction stream.  Here a
+// workgroup has eight waves, two per SIMD, for the same 128 keys:
+//   waves 0-3 ("score" waves, 32 keys each, K and V fragments in registers) compute S = Q.K^T and
+//     dP = dO.V^T of a 32-query block, P and dS from them, and hand P, dS (bf16, already in the
+//     B-operand layout of the next products) to their partner through 4 KB of LDS;
+//   waves 4-7 ("accumulate" waves, the partner on the same SIMD) hold dK and dV and issue
+//     dV^T += dO^T.P and dK^T += Q^T.dS with the Q / dO tiles read transposed; they also issue
+//     every global -> LDS request, which keeps the score waves' instruction stream short.
+// Both run well below 256 registers, so the matrix products write plain VGPRs (no accumulator
+// copies).  Two barriers per 64-query tile: after each, the accumulate waves pick up the block
+// the score waves finished before it, so the two kinds of work overlap with one block of lag.
+// Three LDS stages: tile it is read as rows by the score waves and transposed by the accumulate
+// waves during iteration it; tile it+1 is complete by the first barrier of iteration it (the
+// score waves start on it one block ahead); tile it+2 is requested after that barrier into the
+// stage tile it-1 left at it.
+template <bool PARTIAL>
+__global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ neg_lse2, const float* __restrict__ delta,
+    bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
+    float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, float scale, float scale_log2,
+    QLayout ql, KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  // stage layout: Q tile | dO tile (blocked tiles) | lse[64] fp32 | delta[64] fp32
+  constexpr uint32_t STAGE = 2 * BT_BYTES + 512;  // bytes
+  constexpr int NS = 3;
+  // hand-over area behind the stages: [block parity][key block][slot 0..3][lane] 16 bytes each
+  constexpr uint32_t XCH = NS * STAGE;
+
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int role = wave8 >> 2;  // 0: score wave, 1: accumulate wave
+  const int wave = wave8 & 3;   // key block of the tile
+  const int nkt = s / 128;
+  const int lid_all = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const int part = lid_all % qsplit, lid = lid_all / qsplit;
+  const int kt = lid % nkt;  // low key tiles see the most queries: they come first
+  const int head = (lid / nkt) % nq;
+  const int bi = lid / (nkt * nq);
+  const int per = nq / nkv;
+  const int kvh = head / per;
+  const int key0 = kt * 128;
+  const int kw0 = key0 + wave * 32;
+  const int krow = kw0 + (lane & 31);
+  const int qt_first = key0 / 64;
+  const int niter = (s / 64 - qt_first - part + qsplit - 1) / qsplit;  // this part's query tiles of 64
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
+  const uint32_t xch_lane = lds0 + XCH + wave * 4096 + lane * 16;  // + parity * 16384 + slot * 1024
+
+  if (role == 0) {
+    // ------------------------------------------------------------------ score waves
+    const bf16* kp = k + kl.at(bi, kvh) + (int64_t)krow * kl.s_;
+    const bf16* vp = v + vl.at(bi, kvh) + (int64_t)krow * vl.s_;
+    bf16x8 kf[HD / 16], vf[HD / 16];
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+      kf[kk] = ldg8(kp + kk * 16 + h * 8);
+      vf[kk] = ldg8(vp + kk * 16 + h * 8);
+    }
+    __syncthreads();  // tile 0 (and 1) requested by the accumulate waves have landed
+    // S = Q.K^T and dP = dO.V^T of one 32-query block: sixteen fragments, then sixteen MFMAs
+    auto issue_scores = [&](int stage, int sub, f32x16& sacc, f32x16& dpacc) {
+      uint32_t q_rows = lds0 + stage * STAGE + bt_rows_lane(lane);
+      uint32_t do_rows = q_rows + BT_BYTES;
+      asm volatile("" : "+v"(q_rows), "+v"(do_rows));  // one base register each; the rest are immediates
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        sacc[e] = 0.f;
+        dpacc[e] = 0.f;
+      }
+      bf16x8 qfr[HD / 16], dofr[HD / 16];
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk) {
+        qfr[kk] = bt_rows(q_rows, sub, kk);
+        dofr[kk] = bt_rows(do_rows, sub, kk);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk) {
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], sacc, 0, 0, 0);
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[kk], vf[kk], dpacc, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // P = exp2(S c - lse), dS = P (dP - delta), handed to the partner wave
+    auto finish_block = [&](int stage, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
+      const float* stats = reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) +
+                                                          stage * STAGE + 2 * BT_BYTES);
+      // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that reach the diagonal
+      // pay for the causal mask
+      if (qs0 < kw0 + 31) {
+        const int lim = krow - qs0 - 4 * h;  // element offsets below it are queries before the key
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          float x = 8 * (e >> 2) + (e & 3) < lim ? -INFINITY : sacc[e];
+          asm volatile("" : "+v"(x));  // keeps this a branch: off the diagonal no mask code runs
+          sacc[e] = x;
+        }
+      }
+      bf16x8 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
+          const float ds = p * (dpacc[g * 4 + e] - d4[e]);
+          pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
+          dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
+        }
+      }
+      const uint32_t xa = xch_lane + sub * 16384;
+      *(KR_LDS bf16x8*)(xa) = pb[0];
+      *(KR_LDS bf16x8*)(xa + 1024) = pb[1];
+      *(KR_LDS bf16x8*)(xa + 2048) = dsb[0];
+      *(KR_LDS bf16x8*)(xa + 3072) = dsb[1];
+    };
+    // The score products of a block are issued one block ahead of the exponentials that consume
+    // them and run on the matrix pipe while the vector ALU works on the block before (the first
+    // block of the next tile during the second block of this one: that tile is complete by the
+    // first barrier of the iteration; behind the last tile it reads a stale stage, unused).
+    f32x16 s0, dp0, s1, dp1;
+    issue_scores(0, 0, s0, dp0);
+    for (int it = 0; it < niter; ++it) {
+      const int stage = it % NS;
+      const int q0 = (qt_first + it * qsplit + part) * 64;
+      issue_scores(stage, 1, s1, dp1);
+      finish_block(stage, 0, q0, s0, dp0);
+      __syncthreads();  // hand-over of block 0
+      issue_scores((it + 1) % NS, 0, s0, dp0);
+      finish_block(stage, 1, q0 + 32, s1, dp1);
+      __syncthreads();  // hand-over of block 1
+    }
+    return;
+  }
+
+  // -------------------------------------------------------------------- accumulate waves
+  const bf16* qb = q + ql.at(bi, head, per);
+  const bf16* dob = dout + dol.at(bi, head, per);
+  const int64_t stat0 = ((int64_t)bi * nq + head) * s;
+  auto request_tile = [&](int it) {
+    const int qt = qt_first + it * qsplit + part;
+    const uint32_t tile = lds0 + (it % NS) * STAGE;
+    // the tile's 64 + 64 row statistics: one 4-byte-per-lane request each, by waves 0 and 1
+    if (wave < 2) {
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));
+      dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + qt * 64, (uint32_t)l2 * 4u,
+              tile + 2 * BT_BYTES + wave * 256);
+    }
+    bt_request(qb + (int64_t)qt * 64 * ql.s_, ql.s_, tile, wave, lane);
+    bt_request(dob + (int64_t)qt * 64 * dol.s_, dol.s_, tile + BT_BYTES, wave, lane);
+  };
+  f32x16 dkacc[HD / 32], dvacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      dkacc[dt][e] = 0.f;
+      dvacc[dt][e] = 0.f;
+    }
+  request_tile(0);
+  if (niter > 1) request_tile(1);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  for (int it = 0; it < niter; ++it) {
+    const int stage = it % NS;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      // the transposed fragments do not depend on the score waves: requested ahead of the barrier
+      uint32_t q_cols = lds0 + stage * STAGE + bt_cols_lane(lane);
+      uint32_t do_cols = q_cols + BT_BYTES;
+      asm volatile("" : "+v"(q_cols), "+v"(do_cols));
+      bf16x8 dot[2][HD / 32], qtr[2][HD / 32];
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+          dot[k2][dt] = bt_cols(do_cols, 2 * sub + k2, dt);
+          qtr[k2][dt] = bt_cols(q_cols, 2 * sub + k2, dt);
+        }
+      // tile it+1 (requested after the first barrier of the iteration before) must have landed
+      // before this iteration's first barrier: the score waves start on it right after
+      if (sub == 0) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing newer is in flight
+      __syncthreads();
+      if (sub == 0 && it + 2 < niter) request_tile(it + 2);  // into the stage tile it-1 has left
+      const uint32_t xa = xch_lane + sub * 16384;
+      const bf16x8 pb0 = *(KR_LDS const bf16x8*)(xa);
+      const bf16x8 pb1 = *(KR_LDS const bf16x8*)(xa + 1024);
+      const bf16x8 ds0 = *(KR_LDS const bf16x8*)(xa + 2048);
+      const bf16x8 ds1 = *(KR_LDS const bf16x8*)(xa + 3072);
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt) {
+        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[0][dt], pb0, dvacc[dt], 0, 0, 0);
+        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[0][dt], ds0, dkacc[dt], 0, 0, 0);
+      }
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt) {
+        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[1][dt], pb1, dvacc[dt], 0, 0, 0);
+        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[1][dt], ds1, dkacc[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  // The hand-over slice this wave read last is its own: use the other one (block parity 0, read
+  // one barrier earlier by this wave only) for the output transposition.
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + XCH + wave * 4096, lane);
+  if (PARTIAL) {
+    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + kw0;
+    store_rows_f32(rs, dkacc, scale, part_k + prow * HD, HD);
+    store_rows_f32(rs, dvacc, 1.0f, part_v + prow * HD, HD);
+  } else {
+    store_rows_bf16(rs, dkacc, scale, dk + dkl.at(bi, kvh) + (int64_t)kw0 * dkl.s_, dkl.s_);
+    store_rows_bf16(rs, dvacc, 1.0f, dv + dvl.at(bi, kvh) + (int64_t)kw0 * dvl.s_, dvl.s_);
+  }
+}
+
 // dk/dv[b, kvh, i, :] = sum over the group's query heads of the fp32 partials; one thread per
 // 8 channels (two 16-byte reads per partial, one 16-byte bf16 store).
 __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
@@ -945,6 +1168,14 @@ template __global__ void attn_bwd_dq_kernel<1>(KR_ATTN_DQ_ARGS);
 template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
 #undef KR_ATTN_DQ_ARGS
 
+#define KR_ATTN_DKDV_ARGS                                                                          \
+  const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, bf16*, \
+      float*, float*, int, int, int, int, float, float, QLayout, KLayout, KLayout, QLayout,      \
+      KLayout, KLayout
+template __global__ void attn_bwd_dkdv_ws_kernel<false>(KR_ATTN_DKDV_ARGS);
+template __global__ void attn_bwd_dkdv_ws_kernel<true>(KR_ATTN_DKDV_ARGS);
+#undef KR_ATTN_DKDV_ARGS
+
 template __global__ void attn_bwd_dkdv_kernel<false>(const bf16*, const bf16*, const bf16*, const bf16*,
                                                      const float*, const float*, bf16*, bf16*, float*,
                                                      float*, int, int, int, int, float, float,
@@ -1001,6 +1232,7 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
   constexpr size_t lds_dkdv = 4 * (2 * BT_BYTES + 512);  // four stages: Q tile, dO tile, statistics
+  constexpr size_t lds_dkdv_ws = 3 * (2 * BT_BYTES + 512) + 32768;  // three stages + the hand-over area
   constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
@@ -1008,6 +1240,12 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
     if (e == hipSuccess)
       e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_ws_kernel<false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv_ws);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_ws_kernel<true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv_ws);
     if (e == hipSuccess)
       e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
@@ -1024,7 +1262,27 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
   const dim3 grid_kv((s / 128) * nq * b * qsplit);
-  if (partial) {
+  const char* const ws_env = getenv("KR_DKDV_WS");  // experiment switch
+  const bool use_ws = ws_env != nullptr && ws_env[0] == '1';
+  if (use_ws) {
+#define KR_DKDV_WS_LAUNCH(P)                                                                        \
+  hipLaunchKernelGGL((attn_bwd_dkdv_ws_kernel<P>), grid_kv, dim3(512), lds_dkdv_ws, st,             \
+                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout,             \
+                     (const float*)neg_lse2, (const float*)delta, (bf16*)dk, (bf16*)dv, part_k,     \
+                     part_v, s, nq, nkv, partial ? qsplit : 1, scale, scale_log2, ql, kl, vl, dol, \
+                     dkl, dvl)
+    if (partial) {
+      KR_DKDV_WS_LAUNCH(true);
+      if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+      const int64_t total = (int64_t)b * nkv * s * 16;
+      hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                         st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
+                         nkv, qsplit, total, dkl, dvl);
+    } else {
+      KR_DKDV_WS_LAUNCH(false);
+    }
+#undef KR_DKDV_WS_LAUNCH
+  } else if (partial) {
     hipLaunchKernelGGL(attn_bwd_dkdv_kernel<true>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
                        (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,
                        (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, qsplit, scale,
