@@ -17,8 +17,6 @@
 //   P nor V is ever transposed through memory.
 // Tensors are addressed through (seq, batch, head) strides, so sequence-major [s, b, h, d]
 // views of the fused QKV projection are consumed in place.
-#include <stdlib.h>
-
 #include "kr_common.h"
 
 namespace {
@@ -141,9 +139,10 @@ static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
 // Backward.  Launches: delta pre-pass, dK/dV pass, (group reduction), dQ pass.  No atomics,
 // deterministic.
 //   1. delta[b, h, i] = sum_d dO[i, d] * O[i, d]                      (HBM-bound pre-pass)
-//   2. dK, dV: a workgroup owns 128 keys of one (batch, QUERY head) — 32 per wave, their K and
-//      V fragments in registers — and streams every query tile at or below the diagonal
-//      through LDS.  Per 32x32 block:
+//   2. dK, dV: a workgroup owns 128 keys of one (batch, QUERY head) — 32 per pair of waves,
+//      their K and V fragments in the registers of the pair's score wave, dK and dV in those of
+//      its accumulate wave — and streams every query tile at or below the diagonal through LDS.
+//      Per 32x32 block:
 //        S = Q.K^T, dP = dO.V^T (rows = queries on the MFMA A port, so a lane holds one key
 //        column), P = exp2(S*c - lse), dS = P*(dP - delta), then dV^T += dO^T.P and
 //        dK^T += Q^T.dS with the Q / dO tiles read back transposed (ds_read_b64_tr_b16).
@@ -545,229 +544,11 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
   }
 }
 
-// PARTIAL = true: fp32 results for this query head go to part_k / part_v [b, nq, s, 128]
-template <bool PARTIAL>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
-    const bf16* __restrict__ dout, const float* __restrict__ neg_lse2, const float* __restrict__ delta,
-    bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
-    float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, float scale, float scale_log2,
-    QLayout ql,
-    KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
-  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
-  // stage layout: Q tile | dO tile (blocked tiles) | lse[64] fp32 | delta[64] fp32
-  constexpr uint32_t STAGE = 2 * BT_BYTES + 512;  // bytes
-
-  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nkt = s / 128;
-  // qsplit workgroups share a key tile and take every qsplit-th query tile (fp32 partials, summed
-  // by the group-reduce kernel): with few workgroups the first key tiles, which see all queries,
-  // would otherwise set the kernel's time
-  const int lid_all = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int part = lid_all % qsplit, lid = lid_all / qsplit;
-  const int kt = lid % nkt;  // low key tiles see the most queries: they come first
-  const int head = (lid / nkt) % nq;
-  const int bi = lid / (nkt * nq);
-  const int per = nq / nkv;
-  const int kvh = head / per;
-  const int key0 = kt * 128;
-  const int kw0 = key0 + wave * 32;
-  const int krow = kw0 + (lane & 31);
-
-  const bf16* kp = k + kl.at(bi, kvh) + (int64_t)krow * kl.s_;
-  const bf16* vp = v + vl.at(bi, kvh) + (int64_t)krow * vl.s_;
-  bf16x8 kf[HD / 16], vf[HD / 16];
-#pragma unroll
-  for (int kk = 0; kk < HD / 16; ++kk) {
-    kf[kk] = ldg8(kp + kk * 16 + h * 8);
-    vf[kk] = ldg8(vp + kk * 16 + h * 8);
-  }
-  f32x16 dkacc[HD / 32], dvacc[HD / 32];
-#pragma unroll
-  for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      dkacc[dt][e] = 0.f;
-      dvacc[dt][e] = 0.f;
-    }
-
-  const int qt_first = key0 / 64;
-  const int niter = (s / 64 - qt_first - part + qsplit - 1) / qsplit;  // this part's query tiles of 64
-  const bf16* qb = q + ql.at(bi, head, per);
-  const bf16* dob = dout + dol.at(bi, head, per);
-  const int64_t stat0 = ((int64_t)bi * nq + head) * s;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
-
-  // Q and dO tiles go straight from global memory into LDS; the row statistics pass through a
-  // register of the first 128 threads.  A wave's share of a stage is eight 1-KiB requests
-  // (blocks wave + 4 i of the Q tile, then of the dO tile); request_one(i) issues one of them.
-  // request_begin(it, stage) prepares tile `it`: pointers to the four consecutive rows this wave
-  // fetches of the Q and of the dO tile (rows 4 wave + 0..3, + 16, 32, 48 through the lanes).
-  uint32_t req_tile = 0, req_lane_off = 0;
-  const bf16* req_q = nullptr;
-  const bf16* req_do = nullptr;
-  const bf16* req_row = nullptr;
-  auto request_begin = [&](int it, int stage) {
-    const int req_qt = qt_first + it * qsplit + part;
-    req_tile = lds0 + stage * STAGE;
-    req_q = qb + ((int64_t)req_qt * 64 + 4 * wave) * ql.s_;
-    req_do = dob + ((int64_t)req_qt * 64 + 4 * wave) * dol.s_;
-    // the tile's 64 + 64 row statistics: one 4-byte-per-lane request each, by waves 0 and 1
-    if (wave < 2) {
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));
-      dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + req_qt * 64, (uint32_t)l2 * 4u,
-              req_tile + 2 * BT_BYTES + wave * 256);
-    }
-  };
-  // requests 0..3: the Q tile, 4..7: the dO tile; issued in this order
-  auto request_one = [&](int i) {
-    const bool second = i >= 4;
-    if ((i & 3) == 0) {
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));  // the lane offset lives only across the four requests of a tile
-      const int ss = (int)(second ? dol.s_ : ql.s_);
-      req_lane_off = (uint32_t)((l2 >> 4) * 16 * ss + (l2 & 15) * 8) * 2u;
-      req_row = second ? req_do : req_q;
-    }
-    dma_b128(req_row, req_lane_off, req_tile + (second ? BT_BYTES : 0) + (wave + 4 * (i & 3)) * BT_BLK);
-    req_row += second ? dol.s_ : ql.s_;
-  };
-  // Four stages: while tile `it` is consumed, tile it+1 is already complete (its first score
-  // block is computed one step ahead, see below), tiles it+2 and it+3 are on their way.
-  for (int p = 0; p < 3 && p < niter; ++p) {
-    request_begin(p, p);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) request_one(i);
-  }
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-  __syncthreads();
-
-  // The wave runs alone on its SIMD, so the overlap of matrix and vector work has to come from
-  // inside it: the two score products of a 32-query block (S = Q.K^T, dP = dO.V^T) are issued
-  // one block ahead of the exponentials that consume them, and execute while the vector ALU
-  // works on the previous block; the requests for a later tile are issued one at a time between
-  // those MFMAs (the texture-address path takes ~64 cycles per request and would otherwise
-  // stall the wave for 500 cycles with the matrix pipe idle).  Blocks that lie wholly before
-  // the wave's keys are not skipped but masked to zero (there are at most three per wave): the
-  // loop body stays straight-line code and the accumulators stay where they are.
-  auto scores = [&](int stage, int sub, f32x16& sacc, f32x16& dpacc, bool with_requests) {
-    uint32_t q_rows = lds0 + stage * STAGE + bt_rows_lane(lane);
-    uint32_t do_rows = q_rows + BT_BYTES;
-    asm volatile("" : "+v"(q_rows), "+v"(do_rows));  // one base register each; the rest are immediates
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      sacc[e] = 0.f;
-      dpacc[e] = 0.f;
-    }
-    // all sixteen fragments are requested before the first MFMA (registers are plentiful at one
-    // wave per SIMD)
-    bf16x8 qfr[HD / 16], dofr[HD / 16];
-#pragma unroll
-    for (int kk = 0; kk < HD / 16; ++kk) {
-      qfr[kk] = bt_rows(q_rows, sub, kk);
-      dofr[kk] = bt_rows(do_rows, sub, kk);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int kk = 0; kk < HD / 16; ++kk) {
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], sacc, 0, 0, 0);
-      dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[kk], vf[kk], dpacc, 0, 0, 0);
-      if (with_requests) {
-        request_one(kk);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  };
-  // P = exp2(S c - lse), dS = P (dP - delta); then dV^T += dO^T . P and dK^T += Q^T . dS
-  auto consume = [&](int stage, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
-    const float* stats =
-        reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) + stage * STAGE + 2 * BT_BYTES);
-    // the transposed fragments of the two products at the end are requested first and arrive
-    // while the vector ALU does the exponentials
-    uint32_t q_cols = lds0 + stage * STAGE + bt_cols_lane(lane);
-    uint32_t do_cols = q_cols + BT_BYTES;
-    asm volatile("" : "+v"(q_cols), "+v"(do_cols));
-    bf16x8 dot[2][HD / 32], qtr[2][HD / 32];
-#pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt) {
-        dot[k2][dt] = bt_cols(do_cols, 2 * sub + k2, dt);
-        qtr[k2][dt] = bt_cols(q_cols, 2 * sub + k2, dt);
-      }
-    __builtin_amdgcn_sched_barrier(0);
-    // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that reach the diagonal
-    // pay for the causal mask (wave-uniform branch)
-    if (qs0 < kw0 + 31) {
-      asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
-      const int lim = krow - qs0 - 4 * h;  // element offsets below it are queries before the key
-#pragma unroll
-      for (int e = 0; e < 16; ++e)
-        if (8 * (e >> 2) + (e & 3) < lim) sacc[e] = -INFINITY;
-    }
-    bf16x8 pb[2], dsb[2];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
-        const float ds = p * (dpacc[g * 4 + e] - d4[e]);
-        pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
-        dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);  // the vector work first, then the MFMAs back to back
-#pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt) {
-        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[k2][dt], pb[k2], dvacc[dt], 0, 0, 0);
-        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[k2][dt], dsb[k2], dkacc[dt], 0, 0, 0);
-      }
-  };
-
-  f32x16 s0, dp0, s1, dp1;
-  scores(0, 0, s0, dp0, false);
-  for (int it = 0; it < niter; ++it) {
-    const int cur = it & 3, nxt = (it + 1) & 3, far = (it + 3) & 3;
-    const bool more = it + 3 < niter;  // tile it+3 goes where tile it-1 was read last
-    if (more) request_begin(it + 3, far);
-    const int q0 = (qt_first + it * qsplit + part) * 64;
-    scores(cur, 1, s1, dp1, more);
-    consume(cur, 0, q0, s0, dp0);
-    scores(nxt, 0, s0, dp0, false);  // first block of the next tile (after the last tile: unused)
-    consume(cur, 1, q0 + 32, s1, dp1);
-    // tile it+2 (requested an iteration ago) must have landed before the barrier that makes it
-    // readable as `nxt` of the next iteration; this iteration's eight tile requests, issued
-    // after its statistics request, may fly on
-    if (more)
-      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
-    else
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-    __syncthreads();
-  }
-
-  // the loop ended with a barrier: the staging buffers are free for the output transposition
-  RowStage rs;
-  rs.init(reinterpret_cast<char*>(smem) + wave * 4096, lane);
-  if (PARTIAL) {
-    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + kw0;
-    store_rows_f32(rs, dkacc, scale, part_k + prow * HD, HD);
-    store_rows_f32(rs, dvacc, 1.0f, part_v + prow * HD, HD);
-  } else {
-    store_rows_bf16(rs, dkacc, scale, dk + dkl.at(bi, kvh) + (int64_t)kw0 * dkl.s_, dkl.s_);
-    store_rows_bf16(rs, dvacc, 1.0f, dv + dvl.at(bi, kvh) + (int64_t)kw0 * dvl.s_, dvl.s_);
-  }
-}
-
-// dK/dV with the waves of a SIMD specialised.  The kernel above runs one wave per SIMD and is
-// bound by the number of instructions that wave has to issue (one every 4-5 cycles): scores,
-// exponentials and the two accumulating products all queue in one instruction stream.  Here a
-// workgroup has eight waves, two per SIMD, for the same 128 keys:
+// dK/dV with the waves of a SIMD specialised.  A wave issues at most one instruction every 4-5
+// cycles; with scores, exponentials and both accumulating products in one instruction stream
+// (one wave per SIMD: 128 accumulator and 64 K/V-fragment registers leave no room for a second)
+// the kernel was bound by that rate.  Here a workgroup has eight waves, two per SIMD, for the
+// same 128 keys:
 //   waves 0-3 ("score" waves, 32 keys each, K and V fragments in registers) compute S = Q.K^T and
 //     dP = dO.V^T of a 32-query block, P and dS from them, and hand P, dS (bf16, already in the
 //     B-operand layout of the next products) to their partner through 4 KB of LDS;
@@ -778,11 +559,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
 // copies).  Two barriers per 64-query tile: after each, the accumulate waves pick up the block
 // the score waves finished before it, so the two kinds of work overlap with one block of lag.
 // Three LDS stages: tile it is read as rows by the score waves and transposed by the accumulate
-// waves during iteration it; tile it+1 is complete by the first barrier of iteration it (the
-// score waves start on it one block ahead); tile it+2 is requested after that barrier into the
-// stage tile it-1 left at it.
+// waves; every read of it is issued before the second barrier of iteration it, so tile it+3 is
+// requested right after that barrier into the same stage and has an iteration and a half to
+// land (it must be complete by the first barrier of iteration it+2: the score waves start on a
+// tile one block ahead).
+// PARTIAL = true: fp32 results for this query head go to part_k / part_v [b, nq, qsplit, s, 128].
 template <bool PARTIAL>
-__global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
+__global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ neg_lse2, const float* __restrict__ delta,
     bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
@@ -850,10 +633,29 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    // P = exp2(S c - lse), dS = P (dP - delta), handed to the partner wave
-    auto finish_block = [&](int stage, int sub, int qs0, f32x16& sacc, const f32x16& dpacc) {
+    // One step: P = exp2(S c - lse), dS = P (dP - delta) of block (stage, sub), handed to the
+    // partner wave, while the score products of the block after it (nstage, nsub) are issued.
+    // A wave's instructions issue in order and an MFMA waits for the matrix pipe, so sixteen
+    // MFMAs in a row stall the wave for as long as they take; four at a time between the four
+    // groups of exponentials they cost (almost) nothing.
+    auto step = [&](int stage, int sub, int qs0, f32x16& sacc, const f32x16& dpacc, int nstage, int nsub,
+                    f32x16& nsacc, f32x16& ndpacc) {
       const float* stats = reinterpret_cast<const float*>(reinterpret_cast<const char*>(smem) +
                                                           stage * STAGE + 2 * BT_BYTES);
+      uint32_t q_rows = lds0 + nstage * STAGE + bt_rows_lane(lane);
+      uint32_t do_rows = q_rows + BT_BYTES;
+      asm volatile("" : "+v"(q_rows), "+v"(do_rows));
+      bf16x8 qfr[HD / 16], dofr[HD / 16];
+#pragma unroll
+      for (int kk = 0; kk < HD / 16; ++kk) {
+        qfr[kk] = bt_rows(q_rows, nsub, kk);
+        dofr[kk] = bt_rows(do_rows, nsub, kk);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        nsacc[e] = 0.f;
+        ndpacc[e] = 0.f;
+      }
       // lane: key column krow, query rows qs0 + 8g + 4h + e; only blocks that reach the diagonal
       // pay for the causal mask
       if (qs0 < kw0 + 31) {
@@ -866,10 +668,16 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
         }
       }
       bf16x8 pb[2], dsb[2];
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const f32x4 l4 = *reinterpret_cast<const f32x4*>(stats + sub * 32 + 8 * g + 4 * h);
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(stats + 64 + sub * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int kk = 2 * g; kk < 2 * g + 2; ++kk) {
+          nsacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], nsacc, 0, 0, 0);
+          ndpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dofr[kk], vf[kk], ndpacc, 0, 0, 0);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[g * 4 + e], scale_log2, l4[e]));
@@ -877,6 +685,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
           pb[g >> 1][(g & 1) * 4 + e] = (bf16)p;
           dsb[g >> 1][(g & 1) * 4 + e] = (bf16)ds;
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
       const uint32_t xa = xch_lane + sub * 16384;
       *(KR_LDS bf16x8*)(xa) = pb[0];
@@ -884,20 +693,18 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
       *(KR_LDS bf16x8*)(xa + 2048) = dsb[0];
       *(KR_LDS bf16x8*)(xa + 3072) = dsb[1];
     };
-    // The score products of a block are issued one block ahead of the exponentials that consume
-    // them and run on the matrix pipe while the vector ALU works on the block before (the first
-    // block of the next tile during the second block of this one: that tile is complete by the
-    // first barrier of the iteration; behind the last tile it reads a stale stage, unused).
+    // The score products of a block are thus issued one block ahead of the exponentials that
+    // consume them (the first block of the next tile during the second block of this one: that
+    // tile is complete by the first barrier of the iteration; behind the last tile a stale
+    // stage is read, unused).
     f32x16 s0, dp0, s1, dp1;
     issue_scores(0, 0, s0, dp0);
     for (int it = 0; it < niter; ++it) {
       const int stage = it % NS;
       const int q0 = (qt_first + it * qsplit + part) * 64;
-      issue_scores(stage, 1, s1, dp1);
-      finish_block(stage, 0, q0, s0, dp0);
+      step(stage, 0, q0, s0, dp0, stage, 1, s1, dp1);
       __syncthreads();  // hand-over of block 0
-      issue_scores((it + 1) % NS, 0, s0, dp0);
-      finish_block(stage, 1, q0 + 32, s1, dp1);
+      step(stage, 1, q0 + 32, s1, dp1, (it + 1) % NS, 0, s0, dp0);
       __syncthreads();  // hand-over of block 1
     }
     return;
@@ -907,18 +714,50 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
   const bf16* qb = q + ql.at(bi, head, per);
   const bf16* dob = dout + dol.at(bi, head, per);
   const int64_t stat0 = ((int64_t)bi * nq + head) * s;
-  auto request_tile = [&](int it) {
-    const int qt = qt_first + it * qsplit + part;
-    const uint32_t tile = lds0 + (it % NS) * STAGE;
-    // the tile's 64 + 64 row statistics: one 4-byte-per-lane request each, by waves 0 and 1
-    if (wave < 2) {
-      int l2 = lane;
-      asm volatile("" : "+v"(l2));
-      dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + qt * 64, (uint32_t)l2 * 4u,
-              tile + 2 * BT_BYTES + wave * 256);
+  // A tile is brought in by nine requests per wave (eight for waves 2 and 3): the 64 + 64 row
+  // statistics, 4 bytes per lane, by waves 0 and 1, then four consecutive rows (+ 16, 32, 48
+  // through the lanes) of the Q tile and four of the dO tile.  request_begin names the tile,
+  // request_piece(i) issues piece i = 0..8, in this order (requests retire in order).
+  uint32_t req_tile = 0, req_lane_off = 0;
+  const bf16* req_row = nullptr;
+  int req_qt = 0;
+  auto request_begin = [&](int it) {
+    req_qt = qt_first + it * qsplit + part;
+    req_tile = lds0 + (it % NS) * STAGE;
+  };
+  auto request_piece = [&](int i) {
+    if (i == 0) {
+      if (wave < 2) {
+        int l2 = lane;
+        asm volatile("" : "+v"(l2));
+        dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + req_qt * 64, (uint32_t)l2 * 4u,
+                req_tile + 2 * BT_BYTES + wave * 256);
+      }
+      return;
     }
-    bt_request(qb + (int64_t)qt * 64 * ql.s_, ql.s_, tile, wave, lane);
-    bt_request(dob + (int64_t)qt * 64 * dol.s_, dol.s_, tile + BT_BYTES, wave, lane);
+    const int j = (i - 1) & 3;
+    const bool second = i > 4;
+    if (j == 0) {
+      int l2 = lane;
+      asm volatile("" : "+v"(l2));  // the lane offset lives only across the four requests of a tile
+      const int64_t ss = second ? dol.s_ : ql.s_;
+      req_lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
+      req_row = (second ? dob : qb) + ((int64_t)req_qt * 64 + 4 * wave) * ss;
+    }
+    dma_b128(req_row, req_lane_off, req_tile + (second ? BT_BYTES : 0) + (wave + 4 * j) * BT_BLK);
+    req_row += second ? dol.s_ : ql.s_;
+  };
+  auto request_tile = [&](int it) {
+    request_begin(it);
+#pragma unroll
+    for (int i = 0; i < 9; ++i) request_piece(i);
+  };
+  // wait until at most the requests of one tile (the newest) are in flight
+  auto wait_all_but_newest_tile = [&]() {
+    if (wave < 2)
+      __builtin_amdgcn_s_waitcnt(0x0f79);  // vmcnt(9)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
   };
   f32x16 dkacc[HD / 32], dvacc[HD / 32];
 #pragma unroll
@@ -930,44 +769,70 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_ws_kernel(
     }
   request_tile(0);
   if (niter > 1) request_tile(1);
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  if (niter > 2) {
+    request_tile(2);
+    wait_all_but_newest_tile();
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  }
   __syncthreads();
+  // The sixteen transposed fragments of a block (fr[8 k2 + 2 dt]: dO^T, fr[8 k2 + 2 dt + 1]: Q^T,
+  // queries 16 k2 .. of the block, channels 32 dt ..) live in registers across blocks: each is
+  // refilled for the next block right behind the MFMA that consumed it (one MFMA later), so the
+  // LDS reads of the next block ride under this block's matrix work and the wave reaches the
+  // next barrier with its operands already there.
+  const uint32_t cols_lane = bt_cols_lane(lane);
+  auto frag = [&](uint32_t stage_base, int sub, int f) {
+    const uint32_t base = stage_base + ((f & 1) ? 0u : BT_BYTES);  // odd: Q tile, even: dO tile
+    return bt_cols(base, 2 * sub + (f >> 3), (f >> 1) & 3);
+  };
+  bf16x8 fr[16];
+  {
+    uint32_t base = lds0 + cols_lane;
+    asm volatile("" : "+v"(base));
+#pragma unroll
+    for (int f = 0; f < 16; ++f) fr[f] = frag(base, 0, f);
+  }
   for (int it = 0; it < niter; ++it) {
     const int stage = it % NS;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
-      // the transposed fragments do not depend on the score waves: requested ahead of the barrier
-      uint32_t q_cols = lds0 + stage * STAGE + bt_cols_lane(lane);
-      uint32_t do_cols = q_cols + BT_BYTES;
-      asm volatile("" : "+v"(q_cols), "+v"(do_cols));
-      bf16x8 dot[2][HD / 32], qtr[2][HD / 32];
-#pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt) {
-          dot[k2][dt] = bt_cols(do_cols, 2 * sub + k2, dt);
-          qtr[k2][dt] = bt_cols(q_cols, 2 * sub + k2, dt);
-        }
-      // tile it+1 (requested after the first barrier of the iteration before) must have landed
-      // before this iteration's first barrier: the score waves start on it right after
-      if (sub == 0) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): nothing newer is in flight
+      // tile it+1 (requested an iteration and a half ago) must have landed before this
+      // iteration's first barrier: the score waves start on it right after.  Tile it+2 may still
+      // be on its way.
+      if (sub == 0) {
+        if (it + 2 < niter)
+          wait_all_but_newest_tile();
+        else
+          __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      }
       __syncthreads();
-      if (sub == 0 && it + 2 < niter) request_tile(it + 2);  // into the stage tile it-1 has left
+      // After the second barrier nobody reads tile it any more (this wave fetched its last
+      // fragments of it during the first block, the score waves before the first barrier):
+      // tile it+3 goes into its stage, one request behind each of the first MFMAs below.
+      const bool requesting = sub == 1 && it + 3 < niter;
+      if (requesting) request_begin(it + 3);
       const uint32_t xa = xch_lane + sub * 16384;
-      const bf16x8 pb0 = *(KR_LDS const bf16x8*)(xa);
-      const bf16x8 pb1 = *(KR_LDS const bf16x8*)(xa + 1024);
-      const bf16x8 ds0 = *(KR_LDS const bf16x8*)(xa + 2048);
-      const bf16x8 ds1 = *(KR_LDS const bf16x8*)(xa + 3072);
+      bf16x8 hand[4];  // P (queries 0-15, 16-31 of the block), dS (the same)
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt) {
-        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[0][dt], pb0, dvacc[dt], 0, 0, 0);
-        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[0][dt], ds0, dkacc[dt], 0, 0, 0);
-      }
+      for (int c = 0; c < 4; ++c) hand[c] = *(KR_LDS const bf16x8*)(xa + c * 1024);
+      // next block: the second of this tile, or the first of the next tile (complete since this
+      // iteration's first barrier; behind the last tile a stale stage, unused)
+      uint32_t next_base = lds0 + (sub == 0 ? stage : (it + 1) % NS) * STAGE + cols_lane;
+      asm volatile("" : "+v"(next_base));
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int dt = 0; dt < HD / 32; ++dt) {
-        dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dot[1][dt], pb1, dvacc[dt], 0, 0, 0);
-        dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[1][dt], ds1, dkacc[dt], 0, 0, 0);
+      for (int f = 0; f < 16; ++f) {
+        const int dt = (f >> 1) & 3;
+        if (f & 1)
+          dkacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], hand[2 + (f >> 3)], dkacc[dt], 0, 0, 0);
+        else
+          dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], hand[f >> 3], dvacc[dt], 0, 0, 0);
+        if (f > 0) fr[f - 1] = frag(next_base, sub ^ 1, f - 1);
+        if (requesting && f < 9) request_piece(f);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      fr[15] = frag(next_base, sub ^ 1, 15);
     }
   }
 
@@ -1172,18 +1037,9 @@ template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
   const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, bf16*, \
       float*, float*, int, int, int, int, float, float, QLayout, KLayout, KLayout, QLayout,      \
       KLayout, KLayout
-template __global__ void attn_bwd_dkdv_ws_kernel<false>(KR_ATTN_DKDV_ARGS);
-template __global__ void attn_bwd_dkdv_ws_kernel<true>(KR_ATTN_DKDV_ARGS);
+template __global__ void attn_bwd_dkdv_kernel<false>(KR_ATTN_DKDV_ARGS);
+template __global__ void attn_bwd_dkdv_kernel<true>(KR_ATTN_DKDV_ARGS);
 #undef KR_ATTN_DKDV_ARGS
-
-template __global__ void attn_bwd_dkdv_kernel<false>(const bf16*, const bf16*, const bf16*, const bf16*,
-                                                     const float*, const float*, bf16*, bf16*, float*,
-                                                     float*, int, int, int, int, float, float,
-                                                     QLayout, KLayout, KLayout, QLayout, KLayout, KLayout);
-template __global__ void attn_bwd_dkdv_kernel<true>(const bf16*, const bf16*, const bf16*, const bf16*,
-                                                    const float*, const float*, bf16*, bf16*, float*,
-                                                    float*, int, int, int, int, float, float,
-                                                    QLayout, KLayout, KLayout, QLayout, KLayout, KLayout);
 
 }  // namespace
 
@@ -1231,8 +1087,7 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   const int qsplit = dkdv_query_split(s, b, nq);
   float* part_v = part_k + rows * qsplit * hd;
   const bool partial = nq != nkv || qsplit > 1;
-  constexpr size_t lds_dkdv = 4 * (2 * BT_BYTES + 512);  // four stages: Q tile, dO tile, statistics
-  constexpr size_t lds_dkdv_ws = 3 * (2 * BT_BYTES + 512) + 32768;  // three stages + the hand-over area
+  constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512) + 32768;  // three stages + the hand-over area
   constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
@@ -1240,12 +1095,6 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
     if (e == hipSuccess)
       e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_ws_kernel<false>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv_ws);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_ws_kernel<true>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv_ws);
     if (e == hipSuccess)
       e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
@@ -1262,43 +1111,22 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
   const dim3 grid_kv((s / 128) * nq * b * qsplit);
-  const char* const ws_env = getenv("KR_DKDV_WS");  // experiment switch
-  const bool use_ws = ws_env != nullptr && ws_env[0] == '1';
-  if (use_ws) {
-#define KR_DKDV_WS_LAUNCH(P)                                                                        \
-  hipLaunchKernelGGL((attn_bwd_dkdv_ws_kernel<P>), grid_kv, dim3(512), lds_dkdv_ws, st,             \
-                     (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout,             \
-                     (const float*)neg_lse2, (const float*)delta, (bf16*)dk, (bf16*)dv, part_k,     \
-                     part_v, s, nq, nkv, partial ? qsplit : 1, scale, scale_log2, ql, kl, vl, dol, \
-                     dkl, dvl)
-    if (partial) {
-      KR_DKDV_WS_LAUNCH(true);
-      if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
-      const int64_t total = (int64_t)b * nkv * s * 16;
-      hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                         st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
-                         nkv, qsplit, total, dkl, dvl);
-    } else {
-      KR_DKDV_WS_LAUNCH(false);
-    }
-#undef KR_DKDV_WS_LAUNCH
-  } else if (partial) {
-    hipLaunchKernelGGL(attn_bwd_dkdv_kernel<true>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
-                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,
-                       (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, qsplit, scale,
-                       scale_log2, ql,
-                       kl, vl, dol, dkl, dvl);
+#define KR_DKDV_LAUNCH(P)                                                                           \
+  hipLaunchKernelGGL((attn_bwd_dkdv_kernel<P>), grid_kv, dim3(512), lds_dkdv, st, (const bf16*)q,   \
+                     (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,     \
+                     (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv,         \
+                     partial ? qsplit : 1, scale, scale_log2, ql, kl, vl, dol, dkl, dvl)
+  if (partial) {
+    KR_DKDV_LAUNCH(true);
     if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
     const int64_t total = (int64_t)b * nkv * s * 16;
     hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                        st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
                        nkv, qsplit, total, dkl, dvl);
   } else {
-    hipLaunchKernelGGL(attn_bwd_dkdv_kernel<false>, grid_kv, dim3(256), lds_dkdv, st, (const bf16*)q,
-                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,
-                       (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv, 1, scale, scale_log2, ql, kl,
-                       vl, dol, dkl, dvl);
+    KR_DKDV_LAUNCH(false);
   }
+#undef KR_DKDV_LAUNCH
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int dq_blocks = (s / BQ) * nq * b;
   if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
