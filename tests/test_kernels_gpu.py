@@ -205,7 +205,9 @@ def _grouped(s, b, nq, nkv, hd, seed):
     return fused, fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1]
 
 
-@pytest.mark.parametrize("s,b,nq,nkv", [(128, 1, 1, 1), (256, 2, 4, 2), (512, 1, 3, 1), (384, 1, 8, 8), (1024, 1, 4, 1)])
+@pytest.mark.parametrize("s,b,nq,nkv", [(128, 1, 1, 1), (256, 2, 4, 2), (512, 1, 3, 1), (384, 1, 8, 8), (1024, 1, 4, 1),
+                                        (2048, 1, 2, 1),    # 32 query tiles per key tile: the steady state of the pipelines
+                                        (512, 17, 8, 8)])   # 544 workgroups, one query head per KV head: dK/dV written directly
 def test_attention_forward_backward(be, s, b, nq, nkv):
     hd = 128
     _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=22)
