@@ -800,18 +800,26 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
       // tile it+1 (requested an iteration and a half ago) must have landed before this
       // iteration's first barrier: the score waves start on it right after.  Tile it+2 may still
       // be on its way.
-      if (sub == 0) {
-        if (it + 2 < niter)
-          wait_all_but_newest_tile();
-        else
+      if (sub == 0 && it > 0) {  // (tiles 0 and 1 were awaited before the loop)
+        if (it + 2 < niter) {
+          // in flight behind tile it+1: the first five pieces of tile it+2
+          if (wave < 2)
+            __builtin_amdgcn_s_waitcnt(0x0f75);  // vmcnt(5)
+          else
+            __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+        } else {
           __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        }
       }
       __syncthreads();
       // After the second barrier nobody reads tile it any more (this wave fetched its last
       // fragments of it during the first block, the score waves before the first barrier):
-      // tile it+3 goes into its stage, one request behind each of the first MFMAs below.
-      const bool requesting = sub == 1 && it + 3 < niter;
-      if (requesting) request_begin(it + 3);
+      // tile it+3 goes into its stage, one request behind each of the first MFMAs — pieces 0-4
+      // in this block, pieces 5-8 in the first block of the next iteration, so that neither
+      // block of the accumulate waves outlasts the score waves' step beside it.
+      const bool first_pieces = sub == 1 && it + 3 < niter;
+      const bool last_pieces = sub == 0 && it > 0 && it + 2 < niter;
+      if (first_pieces) request_begin(it + 3);
       const uint32_t xa = xch_lane + sub * 16384;
       bf16x8 hand[4];  // P (queries 0-15, 16-31 of the block), dS (the same)
 #pragma unroll
@@ -829,7 +837,8 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
         else
           dvacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], hand[f >> 3], dvacc[dt], 0, 0, 0);
         if (f > 0) fr[f - 1] = frag(next_base, sub ^ 1, f - 1);
-        if (requesting && f < 9) request_piece(f);
+        if (first_pieces && f < 5) request_piece(f);
+        if (last_pieces && f < 4) request_piece(5 + f);
         __builtin_amdgcn_sched_barrier(0);
       }
       fr[15] = frag(next_base, sub ^ 1, 15);
