@@ -545,10 +545,10 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict_
 }
 
 // dK/dV with the waves of a SIMD specialised.  A wave issues at most one instruction every 4-5
-// cycles; with scores, exponentials and both accumulating products in one instruction stream
-// (one wave per SIMD: 128 accumulator and 64 K/V-fragment registers leave no room for a second)
-// the kernel was bound by that rate.  Here a workgroup has eight waves, two per SIMD, for the
-// same 128 keys:
+// cycles, and one wave that does everything for its 32 keys (scores, exponentials, both
+// accumulating products) needs 128 accumulator and 64 K/V-fragment registers — no room for a
+// second wave on the SIMD — so it is bound by that rate: 850 instructions per 64 MFMAs.  Instead
+// a workgroup has eight waves, two per SIMD, for its 128 keys:
 //   waves 0-3 ("score" waves, 32 keys each, K and V fragments in registers) compute S = Q.K^T and
 //     dP = dO.V^T of a 32-query block, P and dS from them, and hand P, dS (bf16, already in the
 //     B-operand layout of the next products) to their partner through 4 KB of LDS;
