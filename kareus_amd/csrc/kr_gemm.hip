@@ -49,9 +49,10 @@ namespace {
 
 constexpr int BK = 64;
 constexpr int BM = 256, BN = 256;
-constexpr int TM = 4, TN = 2;  // 32x32 MFMA tiles per wave: 128 rows x 64 columns
-constexpr int NTHREADS = 512;
+constexpr int WT = 8;  // 16x16 MFMA tiles per wave along each dimension: a wave owns 128 x 128 of C
+constexpr int NTHREADS = 256;
 constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
+constexpr uint32_t SLOT_BYTES = TILE * sizeof(bf16);
 constexpr int NSLOTS = 5;          // 5 x 32 KB = the whole 160 KB of LDS
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;
@@ -61,153 +62,108 @@ constexpr int kGroupM = 4;
 __device__ __forceinline__ int kmajor_off(int row, int chunk) {
   return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
 }
-// transposed tile [64 k-rows][256]: 512-byte rows, chunk index XORed with 4*(krow&3).
+// transposed tile [64 k-rows][256]: 512-byte rows, 16-byte chunk index XORed with a value made of
+// k-row bits 0, 1 (the four k-rows one 16-lane group reads together) and bit 3 (the two groups
+// of a 32-lane half read k-rows 8 apart).
+__device__ __forceinline__ int transp_swz(int krow) { return ((krow & 3) << 2) | (((krow >> 3) & 1) << 1); }
 __device__ __forceinline__ int transp_off(int krow, int col) {
-  return krow * 256 + ((((col >> 3) ^ ((krow & 3) << 2))) << 3) + (col & 7);
+  return krow * 256 + (((col >> 3) ^ transp_swz(krow)) << 3) + (col & 7);
 }
 
 // ---- direct global -> LDS loads ---------------------------------------------------------------
 // Issued through inline assembly on purpose.  A workgroup barrier is a release fence for LDS,
 // and the compiler drains every LDS-direct load it knows of (vmcnt(0)) in front of one — which
-// would empty the prefetch pipeline twice per K-step.  Written this way the loads are invisible
+// would empty the prefetch pipeline once per K-step.  Written this way the loads are invisible
 // to its wait-count bookkeeping; their completion is tracked by hand with explicit vmcnt waits
 // placed before the barrier that publishes the data.  The loads have no register destination,
 // so nothing can be clobbered behind the register allocator's back.
 // base: wave-uniform global address; byte_off: this lane's unsigned 32-bit byte offset from it;
-// lds_byte: wave-uniform LDS byte address of a 1-KiB block (lane p lands at +16p).
-__device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, uint32_t lds_byte) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+// lds_base + IMM: wave-uniform LDS byte address of a 1-KiB block (lane p lands at +16p).
+template <int IMM>
+__device__ __forceinline__ void dma_b128(const void* base, uint32_t byte_off, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(lds_byte), "v"(byte_off), "s"(base)
-               : "memory", "m0");
+               : "s"(lds_base), "v"(byte_off), "s"(base), "n"(IMM)
+               : "memory", "m0", "scc");
 }
 __device__ __forceinline__ uint32_t lds_addr(const bf16* p) {
   return (uint32_t)(uintptr_t)(KR_LDS const bf16*)p;
 }
 
-// ---- direct global -> LDS tile loads, issued by the 4 waves of the loading group -----------
-// One wave-level load moves 1 KiB into LDS at [base + lane*16].  Block b of a K-major tile
-// holds rows 8b..8b+7; block b of a transposed tile holds contraction rows 2b, 2b+1.
+// ---- which 16-byte chunk a lane fetches ------------------------------------------------------
+// The four waves share every operand tile: wave w issues loads i = 0..7, load i fills the 1-KiB
+// block w + 4 i.  Block b of a K-major tile holds rows 8b..8b+7; block b of a transposed tile
+// holds contraction rows 2b, 2b+1.  The swizzle is applied on the global side: each lane
+// fetches the chunk that belongs at its LDS position.
+// Returns the element offset from the K-step's base pointer.  Rows beyond the matrix are
+// clamped to the last valid row; a chunk that would start beyond the contraction range
+// (k_left = elements from the K-step's base to the end, >= 8) is redirected to a valid address —
+// it is zeroed in LDS afterwards, so what it fetches does not matter.
 template <bool TRANSPOSED>
-struct TileLoader {
-  // K-major:    load i covers tile row r0 + 32*i (clamped to rmax), 16-byte chunk `chunk`
-  // transposed: load i covers contraction row k0 + 8*i, column offset `chunk` (clamped)
-  int r0, rmax, chunk;
-  int64_t ld;
-  __device__ __forceinline__ void init(int64_t ld_, int row0, int rows_total, int wave4, int lane) {
-    ld = ld_;
-    if (!TRANSPOSED) {
-      const int row = 8 * wave4 + (lane >> 3);  // + 32*i; (row >> 1) & 7 does not depend on i
-      chunk = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
-      r0 = row0 + row;
-      rmax = rows_total - 1;
-    } else {
-      const int krow = 2 * wave4 + (lane >> 5);  // + 8*i; krow & 3 does not depend on i
-      int c = row0 + ((lane & 31) ^ ((krow & 3) << 2)) * 8;
-      chunk = c + 8 <= rows_total ? c : rows_total - 8;
-      r0 = krow;
-      rmax = 0;
-    }
+__device__ __forceinline__ uint32_t load_offset(int i, int wave, int lane, int ld, int row0,
+                                                int rows_total, int k_left) {
+  if (!TRANSPOSED) {
+    const int row = 8 * wave + (lane >> 3) + 32 * i;
+    int chunk = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
+    int r = row0 + row;
+    r = r < rows_total ? r : rows_total - 1;
+    chunk = chunk + 8 <= k_left ? chunk : k_left - 8;
+    return (uint32_t)(r * ld + chunk);
   }
-  // k_left: contraction elements from this K-step's base to the end of the operand (>= 8).
-  // A chunk that would start beyond it is redirected to a valid address; it is zeroed in LDS
-  // afterwards, so what it fetches does not matter — only that the address is inside the matrix.
-  __device__ __forceinline__ uint32_t goff(int i, int k_left) const {
-    if (!TRANSPOSED) {
-      int r = r0 + 32 * i;
-      r = r < rmax ? r : rmax;
-      const int kc = chunk + 8 <= k_left ? chunk : k_left - 8;
-      return (uint32_t)(r * (int)ld + kc);
-    }
-    int kr = r0 + 8 * i;
-    kr = kr < k_left ? kr : k_left - 1;
-    return (uint32_t)(kr * (int)ld + chunk);
+  int krow = 2 * wave + (lane >> 5) + 8 * i;
+  int c = row0 + ((lane & 31) ^ transp_swz(krow)) * 8;
+  c = c + 8 <= rows_total ? c : rows_total - 8;
+  krow = krow < k_left ? krow : k_left - 1;
+  return (uint32_t)(krow * ld + c);
+}
+// contraction index (relative to the K-step) of the chunk that load i of this lane fills
+template <bool TRANSPOSED>
+__device__ __forceinline__ int load_k(int i, int wave, int lane) {
+  if (!TRANSPOSED) {
+    const int row = 8 * wave + (lane >> 3);  // (row >> 1) & 7 does not depend on i
+    return ((lane & 7) ^ ((row >> 1) & 7)) * 8;
   }
-  // contraction index (relative to the K-step) covered by load i of this lane
-  __device__ __forceinline__ int k_of(int i, int wave4, int lane) const {
-    if (!TRANSPOSED) {
-      const int row = 8 * wave4 + (lane >> 3);
-      return ((lane & 7) ^ ((row >> 1) & 7)) * 8;
-    }
-    return 2 * (wave4 + 4 * i) + (lane >> 5);
-  }
-  __device__ __forceinline__ void issue_one(const bf16* __restrict__ kbase, bf16* tile, int wave4,
-                                            int k_left, int i) const {
-    dma_b128(kbase, goff(i, k_left) * 2u, lds_addr(tile + (wave4 + 4 * i) * 512));
-  }
-  __device__ __forceinline__ void issue(const bf16* __restrict__ kbase, bf16* tile, int wave4,
-                                        int k_left) const {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int b = wave4 + 4 * i;
-      dma_b128(kbase, goff(i, k_left) * 2u, lds_addr(tile + b * 512));
-    }
-  }
-  // zero this lane's chunks whose contraction index is >= k_valid (tile already landed)
-  __device__ __forceinline__ void zero_tail(bf16* tile, int k_valid, int wave4, int lane) const {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int b = wave4 + 4 * i;
-      if (k_of(i, wave4, lane) >= k_valid)
-        *reinterpret_cast<bf16x8*>(tile + b * 512 + lane * 8) = zero8();
-    }
-  }
-};
+  return 2 * wave + (lane >> 5) + 8 * i;
+}
 
 // ---- LDS -> MFMA operand fragments ----------------------------------------------------------
-// Fragment (t, kk): lane gets tile row (row0 + 32*t + lane%32), k = 16*kk + 8*(lane/32) + 0..7.
-// Per-lane base offsets are computed once; everything that varies inside the K loop is an
-// instruction immediate.
-template <bool TRANSPOSED, int NTILES>
+// v_mfma_f32_16x16x32_bf16 wants from lane l the 8 contraction elements 8 (l / 16) .. + 7 of
+// operand row l % 16.  Fragment (g, h): operand rows row0 + 16 g .., contraction half h (32
+// elements) of the K-step.
+template <bool TRANSPOSED>
 struct FragReader {
-  // K-major: one base per kk (the swizzle XOR depends on kk), tile index t is an immediate
-  // transposed: one base per t (the XOR depends on the column), kk / half are immediates
-  int base[TRANSPOSED ? NTILES : BK / 16];
+  // K-major: one base per half (the swizzle XOR depends on the chunk), g is an immediate
+  // transposed: one base per g (the XOR depends on the column), the half is an immediate
+  static constexpr int NBASE = TRANSPOSED ? WT : 2;
+  uint32_t base[NBASE];  // byte offsets inside a tile
   __device__ __forceinline__ void init(int row0, int lane) {
     if (!TRANSPOSED) {
-      const int row = row0 + (lane & 31);
 #pragma unroll
-      for (int kk = 0; kk < BK / 16; ++kk) base[kk] = kmajor_off(row, 2 * kk + (lane >> 5));
+      for (int h = 0; h < 2; ++h) base[h] = 2u * (uint32_t)kmajor_off(row0 + (lane & 15), 4 * h + (lane >> 4));
     } else {
+      // transposing read: within each group of 16 lanes, lane p supplies the address of 4
+      // consecutive operand rows in contraction row p / 4 and receives, for operand row p, the
+      // elements of the group's 4 contraction rows
       const int p = lane & 15;
-      const int krow = (lane >> 5) * 8 + (p >> 2);
+      const int krow = 8 * (lane >> 4) + (p >> 2);
 #pragma unroll
-      for (int t = 0; t < NTILES; ++t)
-        base[t] = transp_off(krow, row0 + 32 * t + ((lane >> 4) & 1) * 16 + (p & 3) * 4);
-    }
-  }
-  // LDS byte address of this lane's base n inside `tile`, made opaque so that the compiler adds
-  // nothing but instruction immediates (all below 64 KiB) to it and keeps no per-slot copies.
-  __device__ __forceinline__ uint32_t addr(const bf16* tile, int n) const {
-    uint32_t v = (uint32_t)(uintptr_t)(KR_LDS const bf16*)tile + 2u * (uint32_t)base[n];
-    asm volatile("" : "+v"(v));
-    return v;
-  }
-  static constexpr int NBASE = TRANSPOSED ? NTILES : BK / 16;
-  // a[]: addr(tile, n) for every base n
-  __device__ __forceinline__ bf16x8 read(const uint32_t (&a)[NBASE], int t, int kk) const {
-    if (!TRANSPOSED) {
-      return *(KR_LDS const bf16x8*)(a[kk] + 2u * (uint32_t)(t * 32 * BK));
-    } else {
-      // Transposing read: within each group of 16 lanes, lane p supplies the address of 4
-      // consecutive row-of-C elements in contraction row (p/4); it receives, for its own
-      // row-of-C, the elements of the group's 4 contraction rows.
-      const uint32_t a0 = a[t] + 2u * (uint32_t)(kk * 16 * 256);
-      union {
-        struct { s16x4 lo, hi; } s;
-        bf16x8 v;
-      } u;
-      u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
-      u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 2u * 4 * 256));
-      return u.v;
+      for (int g = 0; g < WT; ++g) base[g] = 2u * (uint32_t)transp_off(krow, row0 + 16 * g + (p & 3) * 4);
     }
   }
 };
-
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+// slot: LDS byte address of the tile; for K-major operands `a` is slot + base[h] (opaque)
+__device__ __forceinline__ bf16x8 frag_kmajor(uint32_t a, int g) {
+  return *(KR_LDS const bf16x8*)(a + (uint32_t)(g * 16 * BK * 2));
+}
+__device__ __forceinline__ bf16x8 frag_transp(uint32_t a, int h) {
+  const uint32_t a0 = a + (uint32_t)(h * 32 * 256 * 2);
+  union {
+    struct { s16x4 lo, hi; } s;
+    bf16x8 v;
+  } u;
+  u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0));
+  u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a0 + 2u * 4 * 256));
+  return u.v;
 }
 
 __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, int tiles_n,
@@ -226,6 +182,12 @@ __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, i
   tn = in_band / band_rows;
 }
 
+struct Frags {
+  bf16x8 a[WT], b[WT];
+};
+struct Yes { static constexpr bool value = true; };
+struct No { static constexpr bool value = false; };
+
 template <bool A_T, bool B_T>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
@@ -235,12 +197,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int group = wave >> 2;  // 0: computes first and requests the B tiles, 1: the A tiles
-  const int wave4 = wave & 3;
-  const int wm = group, wn = wave4;  // wave tile: rows wm*128.., columns wn*64..
+  const int wm = wave >> 1, wn = wave & 1;  // wave tile: rows wm*128.., columns wn*128..
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const bool split_k = partial != nullptr;
+  const uint32_t smem_b = lds_addr(smem);
+  const uint32_t wave_blk = (uint32_t)wave * 1024u;
 
   // Persistent workgroups: work item v = (output tile, split-K range); this workgroup takes
   // items blockIdx.x, blockIdx.x + gridDim.x, ...  The state below describes the current item.
@@ -262,341 +224,315 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       p_off = split * M * N;
     }
     nk = (kc + BK - 1) / BK;
-    k_tail = kc - (nk - 1) * BK;  // valid contraction rows of the last K-step (1..64)
+    k_tail = kc - (nk - 1) * BK;  // valid contraction rows of the last K-step (8..64)
+  };
+  auto a_base = [&](int t) { return A + a_off + (int64_t)t * (A_T ? BK * lda : BK); };
+  auto b_base = [&](int t) { return B + b_off + (int64_t)t * (B_T ? BK * ldb : BK); };
+
+  // The ring of five 32 KB slots as LDS byte addresses, in ring order starting at A of the
+  // current K-step t: r0 = A(t), r1 = B(t), r2 = A(t+1), r3 = B(t+1), r4 = A(t+2); B(t+2) goes
+  // where A(t) was.  Rotated by two positions per K-step.
+  uint32_t r0 = smem_b, r1 = smem_b + SLOT_BYTES, r2 = smem_b + 2 * SLOT_BYTES,
+           r3 = smem_b + 3 * SLOT_BYTES, r4 = smem_b + 4 * SLOT_BYTES;
+  auto rotate = [&]() {
+    const uint32_t o0 = r0, o1 = r1;
+    r0 = r2; r1 = r3; r2 = r4; r3 = o0; r4 = o1;
   };
 
-  f32x16 acc[TN][TM];
-  bf16x8 af[BK / 16][TM], bfr[BK / 16][TN];
+  // accumulators live in the accumulation registers (the MFMAs are written as inline assembly
+  // with that register class, see mfma() below); fragments in ordinary vector registers
+  f32x4 acc[WT][WT];
+  Frags X, Y;
+  uint32_t la[8], lb[8];  // byte offsets of this lane's chunk in the 8 loads of an A / a B tile
 
-  // Per-lane fragment offsets are recomputed from an opaque copy of the lane id whenever
-  // fragments are read (a handful of VALU instructions in the data-movement half-period)
-  // instead of occupying eight registers through the MFMA phases.
-  auto read_frags = [&](int t) {
-    int lf = lane;
-    asm volatile("" : "+v"(lf));
-    FragReader<A_T, TM> fa;
-    FragReader<B_T, TN> fb;
-    fa.init(wm * TM * 32, lf);
-    fb.init(wn * TN * 32, lf);
-    const bf16* at = smem + ((2 * t) % NSLOTS) * TILE;
-    const bf16* bt = smem + ((2 * t + 1) % NSLOTS) * TILE;
-    uint32_t aa[fa.NBASE], ba[fb.NBASE];
-#pragma unroll
-    for (int n = 0; n < fa.NBASE; ++n) aa[n] = fa.addr(at, n);
-#pragma unroll
-    for (int n = 0; n < fb.NBASE; ++n) ba[n] = fb.addr(bt, n);
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i) af[kk][i] = fa.read(aa, i, kk);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) bfr[kk][j] = fb.read(ba, j, kk);
-    }
-  };
-  auto compute = [&]() {
-    __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-          acc[j][i] =
-              __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[kk][j], af[kk][i], acc[j][i], 0, 0, 0);
-    __builtin_amdgcn_s_setprio(0);
-  };
-
-  // LDS is a ring of five 32 KB slots; operand tile x (0 = A, 1 = B) of K-step t lives in slot
-  // (2t + x) mod 5.  Two slots hold the K-step being consumed, three are being filled.
-  auto slot_of = [&](int t, int x) { return smem + ((2 * t + x) % NSLOTS) * TILE; };
-  // Each group loads one operand: group 1 the A tiles, group 0 the B tiles, 8 loads per wave.
-  // The per-lane load coordinates are recomputed from an opaque copy of the lane id every time:
-  // keeping them alive across the MFMA phases would push the wave over its register budget.
-  auto issue_mine = [&](int t) {
+  auto set_offsets = [&](int k_left) {
     int l2 = lane;
     asm volatile("" : "+v"(l2));
-    if (group) {
-      TileLoader<A_T> la;
-      la.init(lda, m0, M, wave4, l2);
-      la.issue(A + a_off + (int64_t)t * (A_T ? BK * lda : BK), slot_of(t, 0), wave4, kc - t * BK);
-    } else {
-      TileLoader<B_T> lb;
-      lb.init(ldb, n0, N, wave4, l2);
-      lb.issue(B + b_off + (int64_t)t * (B_T ? BK * ldb : BK), slot_of(t, 1), wave4, kc - t * BK);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      la[i] = 2u * load_offset<A_T>(i, wave, l2, lda, m0, M, k_left);
+      lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left);
     }
   };
-  // The data-movement half-period: read this wave's fragments of K-step t_read and request
-  // this wave's 8 blocks of K-step t_load, one request after every third fragment read.  The
-  // texture-address path takes about as long to accept a group's 32 KB as LDS takes to deliver
-  // its fragments; back to back the two would outlast the other group's MFMA burst, woven
-  // together they fit inside it.
-  auto move_data = [&](int t_read, int t_load) {
-    int lf = lane;
-    asm volatile("" : "+v"(lf));
-    FragReader<A_T, TM> fa;
-    FragReader<B_T, TN> fb;
-    fa.init(wm * TM * 32, lf);
-    fb.init(wn * TN * 32, lf);
-    const bf16* at = smem + ((2 * t_read) % NSLOTS) * TILE;
-    const bf16* bt = smem + ((2 * t_read + 1) % NSLOTS) * TILE;
-    uint32_t aa[fa.NBASE], ba[fb.NBASE];
+  auto request = [&](const bf16* base, const uint32_t (&off)[8], uint32_t slot) {
+    const uint32_t dst = slot + wave_blk;
+    dma_b128<0 * 4096>(base, off[0], dst);
+    dma_b128<1 * 4096>(base, off[1], dst);
+    dma_b128<2 * 4096>(base, off[2], dst);
+    dma_b128<3 * 4096>(base, off[3], dst);
+    dma_b128<4 * 4096>(base, off[4], dst);
+    dma_b128<5 * 4096>(base, off[5], dst);
+    dma_b128<6 * 4096>(base, off[6], dst);
+    dma_b128<7 * 4096>(base, off[7], dst);
+  };
+  // K-steps 0 and 1 of the current item into r0..r3
+  auto request_first_two = [&]() {
+    set_offsets(nk == 1 ? k_tail : BK);
+    request(a_base(0), la, r0);
+    request(b_base(0), lb, r1);
+    if (nk > 1) {
+      if (nk == 2 && k_tail != BK) set_offsets(k_tail);
+      request(a_base(1), la, r2);
+      request(b_base(1), lb, r3);
+    }
+  };
+  // After this wave's loads of the last K-step have landed (A in slot sa, B in slot sb): zero
+  // the chunks beyond the contraction range.
+  auto fix_tail = [&](uint32_t sa, uint32_t sb) {
+    if (k_tail == BK) return;
+    int l2 = lane;
+    asm volatile("" : "+v"(l2));
 #pragma unroll
-    for (int n = 0; n < fa.NBASE; ++n) aa[n] = fa.addr(at, n);
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t blk = (uint32_t)(wave + 4 * i) * 1024u + (uint32_t)l2 * 16u;
+      if (load_k<A_T>(i, wave, l2) >= k_tail) *(KR_LDS bf16x8*)(sa + blk) = zero8();
+      if (load_k<B_T>(i, wave, l2) >= k_tail) *(KR_LDS bf16x8*)(sb + blk) = zero8();
+    }
+  };
+
+  // fragment addressing, recomputed per item from an opaque copy of the lane id so that it is
+  // not live through the epilogue
+  FragReader<A_T> fa;
+  FragReader<B_T> fb;
+  // addresses for reading half h of the tiles in slots sa / sb
+  auto frag_addrs = [&](uint32_t sa, uint32_t sb, int h, uint32_t (&aa)[FragReader<A_T>::NBASE],
+                        uint32_t (&ba)[FragReader<B_T>::NBASE]) {
+    if (!A_T) {
+      aa[0] = sa + fa.base[h];
+      asm volatile("" : "+v"(aa[0]));
+    } else {
 #pragma unroll
-    for (int n = 0; n < fb.NBASE; ++n) ba[n] = fb.addr(bt, n);
-    auto body = [&](const auto& loader, const bf16* kbase, bf16* dst) {
-      const int k_left = kc - t_load * BK;
-#pragma unroll
-      for (int kk = 0; kk < BK / 16; ++kk) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          af[kk][i] = fa.read(aa, i, kk);
-          const int n = kk * (TM + TN) + i;
-          if (n % 3 == 2) loader.issue_one(kbase, dst, wave4, k_left, n / 3);
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          bfr[kk][j] = fb.read(ba, j, kk);
-          const int n = kk * (TM + TN) + TM + j;
-          if (n % 3 == 2) loader.issue_one(kbase, dst, wave4, k_left, n / 3);
-        }
+      for (int g = 0; g < WT; ++g) {
+        aa[g] = sa + fa.base[g];
+        asm volatile("" : "+v"(aa[g]));
       }
-    };
-    int l2 = lane;
-    asm volatile("" : "+v"(l2));
-    if (group) {
-      TileLoader<A_T> la;
-      la.init(lda, m0, M, wave4, l2);
-      body(la, A + a_off + (int64_t)t_load * (A_T ? BK * lda : BK), slot_of(t_load, 0));
+    }
+    if (!B_T) {
+      ba[0] = sb + fb.base[h];
+      asm volatile("" : "+v"(ba[0]));
     } else {
-      TileLoader<B_T> lb;
-      lb.init(ldb, n0, N, wave4, l2);
-      body(lb, B + b_off + (int64_t)t_load * (B_T ? BK * ldb : BK), slot_of(t_load, 1));
+#pragma unroll
+      for (int g = 0; g < WT; ++g) {
+        ba[g] = sb + fb.base[g];
+        asm volatile("" : "+v"(ba[g]));
+      }
     }
   };
-  // After this wave's loads of tile t have landed: zero a contraction tail of the last K-step.
-  auto fix_tail_mine = [&](int t) {
-    if (t != nk - 1 || k_tail == BK) return;
-    int l2 = lane;
-    asm volatile("" : "+v"(l2));
-    if (group) {
-      TileLoader<A_T> la;
-      la.init(lda, m0, M, wave4, l2);
-      la.zero_tail(slot_of(t, 0), k_tail, wave4, l2);
-    } else {
-      TileLoader<B_T> lb;
-      lb.init(ldb, n0, N, wave4, l2);
-      lb.zero_tail(slot_of(t, 1), k_tail, wave4, l2);
+  auto read_a = [&](const uint32_t (&aa)[FragReader<A_T>::NBASE], int g, int h) {
+    if constexpr (!A_T) return frag_kmajor(aa[0], g); else return frag_transp(aa[g], h);
+  };
+  auto read_b = [&](const uint32_t (&ba)[FragReader<B_T>::NBASE], int g, int h) {
+    if constexpr (!B_T) return frag_kmajor(ba[0], g); else return frag_transp(ba[g], h);
+  };
+
+  // One half-step: the 64 MFMAs of one 32-element half of a K-step on `cur`, with the 16
+  // fragment reads of the next half-step (half h of the tiles in slots sa / sb, into `nxt`) and,
+  // if DMA, the 8 requests of one operand tile woven in between in exactly this order.  The
+  // operands are swapped (the B fragment feeds the instruction's A port), so a lane ends up
+  // with four consecutive columns of one row of C.
+  auto half = [&](Frags& cur, Frags& nxt, uint32_t sa, uint32_t sb, int h, auto dma_tag,
+                  const bf16* dbase, const uint32_t (&doff)[8], uint32_t dslot) {
+    uint32_t aa[FragReader<A_T>::NBASE], ba[FragReader<B_T>::NBASE];
+    frag_addrs(sa, sb, h, aa, ba);
+    const uint32_t dst = dslot + wave_blk;
+#pragma unroll
+    for (int g = 0; g < WT; ++g) {
+#pragma unroll
+      for (int nt = 0; nt < WT; ++nt) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                     : "+a"(acc[g][nt])
+                     : "v"(cur.b[nt]), "v"(cur.a[g]));
+        if (nt == 0) nxt.a[g] = read_a(aa, g, h);
+        if (nt == 2) nxt.b[g] = read_b(ba, g, h);
+        if constexpr (decltype(dma_tag)::value) {
+          if (nt == 4) {
+            if (g == 0) dma_b128<0 * 4096>(dbase, doff[0], dst);
+            if (g == 1) dma_b128<1 * 4096>(dbase, doff[1], dst);
+            if (g == 2) dma_b128<2 * 4096>(dbase, doff[2], dst);
+            if (g == 3) dma_b128<3 * 4096>(dbase, doff[3], dst);
+            if (g == 4) dma_b128<4 * 4096>(dbase, doff[4], dst);
+            if (g == 5) dma_b128<5 * 4096>(dbase, doff[5], dst);
+            if (g == 6) dma_b128<6 * 4096>(dbase, doff[6], dst);
+            if (g == 7) dma_b128<7 * 4096>(dbase, doff[7], dst);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
-  // Two barriers per K-step delimit the half-periods.  The one in the middle of a K-step (after
-  // it, group 1 computes and group 0 moves) orders every LDS hazard: data of the next K-step
-  // visible, slots of the current one free.  The one at the start of a K-step only keeps the two
-  // groups' MFMA bursts apart; every slot a group overwrites after it was last read before the
-  // previous middle barrier.  With a transposed B operand the kernel is a little faster when the
-  // hand-over at the start is left to the hardware (the next burst may begin while the last one
-  // drains); with both operands K-major it is clearly slower, so there the barrier stays.
-  constexpr bool kFreeHandoff = B_T;
   const int total_items = ntiles * (split_k ? splits : 1);
   int item = blockIdx.x;
   select_item(item);
-  // K-steps 0 and 1 of the first item
-  issue_mine(0);
-  if (nk > 1) issue_mine(1);
+  request_first_two();
 
   for (;;) {
-  // K-steps 0 and 1 complete in LDS (requested above, or before the previous item's epilogue)
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); lgkmcnt and expcnt untouched
-  if (nk == 1) fix_tail_mine(0);
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[j][i][e] = 0.f;
-
-  if (group == 0) {
-    read_frags(0);
-    for (int ks = 0; ks < nk; ++ks) {
-      // half-period 2ks: this group computes, the other moves data
-      if (!kFreeHandoff) lds_barrier();
-      compute();
-      if (ks + 1 < nk) {
-        // B of step ks+1 was requested one K-step ago
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        fix_tail_mine(ks + 1);
-      }
-      lds_barrier();  // half-period 2ks+1: this group moves data, the other computes
-      // B(ks+2) replaces A(ks), which group 1 finished reading before the barrier above
-      if (ks + 2 < nk)
-        move_data(ks + 1, ks + 2);
-      else if (ks + 1 < nk)
-        read_frags(ks + 1);
+    {
+      int lf = lane;
+      asm volatile("" : "+v"(lf));
+      fa.init(wm * 128, lf);
+      fb.init(wn * 128, lf);
     }
-  } else {
-    for (int ks = 0; ks < nk; ++ks) {
-      if (!kFreeHandoff) lds_barrier();
-      // A(ks+2) replaces B(ks-1), dead since the previous K-step
-      if (ks + 2 < nk)
-        move_data(ks, ks + 2);
-      else
-        read_frags(ks);
-      if (ks + 1 < nk) {
-        // A of step ks+1 (requested one K-step ago) must be in LDS before group 0 reads it
-        // after the next barrier; the 8 loads just issued may stay in flight (loads retire in
-        // order)
-        if (ks + 2 < nk)
-          __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
-        else
-          __builtin_amdgcn_s_waitcnt(0x0f70);
-        fix_tail_mine(ks + 1);
-      }
-      lds_barrier();
-      compute();
+#pragma unroll
+    for (int i = 0; i < WT; ++i)
+#pragma unroll
+      for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // K-step 0 complete in LDS (requested above, or before the previous item's epilogue); the
+    // 16 loads of K-step 1 may still be in flight (loads retire in order)
+    if (nk > 1) {
+      __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16); lgkmcnt and expcnt untouched
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      fix_tail(r0, r1);
     }
-  }
+    __syncthreads();
+    {
+      uint32_t aa[FragReader<A_T>::NBASE], ba[FragReader<B_T>::NBASE];
+      frag_addrs(r0, r1, 0, aa, ba);
+#pragma unroll
+      for (int g = 0; g < WT; ++g) {
+        X.a[g] = read_a(aa, g, 0);
+        X.b[g] = read_b(ba, g, 0);
+      }
+    }
 
+    // K loop.  In K-step t: first half-step computes on X (half 0) while Y is read from the
+    // tiles of t (half 1) and A(t+2) is requested into r4, dead since the barrier of K-step
+    // t-1; then every load but those eight must have landed (that is all of K-step t+1), one
+    // barrier publishes them and retires the tiles of t; the second half-step computes on Y
+    // while X is read from the tiles of t+1 and B(t+2) is requested where A(t) was.
+    int t = 0;
+    for (; t + 2 < nk; ++t) {
+      if (t + 3 == nk && k_tail != BK) set_offsets(k_tail);
+      half(X, Y, r0, r1, 1, Yes{}, a_base(t + 2), la, r4);
+      __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
+      __syncthreads();
+      half(Y, X, r2, r3, 0, Yes{}, b_base(t + 2), lb, r0);
+      rotate();
+    }
+    for (; t < nk; ++t) {
+      half(X, Y, r0, r1, 1, No{}, nullptr, la, 0u);
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      if (t + 2 == nk) fix_tail(r2, r3);
+      __syncthreads();
+      // (after the last K-step this reads tiles that do not exist: unused)
+      half(Y, X, r2, r3, 0, No{}, nullptr, lb, 0u);
+      rotate();
+    }
 
-  // Every LDS read of this item finished before the last barrier, so the ring is free: request
-  // the first two K-steps of the next item now and let them fly during the epilogue.
-  const int out_m0 = m0, out_n0 = n0;
-  float* const out_partial = split_k ? partial + p_off : nullptr;
-  const int next = item + (int)gridDim.x;
-  const bool more = next < total_items;
-  if (more) {
-    select_item(next);
-    issue_mine(0);
-    if (nk > 1) issue_mine(1);
-  }
+    // Every LDS read of this item that matters finished before the last barrier, so slots
+    // r0..r3 are free: request the first two K-steps of the next item now and let them fly
+    // during the epilogue.
+    const int out_m0 = m0, out_n0 = n0;
+    float* const out_partial = split_k ? partial + p_off : nullptr;
+    const int next = item + (int)gridDim.x;
+    const bool more = next < total_items;
+    if (more) {
+      select_item(next);
+      request_first_two();
+    }
+    // the compiler does not know the MFMAs' latency: let the last ones finish before their
+    // results are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
-  // Epilogue.  A lane holds C[m][n..n+3] for m = tile row (lane%32), n = 8g + 4*(lane/32):
-  // stored from there, every instruction would scatter 64 eight-byte pieces over 32 rows and
-  // the texture-address path, which takes such pieces one at a time, would need ~10 us per
-  // tile.  Instead each wave transposes through its own 4 KB of ring slot 4 (idle until K-step
-  // 2 of the next item is requested, after the next workgroup barrier): 32 rows of 128 bytes
-  // go in from the MFMA layout and come out as whole rows, 8 lanes per row, so an instruction
-  // writes 8 full 128-byte (bf16 output) or 8 contiguous row segments (fp32 partial tiles and
-  // accumulation into C, staged as fp32 so that the sum is rounded once).  Only lanes of the
-  // same wave exchange data: program order of its LDS instructions is all the ordering needed.
-  {
-    char* const stage = reinterpret_cast<char*>(smem + (NSLOTS - 1) * TILE) + wave * 4096;
-    int le = lane;  // opaque copy: nothing derived from it is kept alive through the K loop
-    asm volatile("" : "+v"(le));
-    const int r = le & 31, h = le >> 5;
-    const int wr = r * 128, wsw = (r >> 1) & 7;       // write side: row of the MFMA layout
-    const int rrow = le >> 3, rch = le & 7;           // read side: row 8q + rrow, 16-byte chunk rch
-    const int m_wave = out_m0 + wm * TM * 32, n_wave = out_n0 + wn * TN * 32;
-    auto wave_sync = [&]() {
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-    };
-    // Global addresses are a wave-uniform block base plus a 32-bit lane offset (row 8q + rrow
-    // of the block, this lane's chunk): four offset registers serve every access of the tile.
-    const bool rows_in = m_wave + TM * 32 <= M;  // wave-uniform: no row of the wave tile is cut off
-    if (out_partial == nullptr && !accumulate) {
-      uint32_t lo[4];
+    // Epilogue.  A lane holds C[m][n..n+3] for m = 16 mt + lane%16, n = 16 nt + 4 (lane/16):
+    // stored from there, every instruction would scatter 64 eight-byte pieces over 16 rows.
+    // Instead each wave transposes through its own 8 KB of slot r4 (idle until K-step 2 of the
+    // next item is requested, after the next workgroup barrier): a block of 16 rows goes in
+    // from the MFMA layout and comes out as whole rows, so a store instruction writes complete
+    // 256-byte (bf16) or 512-byte (fp32) row segments.  Only lanes of the same wave exchange
+    // data: program order of its LDS instructions is all the ordering needed.
+    {
+      const uint32_t stage = r4 + (uint32_t)wave * 8192u;
+      int le = lane;  // opaque copy: nothing derived from it is kept alive through the K loop
+      asm volatile("" : "+v"(le));
+      const int row16 = le & 15, quad = le >> 4;
+      const int m_wave = out_m0 + wm * 128, n_wave = out_n0 + wn * 128;
+      auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+      };
+      const bool rows_in = m_wave + 128 <= M;  // wave-uniform: no row of the wave tile is cut off
+      if (out_partial == nullptr && !accumulate) {
+        // bf16: 16 rows x 256 bytes per block, two buffers; chunk index XORed with the row
+        const int rch = le & 15;  // read side: row 4q + quad, 16-byte chunk rch
+        uint32_t lo[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * ldc + 8 * rch);
-      const bool cols_in = n_wave + 8 * rch < N;
+        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((4 * q + quad) * ldc + 8 * rch);
+        const bool cols_in = n_wave + 8 * rch < N;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
+        for (int mt = 0; mt < WT; ++mt) {
+          const uint32_t buf = stage + (uint32_t)(mt & 1) * 4096u;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
+          for (int nt = 0; nt < WT; ++nt) {
             bf16x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (bf16)acc[j][i][g * 4 + e];
-            *reinterpret_cast<bf16x4*>(stage + wr + (((4 * j + g) ^ wsw) << 4) + 8 * h) = o;
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)acc[mt][nt][e];
+            *(KR_LDS bf16x4*)(buf + row16 * 256 + (((2 * nt + (quad >> 1)) ^ row16) << 4) + (quad & 1) * 8) = o;
           }
-        wave_sync();
-        bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave);
+          wave_sync();
+          bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int rr = 8 * q + rrow;
-          const bf16x8 v =
-              *reinterpret_cast<const bf16x8*>(stage + rr * 128 + ((rch ^ ((rr >> 1) & 7)) << 4));
-          if (cols_in && (rows_in || m_wave + i * 32 + rr < M)) stg8(cb + lo[q], v);
-        }
-        wave_sync();
-      }
-    } else {
-      // fp32 staging, one 32 x 32 block per pass; `emit(i, j, q, v)` gets four consecutive
-      // columns of row 8q + rrow of block (i, j)
-      auto fp32_passes = [&](auto&& before_block_row, auto&& emit) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          before_block_row(i);
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              f32x4 pv;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) pv[e] = acc[j][i][g * 4 + e];
-              *reinterpret_cast<f32x4*>(stage + wr + (((2 * g + h) ^ wsw) << 4)) = pv;
-            }
-            wave_sync();
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int rr = 8 * q + rrow;
-              const f32x4 v = *reinterpret_cast<const f32x4*>(stage + rr * 128 +
-                                                              ((rch ^ ((rr >> 1) & 7)) << 4));
-              emit(i, j, q, v);
-            }
-            wave_sync();
+          for (int q = 0; q < 4; ++q) {
+            const int rr = 4 * q + quad;
+            const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
+            if (cols_in && (rows_in || m_wave + mt * 16 + rr < M)) stg8(cb + lo[q], v);
           }
         }
-      };
-      if (out_partial != nullptr) {
-        uint32_t lo[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * N + 4 * rch);
-        fp32_passes([](int) {},
-                    [&](int i, int j, int q, const f32x4& v) {
-                      float* const pb = out_partial + ((int64_t)(m_wave + i * 32) * N + n_wave + j * 32);
-                      if (n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M))
-                        *reinterpret_cast<f32x4*>(pb + lo[q]) = v;
-                    });
       } else {
-        // accumulation into C: the old values of a 32-row block (the same row segments the
-        // results go to) are requested one block ahead of the passes that use them, so their
-        // memory latency is paid once per tile, not once per pass.  Positions beyond the matrix
-        // read a valid neighbour instead and are never stored back.
-        uint32_t lo[4];
+        // fp32: 16 rows x 512 bytes per block, one buffer.  Read side: row 2q + half, 16-byte
+        // chunk ch = four consecutive columns.
+        const int hrow = le >> 5, ch = le & 31;
+        const bool cols_in = n_wave + 4 * ch < N;
+        const int ldo = out_partial != nullptr ? N : ldc;
+        uint32_t lo[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((8 * q + rrow) * ldc + 4 * rch);
-        bf16x4 oldc[2][TN][4];
-        auto fetch_old = [&](int i) {
+        for (int q = 0; q < 8; ++q) lo[q] = (uint32_t)((2 * q + hrow) * ldo + 4 * ch);
+        // accumulation into C: the old values of a 16-row block are requested one block ahead
+        // of the pass that uses them.  Positions beyond the matrix read a valid neighbour
+        // instead and are never stored back.
+        bf16x4 oldc[2][8];
+        auto fetch_old = [&](int mt) {
+          const bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
 #pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            const bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave + j * 32);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const bool in = n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M);
-              oldc[i & 1][j][q] = *reinterpret_cast<const bf16x4*>(in ? cb + lo[q] : C);
-            }
+          for (int q = 0; q < 8; ++q) {
+            const bool in = cols_in && (rows_in || m_wave + mt * 16 + 2 * q + hrow < M);
+            oldc[mt & 1][q] = *reinterpret_cast<const bf16x4*>(in ? cb + lo[q] : C);
           }
         };
-        fetch_old(0);
-        fp32_passes([&](int i) { if (i + 1 < TM) fetch_old(i + 1); },
-                    [&](int i, int j, int q, const f32x4& v) {
-                      bf16* const cb = C + ((int64_t)(m_wave + i * 32) * ldc + n_wave + j * 32);
-                      if (n_wave + j * 32 + 4 * rch < N && (rows_in || m_wave + i * 32 + 8 * q + rrow < M)) {
-                        bf16x4 o;
+        if (out_partial == nullptr) fetch_old(0);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[i & 1][j][q][e]);
-                        *reinterpret_cast<bf16x4*>(cb + lo[q]) = o;
-                      }
-                    });
+        for (int mt = 0; mt < WT; ++mt) {
+          if (out_partial == nullptr && mt + 1 < WT) fetch_old(mt + 1);
+#pragma unroll
+          for (int nt = 0; nt < WT; ++nt)
+            *(KR_LDS f32x4*)(stage + row16 * 512 + (((4 * nt + quad) ^ row16) << 4)) = acc[mt][nt];
+          wave_sync();
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int rr = 2 * q + hrow;
+            const f32x4 v = *(KR_LDS const f32x4*)(stage + rr * 512 + ((ch ^ rr) << 4));
+            const bool in = cols_in && (rows_in || m_wave + mt * 16 + rr < M);
+            if (out_partial != nullptr) {
+              float* const pb = out_partial + ((int64_t)(m_wave + mt * 16) * N + n_wave);
+              if (in) *reinterpret_cast<f32x4*>(pb + lo[q]) = v;
+            } else {
+              bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
+              if (in) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
+                *reinterpret_cast<bf16x4*>(cb + lo[q]) = o;
+              }
+            }
+          }
+          wave_sync();
+        }
       }
     }
-  }
-  if (!more) break;
-  item = next;
+    if (!more) break;
+    item = next;
   }
 }
 
