@@ -436,17 +436,21 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // Epilogue.  A lane holds C[m][n..n+3] for m = 16 mt + lane%16, n = 16 nt + 4 (lane/16):
-    // stored from there, every instruction would scatter 64 eight-byte pieces over 16 rows.
-    // Instead each wave transposes through its own 8 KB of slot r4 (idle until K-step 2 of the
-    // next item is requested, after the next workgroup barrier): a block of 16 rows goes in
-    // from the MFMA layout and comes out as whole rows, so a store instruction writes complete
-    // 256-byte (bf16) or 512-byte (fp32) row segments.  Only lanes of the same wave exchange
-    // data: program order of its LDS instructions is all the ordering needed.
+    // stored from there, every instruction would scatter 64 small pieces over 16 rows.  Instead
+    // each wave transposes through its own 8 KB of slot r4 (idle until K-step 2 of the next
+    // item is requested, after the next workgroup barrier): a block of 16 rows x 128 columns
+    // goes in as fp32 from the MFMA layout and comes out as whole rows (32 lanes per row, four
+    // consecutive columns per lane), so a store instruction writes complete row segments of
+    // 256 bytes (bf16 output) or 512 bytes (fp32 partial tiles); accumulation into C adds the
+    // old values in fp32, so the sum is rounded once.  Only lanes of the same wave exchange
+    // data: program order of its LDS instructions is all the ordering needed.  The accumulators
+    // are read in one place for all three kinds of output.
     {
       const uint32_t stage = r4 + (uint32_t)wave * 8192u;
       int le = lane;  // opaque copy: nothing derived from it is kept alive through the K loop
       asm volatile("" : "+v"(le));
       const int row16 = le & 15, quad = le >> 4;
+      const int hrow = le >> 5, ch = le & 31;  // read side: row 2q + hrow, columns 4 ch .. + 3
       const int m_wave = out_m0 + wm * 128, n_wave = out_n0 + wn * 128;
       auto wave_sync = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
@@ -454,81 +458,54 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
       };
       const bool rows_in = m_wave + 128 <= M;  // wave-uniform: no row of the wave tile is cut off
-      if (out_partial == nullptr && !accumulate) {
-        // bf16: 16 rows x 256 bytes per block, two buffers; chunk index XORed with the row
-        const int rch = le & 15;  // read side: row 4q + quad, 16-byte chunk rch
-        uint32_t lo[4];
+      const bool cols_in = n_wave + 4 * ch < N;
+      const bool to_partial = out_partial != nullptr;
+      const bool add_old = !to_partial && accumulate;
+      const int ldo = to_partial ? N : ldc;
+      uint32_t lo[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) lo[q] = (uint32_t)((4 * q + quad) * ldc + 8 * rch);
-        const bool cols_in = n_wave + 8 * rch < N;
+      for (int q = 0; q < 8; ++q) lo[q] = (uint32_t)((2 * q + hrow) * ldo + 4 * ch);
+      // accumulation into C: the old values of a 16-row block are requested one block ahead of
+      // the pass that uses them (zeros otherwise).  Positions beyond the matrix read a valid
+      // neighbour instead and are never stored back.
+      bf16x4 oldc[2][8];
 #pragma unroll
-        for (int mt = 0; mt < WT; ++mt) {
-          const uint32_t buf = stage + (uint32_t)(mt & 1) * 4096u;
+      for (int q = 0; q < 8; ++q)
 #pragma unroll
-          for (int nt = 0; nt < WT; ++nt) {
+        for (int e = 0; e < 4; ++e) oldc[0][q][e] = oldc[1][q][e] = (bf16)0.f;
+      auto fetch_old = [&](int mt) {
+        const bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const bool in = cols_in && (rows_in || m_wave + mt * 16 + 2 * q + hrow < M);
+          oldc[mt & 1][q] = *reinterpret_cast<const bf16x4*>(in ? cb + lo[q] : C);
+        }
+      };
+      if (add_old) fetch_old(0);
+#pragma unroll
+      for (int mt = 0; mt < WT; ++mt) {
+        if (add_old && mt + 1 < WT) fetch_old(mt + 1);
+#pragma unroll
+        for (int nt = 0; nt < WT; ++nt)
+          *(KR_LDS f32x4*)(stage + row16 * 512 + (((4 * nt + quad) ^ row16) << 4)) = acc[mt][nt];
+        wave_sync();
+        const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + n_wave;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int rr = 2 * q + hrow;
+          const f32x4 v = *(KR_LDS const f32x4*)(stage + rr * 512 + ((ch ^ rr) << 4));
+          const bool in = cols_in && (rows_in || m_wave + mt * 16 + rr < M);
+          if (to_partial) {
+            if (in) *reinterpret_cast<f32x4*>(out_partial + blk + lo[q]) = v;
+          } else {
             bf16x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (bf16)acc[mt][nt][e];
-            *(KR_LDS bf16x4*)(buf + row16 * 256 + (((2 * nt + (quad >> 1)) ^ row16) << 4) + (quad & 1) * 8) = o;
-          }
-          wave_sync();
-          bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int rr = 4 * q + quad;
-            const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
-            if (cols_in && (rows_in || m_wave + mt * 16 + rr < M)) stg8(cb + lo[q], v);
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
+            if (in) *reinterpret_cast<bf16x4*>(C + blk + lo[q]) = o;
           }
         }
-      } else {
-        // fp32: 16 rows x 512 bytes per block, one buffer.  Read side: row 2q + half, 16-byte
-        // chunk ch = four consecutive columns.
-        const int hrow = le >> 5, ch = le & 31;
-        const bool cols_in = n_wave + 4 * ch < N;
-        const int ldo = out_partial != nullptr ? N : ldc;
-        uint32_t lo[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) lo[q] = (uint32_t)((2 * q + hrow) * ldo + 4 * ch);
-        // accumulation into C: the old values of a 16-row block are requested one block ahead
-        // of the pass that uses them.  Positions beyond the matrix read a valid neighbour
-        // instead and are never stored back.
-        bf16x4 oldc[2][8];
-        auto fetch_old = [&](int mt) {
-          const bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
-#pragma unroll
-          for (int q = 0; q < 8; ++q) {
-            const bool in = cols_in && (rows_in || m_wave + mt * 16 + 2 * q + hrow < M);
-            oldc[mt & 1][q] = *reinterpret_cast<const bf16x4*>(in ? cb + lo[q] : C);
-          }
-        };
-        if (out_partial == nullptr) fetch_old(0);
-#pragma unroll
-        for (int mt = 0; mt < WT; ++mt) {
-          if (out_partial == nullptr && mt + 1 < WT) fetch_old(mt + 1);
-#pragma unroll
-          for (int nt = 0; nt < WT; ++nt)
-            *(KR_LDS f32x4*)(stage + row16 * 512 + (((4 * nt + quad) ^ row16) << 4)) = acc[mt][nt];
-          wave_sync();
-#pragma unroll
-          for (int q = 0; q < 8; ++q) {
-            const int rr = 2 * q + hrow;
-            const f32x4 v = *(KR_LDS const f32x4*)(stage + rr * 512 + ((ch ^ rr) << 4));
-            const bool in = cols_in && (rows_in || m_wave + mt * 16 + rr < M);
-            if (out_partial != nullptr) {
-              float* const pb = out_partial + ((int64_t)(m_wave + mt * 16) * N + n_wave);
-              if (in) *reinterpret_cast<f32x4*>(pb + lo[q]) = v;
-            } else {
-              bf16* const cb = C + ((int64_t)(m_wave + mt * 16) * ldc + n_wave);
-              if (in) {
-                bf16x4 o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
-                *reinterpret_cast<bf16x4*>(cb + lo[q]) = o;
-              }
-            }
-          }
-          wave_sync();
-        }
+        wave_sync();
+        __builtin_amdgcn_sched_barrier(0);  // keep the accumulator reads of later blocks below
       }
     }
     if (!more) break;
