@@ -1,44 +1,43 @@
 // bf16 GEMM on the gfx950 matrix cores: C[M,N] = A . B with fp32 accumulation, bf16 store.
 //
-// Roofline: MFMA (v_mfma_f32_32x32x16_bf16, 32768 FLOP per wave instruction).  Algorithmic
+// Roofline: MFMA (v_mfma_f32_16x16x32_bf16, 16384 FLOP per wave instruction).  Algorithmic
 // work per launch is 2*M*N*K FLOP.
 //
-// Structure ("8-wave ping-pong")
-//   * A workgroup of 8 waves owns a 256 x 256 tile of C and walks K in steps of 64.  Each wave
-//     owns 128 x 64 of the tile as 4 x 2 MFMA tiles of 32x32 held in registers for the whole
-//     K loop.
-//   * The waves form two groups of four, one wave of each group per SIMD.  Time is cut into
-//     half-periods by workgroup barriers.  In every half-period one group only issues MFMAs
-//     (all 32 of a K-step, operands already in registers) while the other group only moves
-//     data: it issues the global loads of one operand tile of K-step k+2 and reads its operand
-//     fragments of the next K-step out of LDS.  Then the roles swap.  The matrix pipe of every
-//     SIMD always has exactly one wave feeding it, and no wave ever waits on memory in the
-//     middle of its MFMA burst.
+// Structure ("one instruction stream per SIMD")
+//   * A workgroup of 4 waves, one per SIMD, owns a 256 x 256 tile of C and walks K in steps of
+//     64.  Each wave owns 128 x 128 of the tile as 8 x 8 MFMA tiles of 16x16: 256 accumulator
+//     registers, which are the wave's accumulation registers (the MFMAs are written as inline
+//     assembly to pin them there); its 256 ordinary registers hold two sets of operand
+//     fragments and the addressing.
+//   * The K loop is a fixed, hand-ordered sequence.  A half-step is the 64 MFMAs of one
+//     32-element half of a K-step; woven between them, one behind each MFMA, are the 16
+//     fragment reads of the next half-step and the 8 global loads of one operand tile two
+//     K-steps ahead.  An MFMA holds the matrix pipe for 16 cycles and the wave can issue
+//     another instruction every 4-5, so these ride along without opening a gap in the pipe.
+//     One workgroup barrier per K-step publishes the next tiles and retires the current ones.
 //   * Global memory goes straight into LDS (global_load_lds_dwordx4): no staging registers, no
 //     LDS store instructions.  The hardware places the 64 lanes of such a load contiguously in
 //     LDS, so bank conflicts are avoided by an XOR swizzle applied on the *global* side — each
 //     lane fetches the 16-byte chunk that belongs at its LDS slot.
 //   * All 160 KB of LDS form a ring of five 32 KB slots, one operand tile (A or B of one
-//     K-step) per slot: two slots are being consumed, three are being filled.  Group 1 requests
-//     the A tiles (a flight window of three half-periods), group 0 the B tiles (two
-//     half-periods), so the texture-address path sees an even 32 KB per half-period — half of
-//     what it can carry — and every load has at least a full half-period to land after the
-//     last request of its tile went out.  With only two 64 KB stages the loads of a whole
-//     K-step had to be pushed out back to back and their tail had no time left.
+//     K-step) per slot.  In K-step t the first half-step requests A(t+2) into the slot B(t-1)
+//     left at the previous barrier, the second half-step B(t+2) into the slot A(t) leaves at
+//     this one: an even 32 KB per half-step, and every tile has one to two K-steps to land.
 //   * Loads are 16-byte vectors along whichever dimension is contiguous in memory.  An operand
 //     whose contraction dimension is contiguous ("K-major") is fetched from LDS with
 //     ds_read_b128; an operand whose contraction dimension is the row index ("transposed": the
 //     weight in dgrad, both operands in wgrad) with the transposing LDS read
 //     ds_read_b64_tr_b16.  No transposed copy of any operand is ever made.
 //   * The MFMA is issued with the operands swapped (the B tile feeds the instruction's A
-//     port), so a lane ends up with four consecutive N-columns of one C row and the epilogue
-//     stores 8-byte bf16 quads contiguous along the row.
+//     port), so a lane ends up with four consecutive N-columns of one C row; the epilogue
+//     transposes 16-row blocks through LDS and stores whole rows.
 //   * Rows beyond the matrix edge are clamped to the last valid row instead of predicated: an
 //     output element depends only on its own A row and B row, and out-of-range outputs are
 //     never stored.  A contraction tail (K not a multiple of 64) is zeroed in LDS after its
 //     tile has landed.
-//   * Workgroup ids are remapped so that the tiles resident on one XCD (ids congruent mod 8)
-//     form a compact band of C and share A/B panels in that XCD's L2.
+//   * Workgroups are persistent (one per compute unit); ids are remapped so that the tiles
+//     resident on one XCD (ids congruent mod 8) form a compact band of C and share A/B panels
+//     in that XCD's L2.
 //   * Split-K: when C has too few tiles to fill 256 CUs (weight gradients: a small N x K
 //     output contracted over all tokens), the contraction is cut into up to 16 ranges, each
 //     workgroup writes an fp32 partial tile into a caller-provided workspace, and a small
