@@ -618,8 +618,19 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
       n = 256;
     return n;
   }();
+  // Items are spread evenly: with r = ceil(items / CUs) rounds, ceil(items / r) workgroups (rounded
+  // up to a multiple of 8, which keeps item ids and XCDs aligned) finish at the same time as one
+  // workgroup per CU would, and the CUs left over are free for other streams' kernels from the
+  // start of the launch instead of from the end of its first round.
+  auto grid_for = [&](int items) {
+    if (items <= num_cus) return items;
+    const int rounds = (items + num_cus - 1) / num_cus;
+    int g = (items + rounds - 1) / rounds;
+    g = (g + 7) / 8 * 8;
+    return g < num_cus ? g : num_cus;
+  };
   if (splits == 1) {
-    const int grid = tiles < num_cus ? tiles : num_cus;
+    const int grid = grid_for(tiles);
     hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
                        (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr);
     return kr_launch_status();
@@ -628,7 +639,7 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   k_per = (k_per + BK - 1) / BK * BK;
   splits = (K + k_per - 1) / k_per;
   const int items = tiles * splits;
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(items < num_cus ? items : num_cus), dim3(NTHREADS),
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(grid_for(items)), dim3(NTHREADS),
                      lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
