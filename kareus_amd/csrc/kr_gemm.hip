@@ -47,8 +47,8 @@
 namespace {
 
 constexpr int BK = 64;
-constexpr int BM = 256, BN = 256;
-constexpr int WT = 8;  // 16x16 MFMA tiles per wave along each dimension: a wave owns 128 x 128 of C
+constexpr int BM = 256, BN = 256;  // BN: the widest tile; a kernel instance covers 32 * WN columns
+constexpr int WT = 8;  // 16x16 MFMA tiles per wave along M: a wave owns 128 rows x 16 * WN columns of C
 constexpr int NTHREADS = 256;
 constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
 constexpr uint32_t SLOT_BYTES = TILE * sizeof(bf16);
@@ -181,13 +181,17 @@ __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, i
   tn = in_band / band_rows;
 }
 
+template <int WN>
 struct Frags {
-  bf16x8 a[WT], b[WT];
+  bf16x8 a[WT], b[WN];
 };
-struct Yes { static constexpr bool value = true; };
-struct No { static constexpr bool value = false; };
+template <int N>
+struct Count { static constexpr int value = N; };
 
-template <bool A_T, bool B_T>
+// WN: 16-column MFMA tiles per wave along N (5..8): the workgroup's tile is 256 x 32 * WN.  Narrower
+// tiles let the host avoid a mostly empty last round of workgroups or a mostly padded last tile
+// column; the B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
+template <bool A_T, bool B_T, int WN>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
                                                         bf16* __restrict__ C, int ldc, int M,
@@ -196,8 +200,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;  // wave tile: rows wm*128.., columns wn*128..
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  constexpr int BN_ = 32 * WN;
+  const int wm = wave >> 1, wn = wave & 1;  // wave tile: rows wm*128.., columns wn*16*WN..
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_ - 1) / BN_;
   const int ntiles = tiles_m * tiles_n;
   const bool split_k = partial != nullptr;
   const uint32_t smem_b = lds_addr(smem);
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     int tile_m, tile_n;
     remap_block(v - split * ntiles, ntiles, tiles_m, tiles_n, tile_m, tile_n);
     m0 = tile_m * BM;
-    n0 = tile_n * BN;
+    n0 = tile_n * BN_;
     if (split_k) {
       // split-K: contraction range [split*k_per, split*k_per + kc), fp32 partial tile out
       // (k_per is a multiple of 64)
@@ -240,8 +245,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 
   // accumulators live in the accumulation registers (the MFMAs are written as inline assembly
   // with that register class, see mfma() below); fragments in ordinary vector registers
-  f32x4 acc[WT][WT];
-  Frags X, Y;
+  f32x4 acc[WT][WN];
+  Frags<WN> X, Y;
   uint32_t la[8], lb[8];  // byte offsets of this lane's chunk in the 8 loads of an A / a B tile
 
   auto set_offsets = [&](int k_left) {
@@ -253,26 +258,28 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left);
     }
   };
-  auto request = [&](const bf16* base, const uint32_t (&off)[8], uint32_t slot) {
+  // the first `count` loads of a tile (8 for A, WN for B)
+  auto request = [&](const bf16* base, const uint32_t (&off)[8], uint32_t slot, auto count_tag) {
+    constexpr int COUNT = decltype(count_tag)::value;
     const uint32_t dst = slot + wave_blk;
     dma_b128<0 * 4096>(base, off[0], dst);
     dma_b128<1 * 4096>(base, off[1], dst);
     dma_b128<2 * 4096>(base, off[2], dst);
     dma_b128<3 * 4096>(base, off[3], dst);
     dma_b128<4 * 4096>(base, off[4], dst);
-    dma_b128<5 * 4096>(base, off[5], dst);
-    dma_b128<6 * 4096>(base, off[6], dst);
-    dma_b128<7 * 4096>(base, off[7], dst);
+    if constexpr (COUNT > 5) dma_b128<5 * 4096>(base, off[5], dst);
+    if constexpr (COUNT > 6) dma_b128<6 * 4096>(base, off[6], dst);
+    if constexpr (COUNT > 7) dma_b128<7 * 4096>(base, off[7], dst);
   };
   // K-steps 0 and 1 of the current item into r0..r3
   auto request_first_two = [&]() {
     set_offsets(nk == 1 ? k_tail : BK);
-    request(a_base(0), la, r0);
-    request(b_base(0), lb, r1);
+    request(a_base(0), la, r0, Count<8>{});
+    request(b_base(0), lb, r1, Count<WN>{});
     if (nk > 1) {
       if (nk == 2 && k_tail != BK) set_offsets(k_tail);
-      request(a_base(1), la, r2);
-      request(b_base(1), lb, r3);
+      request(a_base(1), la, r2, Count<8>{});
+      request(b_base(1), lb, r3, Count<WN>{});
     }
   };
   // After this wave's loads of the last K-step have landed (A in slot sa, B in slot sb): zero
@@ -311,7 +318,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       asm volatile("" : "+v"(ba[0]));
     } else {
 #pragma unroll
-      for (int g = 0; g < WT; ++g) {
+      for (int g = 0; g < WN; ++g) {
         ba[g] = sb + fb.base[g];
         asm volatile("" : "+v"(ba[g]));
       }
@@ -329,22 +336,23 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // if DMA, the 8 requests of one operand tile woven in between in exactly this order.  The
   // operands are swapped (the B fragment feeds the instruction's A port), so a lane ends up
   // with four consecutive columns of one row of C.
-  auto half = [&](Frags& cur, Frags& nxt, uint32_t sa, uint32_t sb, int h, auto dma_tag,
+  auto half = [&](Frags<WN>& cur, Frags<WN>& nxt, uint32_t sa, uint32_t sb, int h, auto dma_tag,
                   const bf16* dbase, const uint32_t (&doff)[8], uint32_t dslot) {
+    constexpr int DMA = decltype(dma_tag)::value;  // how many loads to weave in (0: none)
     uint32_t aa[FragReader<A_T>::NBASE], ba[FragReader<B_T>::NBASE];
     frag_addrs(sa, sb, h, aa, ba);
     const uint32_t dst = dslot + wave_blk;
 #pragma unroll
     for (int g = 0; g < WT; ++g) {
 #pragma unroll
-      for (int nt = 0; nt < WT; ++nt) {
+      for (int nt = 0; nt < WN; ++nt) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+a"(acc[g][nt])
                      : "v"(cur.b[nt]), "v"(cur.a[g]));
         if (nt == 0) nxt.a[g] = read_a(aa, g, h);
-        if (nt == 2) nxt.b[g] = read_b(ba, g, h);
-        if constexpr (decltype(dma_tag)::value) {
-          if (nt == 4) {
+        if (nt == 2 && g < WN) nxt.b[g] = read_b(ba, g, h);
+        if constexpr (DMA > 0) {
+          if (nt == 4 && g < DMA) {
             if (g == 0) dma_b128<0 * 4096>(dbase, doff[0], dst);
             if (g == 1) dma_b128<1 * 4096>(dbase, doff[1], dst);
             if (g == 2) dma_b128<2 * 4096>(dbase, doff[2], dst);
@@ -370,16 +378,17 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       int lf = lane;
       asm volatile("" : "+v"(lf));
       fa.init(wm * 128, lf);
-      fb.init(wn * 128, lf);
+      fb.init(wn * 16 * WN, lf);
     }
 #pragma unroll
     for (int i = 0; i < WT; ++i)
 #pragma unroll
-      for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < WN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     // K-step 0 complete in LDS (requested above, or before the previous item's epilogue); the
     // 16 loads of K-step 1 may still be in flight (loads retire in order)
     if (nk > 1) {
-      __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16); lgkmcnt and expcnt untouched
+      // vmcnt(8 + WN); lgkmcnt and expcnt untouched
+      __builtin_amdgcn_s_waitcnt(0x0f70 | ((8 + WN) & 15) | (((8 + WN) >> 4) << 14));
     } else {
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       fix_tail(r0, r1);
@@ -391,7 +400,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
       for (int g = 0; g < WT; ++g) {
         X.a[g] = read_a(aa, g, 0);
-        X.b[g] = read_b(ba, g, 0);
+        if (g < WN) X.b[g] = read_b(ba, g, 0);
       }
     }
 
@@ -403,19 +412,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     int t = 0;
     for (; t + 2 < nk; ++t) {
       if (t + 3 == nk && k_tail != BK) set_offsets(k_tail);
-      half(X, Y, r0, r1, 1, Yes{}, a_base(t + 2), la, r4);
+      half(X, Y, r0, r1, 1, Count<8>{}, a_base(t + 2), la, r4);
       __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
       __syncthreads();
-      half(Y, X, r2, r3, 0, Yes{}, b_base(t + 2), lb, r0);
+      half(Y, X, r2, r3, 0, Count<WN>{}, b_base(t + 2), lb, r0);
       rotate();
     }
     for (; t < nk; ++t) {
-      half(X, Y, r0, r1, 1, No{}, nullptr, la, 0u);
+      half(X, Y, r0, r1, 1, Count<0>{}, nullptr, la, 0u);
       __builtin_amdgcn_s_waitcnt(0x0f70);
       if (t + 2 == nk) fix_tail(r2, r3);
       __syncthreads();
       // (after the last K-step this reads tiles that do not exist: unused)
-      half(Y, X, r2, r3, 0, No{}, nullptr, lb, 0u);
+      half(Y, X, r2, r3, 0, Count<0>{}, nullptr, lb, 0u);
       rotate();
     }
 
@@ -450,14 +459,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       asm volatile("" : "+v"(le));
       const int row16 = le & 15, quad = le >> 4;
       const int hrow = le >> 5, ch = le & 31;  // read side: row 2q + hrow, columns 4 ch .. + 3
-      const int m_wave = out_m0 + wm * 128, n_wave = out_n0 + wn * 128;
+      const int m_wave = out_m0 + wm * 128, n_wave = out_n0 + wn * 16 * WN;
       auto wave_sync = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
       };
       const bool rows_in = m_wave + 128 <= M;  // wave-uniform: no row of the wave tile is cut off
-      const bool cols_in = n_wave + 4 * ch < N;
+      const bool cols_in = 4 * ch < 16 * WN && n_wave + 4 * ch < N;
       const bool to_partial = out_partial != nullptr;
       const bool add_old = !to_partial && accumulate;
       const int ldo = to_partial ? N : ldc;
@@ -481,29 +490,62 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         }
       };
       if (add_old) fetch_old(0);
+      // bf16 output without accumulation goes through the same place as bf16: 16 rows x 256 bytes
+      // per block, two buffers (so one wave-level fence per block), read side row 4q + quad,
+      // 16-byte chunk rch = eight consecutive columns, 16 lanes per row
+      const bool narrow = !to_partial && !add_old;
+      const int rch = le & 15;
+      const bool ncols_in = 8 * rch < 16 * WN && n_wave + 8 * rch < N;
+      uint32_t nlo[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) nlo[q] = (uint32_t)((4 * q + quad) * ldc + 8 * rch);
 #pragma unroll
       for (int mt = 0; mt < WT; ++mt) {
         if (add_old && mt + 1 < WT) fetch_old(mt + 1);
+        f32x4 vals[WN];  // the only place the accumulators are read
 #pragma unroll
-        for (int nt = 0; nt < WT; ++nt)
-          *(KR_LDS f32x4*)(stage + row16 * 512 + (((4 * nt + quad) ^ row16) << 4)) = acc[mt][nt];
-        wave_sync();
+        for (int nt = 0; nt < WN; ++nt) {
+          vals[nt] = acc[mt][nt];
+          asm volatile("" : "+v"(vals[nt]));  // read here, not once in each branch below
+        }
         const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + n_wave;
+        if (narrow) {
+          const uint32_t buf = stage + (uint32_t)(mt & 1) * 4096u;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const int rr = 2 * q + hrow;
-          const f32x4 v = *(KR_LDS const f32x4*)(stage + rr * 512 + ((ch ^ rr) << 4));
-          const bool in = cols_in && (rows_in || m_wave + mt * 16 + rr < M);
-          if (to_partial) {
-            if (in) *reinterpret_cast<f32x4*>(out_partial + blk + lo[q]) = v;
-          } else {
+          for (int nt = 0; nt < WN; ++nt) {
             bf16x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
-            if (in) *reinterpret_cast<bf16x4*>(C + blk + lo[q]) = o;
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)vals[nt][e];
+            *(KR_LDS bf16x4*)(buf + row16 * 256 + (((2 * nt + (quad >> 1)) ^ row16) << 4) + (quad & 1) * 8) = o;
           }
+          wave_sync();
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int rr = 4 * q + quad;
+            const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
+            if (ncols_in && (rows_in || m_wave + mt * 16 + rr < M)) stg8(C + blk + nlo[q], v);
+          }
+        } else {
+#pragma unroll
+          for (int nt = 0; nt < WN; ++nt)
+            *(KR_LDS f32x4*)(stage + row16 * 512 + (((4 * nt + quad) ^ row16) << 4)) = vals[nt];
+          wave_sync();
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int rr = 2 * q + hrow;
+            const f32x4 v = *(KR_LDS const f32x4*)(stage + rr * 512 + ((ch ^ rr) << 4));
+            const bool in = cols_in && (rows_in || m_wave + mt * 16 + rr < M);
+            if (to_partial) {
+              if (in) *reinterpret_cast<f32x4*>(out_partial + blk + lo[q]) = v;
+            } else {
+              bf16x4 o;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
+              if (in) *reinterpret_cast<bf16x4*>(C + blk + lo[q]) = o;
+            }
+          }
+          wave_sync();
         }
-        wave_sync();
         __builtin_amdgcn_sched_barrier(0);  // keep the accumulator reads of later blocks below
       }
     }
@@ -511,14 +553,6 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     item = next;
   }
 }
-
-// the three layouts the library serves
-template __global__ void gemm_kernel<false, false>(const bf16*, int, const bf16*, int, bf16*,
-                                                   int, int, int, int, int, int, int, float*);
-template __global__ void gemm_kernel<false, true>(const bf16*, int, const bf16*, int, bf16*,
-                                                  int, int, int, int, int, int, int, float*);
-template __global__ void gemm_kernel<true, true>(const bf16*, int, const bf16*, int, bf16*,
-                                                 int, int, int, int, int, int, int, float*);
 
 // C = bf16(sum over splits of the fp32 partial tiles [+ C]); one thread per 8 columns.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
@@ -589,20 +623,41 @@ inline int choose_splits(int M, int N, int K, float latency_weight) {
   return best;
 }
 
-template <bool A_T, bool B_T>
+// Tile width for an output that is not split along K: 32 * WN columns, WN in 5..8.  The estimate is
+// the launch's own latency — rounds of tiles over the CUs times the cost of a tile (WN units of
+// MFMA work plus about one unit of prologue and epilogue); ties go to the wider tile, which reads
+// less from LDS per FLOP.  Outputs with fewer than 192 full-width tiles keep the full width (they
+// are candidates for split-K, whose cost model assumes it).
+inline int choose_wn(int M, int N, int num_cus) {
+  const int tiles_m = (M + BM - 1) / BM;
+  if (tiles_m * ((N + BN - 1) / BN) < 192) return 8;
+  int best = 8;
+  long best_cost = 0;
+  for (int wn = 8; wn >= 5; --wn) {
+    const int tiles = tiles_m * ((N + 32 * wn - 1) / (32 * wn));
+    const long cost = (long)((tiles + num_cus - 1) / num_cus) * (wn + 1);
+    if (wn == 8 || cost < best_cost) {
+      best = wn;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+template <bool A_T, bool B_T, int WN>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
-           hipStream_t stream) {
+           hipStream_t stream, int num_cus) {
   constexpr size_t lds_bytes = NSLOTS * TILE * sizeof(bf16);
   // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
   static const hipError_t attr_status =
-      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T>,
+      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
-  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int tiles = ((M + BM - 1) / BM) * ((N + 32 * WN - 1) / (32 * WN));
   // the latency-optimal count, capped by what the caller's workspace holds (a caller that wants
   // fewer splits says so by passing the smaller workspace kr_gemm_workspace_bytes_shared sizes)
-  int splits = choose_splits(M, N, K, 1.f);
+  int splits = WN == 8 ? choose_splits(M, N, K, 1.f) : 1;
   const size_t one = (size_t)M * N * sizeof(float);
   if (workspace == nullptr) {
     splits = 1;
@@ -610,14 +665,7 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
     splits = (int)(workspace_bytes / one);
   }
   if (splits < 2 || (int64_t)splits * M * N >= ((int64_t)1 << 31)) splits = 1;
-  // one persistent workgroup per compute unit (a workgroup owns a whole CU's LDS)
-  static const int num_cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    return n;
-  }();
+  // at most one persistent workgroup per compute unit (a workgroup owns a whole CU's LDS)
   // Items are spread evenly: with r = ceil(items / CUs) rounds, ceil(items / r) workgroups (rounded
   // up to a multiple of 8, which keeps item ids and XCDs aligned) finish at the same time as one
   // workgroup per CU would, and the CUs left over are free for other streams' kernels from the
@@ -631,7 +679,7 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   };
   if (splits == 1) {
     const int grid = grid_for(tiles);
-    hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
+    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
                        (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr);
     return kr_launch_status();
   }
@@ -639,7 +687,7 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   k_per = (k_per + BK - 1) / BK * BK;
   splits = (K + k_per - 1) / k_per;
   const int items = tiles * splits;
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T>), dim3(grid_for(items)), dim3(NTHREADS),
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN>), dim3(grid_for(items)), dim3(NTHREADS),
                      lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
@@ -684,17 +732,33 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   bf16* c = (bf16*)C;
   float* ws = (float*)workspace;
   hipStream_t st = (hipStream_t)stream;
+  static const int num_cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  const int wn = choose_wn(M, N, num_cus);
+#define KR_GEMM_LAUNCH(AT, BT)                                                                           \
+  switch (wn) {                                                                                          \
+    case 5: return launch<AT, BT, 5>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
+    case 6: return launch<AT, BT, 6>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
+    case 7: return launch<AT, BT, 7>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
+    default: return launch<AT, BT, 8>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
+  }
   switch (layout) {
     case KR_GEMM_TN:  // A [M,K], B [N,K]
       if (lda < K || ldb < K || ldc < N) return KR_EINVAL;
-      return launch<false, false>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
+      KR_GEMM_LAUNCH(false, false)
     case KR_GEMM_NN:  // A [M,K], B [K,N]
       if (lda < K || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<false, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
+      KR_GEMM_LAUNCH(false, true)
     case KR_GEMM_NT:  // A [K,M], B [K,N]
       if (lda < M || ldb < N || ldc < N) return KR_EINVAL;
-      return launch<true, true>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st);
+      KR_GEMM_LAUNCH(true, true)
     default:
       return KR_EINVAL;
   }
+#undef KR_GEMM_LAUNCH
 }
