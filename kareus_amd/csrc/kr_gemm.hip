@@ -190,7 +190,7 @@ struct Count { static constexpr int value = N; };
 
 // WN: 16-column MFMA tiles per wave along N (5..8): the workgroup's tile is 256 x 32 * WN.  Narrower
 // tiles let the host avoid a mostly empty last round of workgroups or a mostly padded last tile
-// column; the B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
+// column; a K-major B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
 template <bool A_T, bool B_T, int WN>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
@@ -201,6 +201,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int BN_ = 32 * WN;
+  // loads per wave of a B tile: a K-major tile's unused rows are simply not fetched; in a
+  // transposed tile every load spans all 256 columns
+  constexpr int NB_LOADS = B_T ? 8 : WN;
   const int wm = wave >> 1, wn = wave & 1;  // wave tile: rows wm*128.., columns wn*16*WN..
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_ - 1) / BN_;
   const int ntiles = tiles_m * tiles_n;
@@ -258,7 +261,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left);
     }
   };
-  // the first `count` loads of a tile (8 for A, WN for B)
+  // the first `count` loads of a tile (8 for A, NB_LOADS for B)
   auto request = [&](const bf16* base, const uint32_t (&off)[8], uint32_t slot, auto count_tag) {
     constexpr int COUNT = decltype(count_tag)::value;
     const uint32_t dst = slot + wave_blk;
@@ -275,11 +278,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   auto request_first_two = [&]() {
     set_offsets(nk == 1 ? k_tail : BK);
     request(a_base(0), la, r0, Count<8>{});
-    request(b_base(0), lb, r1, Count<WN>{});
+    request(b_base(0), lb, r1, Count<NB_LOADS>{});
     if (nk > 1) {
       if (nk == 2 && k_tail != BK) set_offsets(k_tail);
       request(a_base(1), la, r2, Count<8>{});
-      request(b_base(1), lb, r3, Count<WN>{});
+      request(b_base(1), lb, r3, Count<NB_LOADS>{});
     }
   };
   // After this wave's loads of the last K-step have landed (A in slot sa, B in slot sb): zero
@@ -387,8 +390,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     // K-step 0 complete in LDS (requested above, or before the previous item's epilogue); the
     // 16 loads of K-step 1 may still be in flight (loads retire in order)
     if (nk > 1) {
-      // vmcnt(8 + WN); lgkmcnt and expcnt untouched
-      __builtin_amdgcn_s_waitcnt(0x0f70 | ((8 + WN) & 15) | (((8 + WN) >> 4) << 14));
+      // vmcnt(8 + NB_LOADS); lgkmcnt and expcnt untouched
+      __builtin_amdgcn_s_waitcnt(0x0f70 | ((8 + NB_LOADS) & 15) | (((8 + NB_LOADS) >> 4) << 14));
     } else {
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
       fix_tail(r0, r1);
@@ -415,7 +418,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       half(X, Y, r0, r1, 1, Count<8>{}, a_base(t + 2), la, r4);
       __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
       __syncthreads();
-      half(Y, X, r2, r3, 0, Count<WN>{}, b_base(t + 2), lb, r0);
+      half(Y, X, r2, r3, 0, Count<NB_LOADS>{}, b_base(t + 2), lb, r0);
       rotate();
     }
     for (; t < nk; ++t) {

@@ -158,7 +158,11 @@ def test_row_strided_nanobatch_slices_need_no_copy(be):
 
 # ------------------------------------------------------------------ GEMM
 SHAPES = [(256, 256, 64), (512, 768, 512), (264, 520, 200), (1024, 2752, 512), (2048, 512, 1376),
-          (8, 8, 8), (4096, 640, 384), (40, 1536, 4096)]
+          (8, 8, 8), (4096, 640, 384), (40, 1536, 4096),
+          # outputs of 192 tiles or more, where the library picks narrower tiles than 256 columns:
+          (4096, 3584, 128),    # 224 columns (16 x 16 tiles fill one round of workgroups)
+          (16384, 768, 64),     # 192 columns
+          (16384, 640, 72)]     # 160 columns, and a contraction tail
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
