@@ -125,7 +125,7 @@ def partition_times(model, x, go, iters=3):
 # `bench.py --copy-calibration`: x2.000 and x1.000).  Keyed by (M, N, K); shapes that were not
 # profiled report null.
 MEASURED_TRAFFIC_BYTES = {
-    (4096, 7168, 4096): 369.5e6 + 58.7e6,
+    (4096, 7168, 4096): 369.7e6 + 58.7e6,
 }
 
 
