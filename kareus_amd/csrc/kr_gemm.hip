@@ -375,6 +375,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   int item = blockIdx.x;
   select_item(item);
   request_first_two();
+  // the accumulators start at zero: here for the first item (behind the latency of its first
+  // loads), in the epilogue for every later one (behind its LDS round trips)
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   for (;;) {
     {
@@ -383,10 +389,6 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       fa.init(wm * 128, lf);
       fb.init(wn * 16 * WN, lf);
     }
-#pragma unroll
-    for (int i = 0; i < WT; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     // K-step 0 complete in LDS (requested above, or before the previous item's epilogue); the
     // 16 loads of K-step 1 may still be in flight (loads retire in order)
     if (nk > 1) {
@@ -510,6 +512,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         for (int nt = 0; nt < WN; ++nt) {
           vals[nt] = acc[mt][nt];
           asm volatile("" : "+v"(vals[nt]));  // read here, not once in each branch below
+          acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + n_wave;
         if (narrow) {
