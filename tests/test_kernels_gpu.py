@@ -173,6 +173,17 @@ def test_gemm_three_layouts(be, m, n, k):
     assert rel(be.linear_wgrad(dy, x), dy.float().t() @ x.float()) <= TOL
 
 
+def test_gemm_is_reproducible(be):
+    """No atomics and a fixed order of accumulation: repeated launches give the same bits (a
+    race on an LDS tile between the waves of a workgroup would show up here)."""
+    m, n, k = 4096, 3584, 1088
+    x, w, dy = rnd(m, k, seed=14), rnd(n, k, scale=0.05, seed=15), rnd(m, n, seed=16)
+    first = (be.linear_fwd(x, w).clone(), be.linear_dgrad(dy, w).clone(), be.linear_wgrad(dy, x).clone())
+    for _ in range(5):
+        again = (be.linear_fwd(x, w), be.linear_dgrad(dy, w), be.linear_wgrad(dy, x))
+        assert all(torch.equal(a, b) for a, b in zip(again, first))
+
+
 def test_gemm_closed_forms(be):
     eye = torch.eye(512, device=DEV, dtype=torch.bfloat16)
     x = rnd(264, 512, seed=14)
