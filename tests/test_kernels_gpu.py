@@ -223,7 +223,9 @@ def _grouped(s, b, nq, nkv, hd, seed):
 @pytest.mark.parametrize("s,b,nq,nkv", [(128, 1, 1, 1), (256, 2, 4, 2), (512, 1, 3, 1), (384, 1, 8, 8), (1024, 1, 4, 1),
                                         (2048, 1, 2, 1),    # 32 query tiles per key tile: the steady state of the pipelines
                                         (512, 17, 8, 8),    # 544 workgroups, one query head per KV head: dK/dV written directly
-                                        (640, 3, 6, 2)])    # odd tile count, three query heads per KV head
+                                        (640, 3, 6, 2),     # odd tile count, three query heads per KV head
+                                        (256, 1, 24, 8),    # the head map of benchmark configuration 3 (Llama-3.2-3B)
+                                        (256, 2, 32, 8)])   # ... and of configuration 5 (Llama-3.1-8B), four query heads per KV head
 def test_attention_forward_backward(be, s, b, nq, nkv):
     hd = 128
     _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=22)
@@ -244,6 +246,21 @@ def test_attention_forward_backward(be, s, b, nq, nkv):
     assert torch.equal(od, o) and torch.equal(lsed, lse)
     dqd, dkd, dvd = be.attn_bwd(do, qd, k.contiguous(), v.contiguous(), od, lsed, hd ** -0.5)
     assert torch.equal(dqd, dq.flatten(2, 3)) and torch.equal(dkd, dk) and torch.equal(dvd, dv)
+
+
+def test_attention_at_sequence_8192(be):
+    """The sequence length of benchmark configuration 5, against the brute-force oracle (two query heads on
+    one KV head keep the oracle's 8192 x 8192 score matrices within a few seconds of CPU time)."""
+    s, b, nq, nkv, hd = 8192, 1, 2, 1, 128
+    _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=70)
+    do = rnd(s, b, nq, hd, seed=71)
+    o, lse = be.attn_fwd(q, k, v, hd ** -0.5)
+    dq, dk, dv = be.attn_bwd(do, q, k, v, o, lse, hd ** -0.5)
+    qf, kf, vf = (t.float().cpu().clone().requires_grad_(True) for t in (q.flatten(2, 3), k, v))
+    ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
+    assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
+    ro.backward(do.float().cpu())
+    assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
 
 
 def test_attention_does_not_depend_on_the_launch_size(be):

@@ -134,6 +134,120 @@ def test_full_size_properties_config4():
     assert torch.isfinite(y4).all() and torch.isfinite(dx4).all()
 
 
+# ---- benchmark configurations 3 and 5: full widths ------------------------------------------------
+C3 = R.LayerDims(3072, 24, 8, 128, 8192)     # Llama-3.2-3B layer, TP=1 (tests/bayesian/common/model_config.py:88-96)
+C5 = R.LayerDims(4096, 32, 8, 128, 14336)    # Llama-3.1-8B layer, full width
+
+
+@pytest.mark.parametrize("nnb", [1, 2, 4])
+def test_config3_widths_match_oracle(nnb):
+    """Configuration 3 at its full widths (24 query / 8 KV heads, ffn 8192), MBS 4, with the sequence cut to
+    256 so the CPU oracle finishes in seconds; nanobatch counts 1 (serial), 2 and 4."""
+    s, b = 256, 4
+    x, go = _inputs(s, b, C3.hidden)
+    model = _build(C3, 1, nnb)
+    y, dx, grads = _run(model, x, go)
+    ry, rdx, rgrads = _oracle(model, C3, x, go)
+    worst = [_rel(y, ry), _rel(dx, rdx)] + [_rel(grads[0][pi], rgrads[0][n]) for pi, (_, n) in enumerate(PARAMS)]
+    print(f"c3 nnb={nnb} max-rel={max(w[0] for w in worst):.3e} max-abs={max(w[1] for w in worst):.3e}")
+    assert max(w[0] for w in worst) <= TOL
+
+
+def _scheduled_step(model, sch, x, go):
+    """One microbatch under the activation-checkpointing plan: a forward and a backward instruction."""
+    for p in model.parameters():
+        p.grad = None
+    xd = x.to("cuda", torch.bfloat16).requires_grad_(True)
+    sch.on_instruction_begin("forward")
+    y = model(xd)
+    sch.on_instruction_end("forward")
+    sch.on_instruction_begin("backward")
+    y.backward(go.to("cuda", torch.bfloat16))
+    sch.on_instruction_end("backward")
+    torch.cuda.synchronize()
+    grads = [[getattr(layer, a).weight.grad.clone() for a, _ in PARAMS] for layer in model.layers]
+    return y.detach(), xd.grad, grads
+
+
+def test_config5_widths_match_oracle():
+    """One layer of configuration 5's widths (32 query / 8 KV heads, ffn 14336), MBS 2, two nanobatches, at the
+    single-layer tolerance."""
+    x, go = _inputs(256, 2, C5.hidden)
+    model = _build(C5, 1, 2)
+    y, dx, grads = _run(model, x, go)
+    ry, rdx, rgrads = _oracle(model, C5, x, go)
+    worst = [_rel(y, ry), _rel(dx, rdx)] + [_rel(grads[0][pi], rgrads[0][n]) for pi, (_, n) in enumerate(PARAMS)]
+    print(f"c5 one layer max-rel={max(w[0] for w in worst):.3e} max-abs={max(w[1] for w in worst):.3e}")
+    assert max(w[0] for w in worst) <= TOL
+
+
+def test_config5_stack_under_a_schedule_file_matches_oracle(fixtures_dir):
+    """Configuration 5 at its full widths, four layers, MBS 2, two nanobatches, activations recomputed, every
+    partition's launch slot taken from a schedule file (two microbatches: both steps of the plan are run and
+    checked); sequence cut to 256 for the oracle.
+
+    Tolerance: 2e-2 is the bf16 bound for ONE layer against fp32.  Through a stack every layer rounds its
+    activations and gradients to bf16 again and the independent rounding errors add in quadrature (measured
+    here: 1.1e-2 for one layer, 1.9e-2 for two, 2.6e-2 for four), so the bound for L layers is 2e-2 * sqrt(L);
+    the single-layer bound is checked by the test above, and the scheduled, recomputing run must equal the
+    plain run of the same stack bit for bit."""
+    s, b, layers = 256, 2, 4
+    tol = TOL * layers ** 0.5
+    model = _build(C5, layers, 2, checkpoint_activations=True)
+    plain = _build(C5, layers, 2)
+    sch = PipelineCommScheduler(os.path.join(fixtures_dir, "single_stage_ac.py"), pp_rank=0,
+                                num_microbatches=2, use_activation_checkpointing=True)
+    model.config.kareus_scheduler = sch
+    sch.on_step_begin()
+    for mb in range(2):
+        x, go = _inputs(s, b, C5.hidden, seed=42 + mb)
+        y, dx, grads = _scheduled_step(model, sch, x, go)
+        py, pdx, pgrads = _run(plain, x, go)
+        assert torch.equal(y, py) and torch.equal(dx, pdx)
+        assert all(torch.equal(a, c) for la, lb in zip(grads, pgrads) for a, c in zip(la, lb))
+        ry, rdx, rgrads = _oracle(model, C5, x, go)
+        worst = [_rel(y, ry), _rel(dx, rdx)]
+        for li in range(layers):
+            worst += [_rel(grads[li][pi], rgrads[li][n]) for pi, (_, n) in enumerate(PARAMS)]
+        print(f"c5 microbatch {mb} max-rel={max(w[0] for w in worst):.3e} max-abs={max(w[1] for w in worst):.3e}")
+        assert max(w[0] for w in worst) <= tol
+    sch.on_step_end()
+
+
+def _size_independent_properties(dims, layers, s, b, counts, cut, **kw):
+    """Properties that hold at any size: results do not depend on the nanobatch count, the layer is
+    causal end to end, the backward is linear in the upstream gradient, everything is finite."""
+    x, go = _inputs(s, b, dims.hidden)
+    runs = {n: _run(_build(dims, layers, n, **kw), x, go) for n in counts}
+    base = runs[counts[0]]
+    for n in counts[1:]:
+        y, dx, g = runs[n]
+        assert _rel(y, base[0])[0] <= TOL and _rel(dx, base[1])[0] <= TOL
+        for la, lb in zip(g, base[2]):
+            for ga, gb in zip(la, lb):
+                assert _rel(ga, gb)[0] <= TOL
+    n = counts[-1]
+    x2 = x.clone()
+    x2[cut:] += 1.0
+    y2, _, _ = _run(_build(dims, layers, n, **kw), x2, go)
+    assert torch.equal(y2[:cut], runs[n][0][:cut]) and not torch.equal(y2[cut:], runs[n][0][cut:])
+    _, dx_double, _ = _run(_build(dims, layers, n, **kw), x, 2 * go)
+    assert torch.equal(dx_double, 2 * runs[n][1])
+    for y, dx, g in runs.values():
+        assert torch.isfinite(y).all() and torch.isfinite(dx).all()
+        assert all(torch.isfinite(t).all() for layer in g for t in layer)
+
+
+def test_full_size_properties_config3():
+    """Configuration 3 at full size (h3072, 24q/8kv, ffn 8192, MBS 4 x seq 4096), nanobatch counts 1, 2, 4."""
+    _size_independent_properties(C3, 1, 4096, 4, [1, 2, 4], cut=3072)
+
+
+def test_full_size_properties_config5():
+    """Configuration 5 at full size (4 layers, h4096, 32q/8kv, ffn 14336, MBS 2 x seq 8192, 2 nanobatches)."""
+    _size_independent_properties(C5, 4, 8192, 2, [1, 2], cut=6144)
+
+
 def test_nanobatch_streams_do_not_share_a_hardware_queue():
     """Streams handed to the nanobatches must overlap for real: a short kernel on one finishes
     while a spinning kernel occupies the other."""
