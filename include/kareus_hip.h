@@ -84,6 +84,20 @@ int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd, const v
                        const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
                        int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
 
+/* kr_rmsnorm_bwd_add without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The fp32 partial rows of the weight gradient go to a 16 MiB array
+ * that the library holds in device memory on every GPU it runs on until the process ends; the
+ * call itself allocates and frees nothing (its first call on a device looks the array's address
+ * up, so make one call per device before a region in which even that is unwelcome).
+ * cols above 8192 return KR_EUNSUPPORTED.  Results are bit-identical to kr_rmsnorm_bwd_add.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams
+ * or threads) race on it and must be ordered by the caller.                                     */
+int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const float* rstd, const void* gamma,
+                               const void* dres, void* dx, void* dgamma, int rows, int cols,
+                               int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld,
+                               void* stream);
+
 /* ---- Rotary position embedding ---------------------------------------------------------
  * Replaces fused_rotary_positional_embedding.forward / backward (Apex), called from
  * kareus/apex/transformer/functional/fused_rope.py:27-35, 41-46.

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_rmsnorm_bwd_add": (_c_int, [_c_void_p] * 8 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
+    "kr_rmsnorm_bwd_add_noalloc": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
     "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
                 + [_c_int, _c_int, _c_int, _c_void_p]),
     "kr_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),

@@ -7,6 +7,8 @@
 // in registers (a lane always owns the same columns), the waves of a block combine through
 // LDS, each block writes one fp32 partial row into the workspace, and a second small kernel
 // sums the partial rows and rounds to bf16.
+#include <mutex>
+
 #include "kr_common.h"
 
 namespace {
@@ -270,10 +272,67 @@ extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
   return (size_t)bwd_blocks(rows, cols) * (size_t)cols * sizeof(float);
 }
 
+namespace {
+int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const void* gamma,
+                     const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
+                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
+}
+
 extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd,
                                   const void* gamma, const void* dres, void* dx, void* dgamma,
                                   void* workspace, int rows, int cols, int64_t dy_ld, int64_t x_ld,
                                   int64_t dres_ld, int64_t dx_ld, void* stream) {
+  return rmsnorm_bwd_impl(dy, x, rstd, gamma, dres, dx, dgamma, workspace, rows, cols, dy_ld, x_ld,
+                          dres_ld, dx_ld, stream);
+}
+
+// ---- the variant that allocates nothing --------------------------------------------------------
+// The partial rows of the weight gradient (at most kMaxBwdBlocks rows of at most 8192 columns,
+// fp32: 16 MiB) live in a file-scope device array instead of a caller workspace.  Each GPU holds
+// its own copy of the array at its own address; the address is looked up once per device.
+namespace {
+constexpr int kScratchCols = 8192;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) float scratch[(size_t)kMaxBwdBlocks * kScratchCols];
+namespace {
+std::mutex scratch_mutex;
+float* scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until looked up
+
+// The device address of `scratch` on the current device (never the array's name: in host code that
+// is a host-side stand-in, not a device address).
+float* scratch_on_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    scratch_ptr[dev] = (float*)p;
+  }
+  return scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const float* rstd,
+                                          const void* gamma, const void* dres, void* dx,
+                                          void* dgamma, int rows, int cols, int64_t dy_ld,
+                                          int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream) {
+  if (rows <= 0 || cols <= 0) return KR_EINVAL;
+  if (cols > kScratchCols) return KR_EUNSUPPORTED;  // beyond what the device array holds
+  float* const ws = scratch_on_current_device();
+  if (ws == nullptr) return KR_ELAUNCH;
+  return rmsnorm_bwd_impl(dy, x, rstd, gamma, dres, dx, dgamma, ws, rows, cols, dy_ld, x_ld, dres_ld,
+                          dx_ld, stream);
+}
+
+namespace {
+int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const void* gamma,
+                     const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
+                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream) {
   if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0 ||
       dy_ld < cols || x_ld < cols || dx_ld < cols || (dres && dres_ld < cols))
     return KR_EINVAL;
@@ -311,6 +370,7 @@ extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rs
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
   return kr_launch_status();
 }
+}  // namespace
 
 extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
                               void* dx, void* dgamma, void* workspace, int rows, int cols,
