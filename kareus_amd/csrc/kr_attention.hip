@@ -17,6 +17,8 @@
 //   P nor V is ever transposed through memory.
 // Tensors are addressed through (seq, batch, head) strides, so sequence-major [s, b, h, d]
 // views of the fused QKV projection are consumed in place.
+#include <initializer_list>
+
 #include "kr_common.h"
 
 namespace {
@@ -133,6 +135,17 @@ static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
   if (s <= 0 || b <= 0 || nq <= 0 || nkv <= 0) return KR_EINVAL;
   if (hd != HD || s % BQ || nq % nkv) return KR_EUNSUPPORTED;
   return KR_OK;
+}
+
+// The kernels keep a sequence stride in 32 bits and build per-lane byte offsets of up to
+// (48 * stride + 128) * 2 from it: strides must be positive and small enough for that.
+template <size_t N>
+inline bool attn_strides_ok(const int64_t (&seq)[N], std::initializer_list<int64_t> others) {
+  for (int64_t ss : seq)
+    if (ss <= 0 || 48 * ss + 128 >= ((int64_t)1 << 31)) return false;
+  for (int64_t st : others)
+    if (st <= 0) return false;
+  return true;
 }
 
 // =============================================================================================
@@ -1084,6 +1097,12 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
        o_sh | do_ss | do_sb | do_sg | do_sh | dq_ss | dq_sb | dq_sg | dq_sh | dk_ss | dk_sb |
        dk_sh | dv_ss | dv_sb | dv_sh) % 8)
     return KR_EINVAL;
+  {
+    const int64_t seq[] = {q_ss, k_ss, v_ss, o_ss, do_ss, dq_ss, dk_ss, dv_ss};
+    if (!attn_strides_ok(seq, {q_sb, q_sg, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sg, o_sh, do_sb, do_sg,
+                               do_sh, dq_sb, dq_sg, dq_sh, dk_sb, dk_sh, dv_sb, dv_sh}))
+      return KR_EUNSUPPORTED;
+  }
   hipStream_t st = (hipStream_t)stream;
   const QLayout ql{q_ss, q_sb, q_sg, q_sh}, ol{o_ss, o_sb, o_sg, o_sh}, dol{do_ss, do_sb, do_sg, do_sh},
       dql{dq_ss, dq_sb, dq_sg, dq_sh};
@@ -1164,6 +1183,11 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
   if ((q_ss | q_sb | q_sg | q_sh | k_ss | k_sb | k_sh | v_ss | v_sb | v_sh | o_ss | o_sb | o_sg |
        o_sh) % 8)
     return KR_EINVAL;
+  {
+    const int64_t seq[] = {q_ss, k_ss, v_ss, o_ss};
+    if (!attn_strides_ok(seq, {q_sb, q_sg, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sg, o_sh}))
+      return KR_EUNSUPPORTED;
+  }
   // two K and two V tiles of 17 KiB (padded blocks) per half; afterwards the same memory holds
   // the hand-over of half 1 (66 KiB) and, from 68 KiB on, 4 KiB of output staging per wave
   constexpr size_t lds_pp = 2 * 2 * 16 * ((1024 + 16) + (1024 + 64));  // 133 KiB

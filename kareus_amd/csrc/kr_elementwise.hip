@@ -193,6 +193,7 @@ extern "C" int kr_rope(const void* t, void* out, const float* freqs, int s, int 
   if (hd % 16 || hd > 256) return KR_EUNSUPPORTED;
   if (!kr_aligned16(t) || !kr_aligned16(out)) return KR_EINVAL;
   if ((ts | tb | th | os | ob | oh) % 8) return KR_EINVAL;
+  if (ts <= 0 || tb <= 0 || th <= 0 || os <= 0 || ob <= 0 || oh <= 0) return KR_EUNSUPPORTED;
   hipLaunchKernelGGL(rope_kernel, dim3(s), dim3(kThreads), 0, (hipStream_t)stream,
                      (const bf16*)t, (bf16*)out, freqs, b, heads, hd, ts, tb, th, os, ob, oh,
                      backward ? -1.0f : 1.0f, group_size, group_rotate);

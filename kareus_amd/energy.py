@@ -12,16 +12,56 @@ then report energy as unmeasured instead of guessing.
 from __future__ import annotations
 
 import glob
+import os
 import threading
 import time
 from typing import Callable, List, Optional, Tuple
 
 
+def pci_bus_id(device_index: int = 0) -> Optional[str]:
+    """``dddd:bb:dd.f`` of the HIP device with this index (the index already reflects
+    HIP_VISIBLE_DEVICES / ROCR_VISIBLE_DEVICES), or None without a device."""
+    try:
+        import torch
+
+        if not torch.cuda.is_available() or device_index >= torch.cuda.device_count():
+            return None
+        p = torch.cuda.get_device_properties(device_index)
+        return f"{p.pci_domain_id:04x}:{p.pci_bus_id:02x}:{p.pci_device_id:02x}.0"
+    except Exception:
+        return None
+
+
+def _card_number(path: str) -> int:
+    digits = "".join(ch for ch in os.path.basename(path) if ch.isdigit())
+    return int(digits) if digits else -1
+
+
+def sysfs_device_dir(device_index: int = 0, sysfs_root: str = "/sys",
+                     bus_id: Optional[str] = None) -> Optional[str]:
+    """The amdgpu sysfs directory of the HIP device: ``/sys/bus/pci/devices/<bus id>`` or the
+    ``/sys/class/drm/card*/device`` link that resolves to that bus id.  None when the device's bus
+    id is unknown or no node matches it: the position of a card in a directory listing says
+    nothing about which GPU this process was given, so it is never used to pick one."""
+    bdf = bus_id if bus_id is not None else pci_bus_id(device_index)
+    if bdf is None:
+        return None
+    direct = os.path.join(sysfs_root, "bus", "pci", "devices", bdf)
+    if os.path.isdir(direct):
+        return direct
+    cards = glob.glob(os.path.join(sysfs_root, "class", "drm", "card[0-9]*", "device"))
+    for dev in sorted(cards, key=lambda d: _card_number(os.path.dirname(d))):
+        if os.path.basename(os.path.realpath(dev)) == bdf:
+            return dev
+    return None
+
+
 def _sysfs_reader(device_index: int) -> Optional[Callable[[], float]]:
+    dev = sysfs_device_dir(device_index)
+    if dev is None:
+        return None
     for name in ("power1_input", "power1_average"):
-        paths = sorted(glob.glob(f"/sys/class/drm/card*/device/hwmon/hwmon*/{name}"))
-        if len(paths) > device_index:
-            path = paths[device_index]
+        for path in sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", name))):
 
             def read(path=path) -> float:
                 with open(path) as f:
@@ -40,7 +80,11 @@ def _amdsmi_reader(device_index: int) -> Optional[Callable[[], float]]:
         import amdsmi  # type: ignore
 
         amdsmi.amdsmi_init()
-        handle = amdsmi.amdsmi_get_processor_handles()[device_index]
+        bdf = pci_bus_id(device_index)
+        handle = next((h for h in amdsmi.amdsmi_get_processor_handles()
+                       if str(amdsmi.amdsmi_get_gpu_device_bdf(h)).lower() == bdf), None)
+        if bdf is None or handle is None:
+            return None
 
         def read() -> float:
             info = amdsmi.amdsmi_get_power_info(handle)
@@ -59,6 +103,7 @@ def _amdsmi_reader(device_index: int) -> Optional[Callable[[], float]]:
 class PowerSampler:
     def __init__(self, device_index: int = 0, hz: float = 100.0) -> None:
         self._read = _sysfs_reader(device_index) or _amdsmi_reader(device_index)
+        self.bus_id = pci_bus_id(device_index)  # which GPU the readings belong to
         self.available = self._read is not None
         self.period = 1.0 / hz
         self.samples: List[Tuple[float, float]] = []

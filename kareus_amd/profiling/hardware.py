@@ -15,14 +15,13 @@ False and rows carry the requested value with ``freq_applied: false``.
 
 from __future__ import annotations
 
-import glob
 import json
 import os
 import time
 from dataclasses import dataclass
 from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
 
-from ..energy import PowerSampler
+from ..energy import PowerSampler, sysfs_device_dir
 
 
 @dataclass(frozen=True)
@@ -87,8 +86,10 @@ def measure(
 
 # ---- clock control (best effort) -------------------------------------------------------------
 def _device_dir(device_index: int) -> Optional[str]:
-    cards = sorted(glob.glob("/sys/class/drm/card[0-9]*/device/pp_dpm_sclk"))
-    return os.path.dirname(cards[device_index]) if len(cards) > device_index else None
+    """sysfs directory of the HIP device, found by its PCI bus id; None (no clock is touched)
+    when it cannot be matched."""
+    d = sysfs_device_dir(device_index)
+    return d if d is not None and os.path.exists(os.path.join(d, "pp_dpm_sclk")) else None
 
 
 def available_frequencies_mhz(device_index: int = 0) -> List[int]:
@@ -121,9 +122,13 @@ def set_gpu_frequency(target_freq_mhz: int, device_index: int = 0, settle_s: flo
     try:
         with open(os.path.join(d, "power_dpm_force_performance_level"), "w") as f:
             f.write("manual")
+    except OSError:
+        return False
+    try:
         with open(os.path.join(d, "pp_dpm_sclk"), "w") as f:
             f.write(str(level))
     except OSError:
+        reset_gpu_clocks(device_index)  # do not leave the card in manual mode without a level
         return False
     if settle_s > 0:
         time.sleep(settle_s)

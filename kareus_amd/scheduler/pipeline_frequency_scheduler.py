@@ -35,7 +35,7 @@ class PipelineFrequencyScheduler:
     the instruction kind and switches the clock when the value differs from the current one.
 
     ``history`` lists ``(name, MHz, applied)`` for the instructions of the current step;
-    ``current_frequency`` is the MHz value last requested.
+    ``current_frequency`` is the MHz value last applied (None until a write succeeds).
     """
 
     def __init__(
@@ -82,9 +82,12 @@ class PipelineFrequencyScheduler:
         if expected != name:
             raise RuntimeError(f"Frequency plan mismatch: expected '{expected}', got '{name}'")
         if mhz != self.current_frequency:
+            # only a write that went through sets the clock in force; after a failed one the clock
+            # is unknown (the setter may have handed it back to the governor), so the next
+            # instruction tries again whatever its value
             self.applied = bool(self._set(mhz))
-            self.current_frequency = mhz
-        self.history.append((name, mhz, self.applied))
+            self.current_frequency = mhz if self.applied else None
+        self.history.append((name, mhz, self.current_frequency == mhz))
 
     def on_instruction_end(self, name: Optional[str] = None) -> None:
         pass

@@ -54,3 +54,32 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 128) == 2 * 256 * 4 * 4 + 2 * 256 * 4 * 2 * 128 * 4
     assert lib.kr_gemm_workspace_bytes(2, 1536, 4096, 16384) > 0 and lib.kr_gemm_workspace_bytes(0, 4096, 7168, 4096) == 0
     assert lib.kr_rmsnorm_bwd_workspace_bytes(8192, 4096) == 512 * 4096 * 4
+
+
+def test_strides_the_kernels_cannot_index_are_refused():
+    """Attention keeps sequence strides in 32 bits (per-lane byte offsets up to (48 * stride + 128) * 2) and no
+    kernel walks backwards: a stride that is not positive or too long is an error, not a wild load."""
+    lib = hip.load_library()
+    good = [1024, 256, 128, 128] + [1024, 256, 128] * 2 + [1024, 256, 128, 128]
+    args = lambda st: [16, 16, 16, 16, 16, 128, 1, 1, 1, 128, 1.0] + st + [None]
+    too_long = (1 << 31) // 48 // 8 * 8
+    for pos in (0, 4, 7, 10):                                  # the four sequence strides
+        bad = list(good)
+        bad[pos] = too_long
+        assert lib.kr_attn_fwd(*args(bad)) == -2
+        bad[pos] = -1024
+        assert lib.kr_attn_fwd(*args(bad)) == -2
+    bad = list(good)
+    bad[1] = 0                                                 # a batch stride of zero
+    assert lib.kr_attn_fwd(*args(bad)) == -2
+    bwd_good = good + [1024, 256, 128, 128] * 2 + [1024, 256, 128] * 2
+    bwd = lambda st: [16] * 10 + [128, 1, 1, 1, 128, 1.0] + st + [None]
+    for pos in (0, 14, 18, 22, 25):
+        bad = list(bwd_good)
+        bad[pos] = too_long
+        assert lib.kr_attn_bwd(*bwd(bad)) == -2
+        bad[pos] = -8
+        assert lib.kr_attn_bwd(*bwd(bad)) == -2
+    rope = lambda st: [16, 16, 16, 4, 1, 2, 128] + st + [0, 1, 1, None]
+    assert lib.kr_rope(*rope([-256, 256, 128, 256, 256, 128])) == -2
+    assert lib.kr_rope(*rope([256, 256, 128, 256, 0, 128])) == -2

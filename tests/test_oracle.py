@@ -200,3 +200,61 @@ def test_layer_is_per_sample_and_param_order():
     z = {k: (torch.zeros_like(t) if k in ("w_proj", "w_fc2") else t) for k, t in p[0].items()}
     f = R.rope_table(10, dims.hd, dims.rope_base, dtype=D)
     assert torch.equal(R.layer_forward(x, z, dims, f), x)
+
+
+def _library_layer(x, p, dims, skip_rope=False):
+    """The layer built from PyTorch library routines only, in the operator order of
+    kareus/megatron/core/transformer/transformer_layer.py:148-174: rms_norm -> linear -> per-group
+    (q.., k, v) split -> rotary position embedding as a complex multiplication -> causal
+    grouped-query scaled_dot_product_attention -> linear -> residual add -> rms_norm -> linear ->
+    silu(gate) * up -> linear -> residual add.  Shares no code with the oracle."""
+    F = torch.nn.functional
+    s, b, h = x.shape
+    per, hd = dims.nq // dims.nkv, dims.hd
+    h1 = F.rms_norm(x, (h,), p["ln1"], dims.eps)
+    mixed = F.linear(h1, p["w_qkv"]).view(s, b, dims.nkv, per + 2, hd)
+    q, k, v = mixed[:, :, :, :per].reshape(s, b, dims.nq, hd), mixed[:, :, :, per], mixed[:, :, :, per + 1]
+    if not skip_rope:
+        # halves layout: channel i pairs with i + hd/2; rotating the pair by angle a_i is the
+        # complex product (t_i + j t_{i+hd/2}) * exp(j a_i)
+        inv = dims.rope_base ** (-torch.arange(0, hd, 2, dtype=x.dtype) / hd)
+        rot = torch.polar(torch.ones(s, hd // 2, dtype=x.dtype), torch.arange(s, dtype=x.dtype)[:, None] * inv)
+
+        def rotate(t):
+            z = torch.complex(t[..., : hd // 2], t[..., hd // 2:]) * rot[:, None, None, :]
+            return torch.cat((z.real, z.imag), dim=-1)
+
+        q, k = rotate(q), rotate(k)
+    o = F.scaled_dot_product_attention(q.permute(1, 2, 0, 3), k.permute(1, 2, 0, 3), v.permute(1, 2, 0, 3),
+                                       is_causal=True, enable_gqa=True)
+    x = x + F.linear(o.permute(2, 0, 1, 3).reshape(s, b, dims.nq * hd), p["w_proj"])
+    gate, up = F.linear(F.rms_norm(x, (h,), p["ln2"], dims.eps), p["w_fc1"]).chunk(2, dim=-1)
+    return x + F.linear(F.silu(gate) * up, p["w_fc2"])
+
+
+def test_layer_composition_equals_a_layer_of_library_routines():
+    """Pins the composition (operator order, the q/k/v split feeding rope and attention, both residual adds):
+    the oracle's layer equals one assembled from library routines in fp64, for values and for every gradient,
+    and the comparison notices a missing rotary embedding."""
+    dims = R.LayerDims(hidden=48, nq=6, nkv=2, hd=16, ffn=40)
+    gen = torch.Generator().manual_seed(7)
+    p = R.init_layer_params(dims, gen, std=0.3, dtype=D)
+    p["ln1"] = 1 + 0.2 * torch.randn(48, generator=gen, dtype=D)
+    p["ln2"] = 1 + 0.2 * torch.randn(48, generator=gen, dtype=D)
+    x = torch.randn(12, 3, 48, generator=gen, dtype=D)
+    go = torch.randn(12, 3, 48, generator=gen, dtype=D)
+    y, dx, grads = R.stack_forward_backward(x, [p], dims, go)
+    xl = x.clone().requires_grad_(True)
+    pl = {k: t.clone().requires_grad_(True) for k, t in p.items()}
+    yl = _library_layer(xl, pl, dims)
+    yl.backward(go)
+    assert torch.allclose(yl, y, atol=1e-11) and torch.allclose(xl.grad, dx, atol=1e-10)
+    for name in R.PARAM_ORDER:
+        assert torch.allclose(pl[name].grad, grads[0][name], atol=1e-9), name
+    # two layers: the stack is the composition of the layers
+    p2 = R.init_layer_params(dims, gen, std=0.3, dtype=D)
+    f = R.rope_table(12, dims.hd, dims.rope_base, dtype=D)
+    assert torch.allclose(R.stack_forward(x, [p, p2], dims, f),
+                          _library_layer(_library_layer(x, p, dims), p2, dims), atol=1e-11)
+    # the check has teeth: without the rotary embedding the library layer is somewhere else
+    assert (_library_layer(x, p, dims, skip_rope=True) - y).abs().max() > 1e-3

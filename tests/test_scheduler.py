@@ -206,3 +206,38 @@ def test_scheduler_state_machine_per_microbatch(fixtures_dir):
     again = PipelineCommScheduler.from_parsed(parsed, 0, 2)
     again.on_instruction_begin("forward")
     assert again.current_schedule == first
+
+
+def test_a_failed_clock_write_is_retried_and_never_recorded_as_applied(fixtures_dir):
+    from kareus_amd.scheduler import PipelineFrequencyScheduler
+
+    path = os.path.join(fixtures_dir, "freqs_pipeline_02328.py")
+    plan = parse_frequency_file(path)[0]
+    outcomes = iter([False, True] + [True] * 64)
+    calls = []
+    sch = PipelineFrequencyScheduler(path, pp_rank=0, set_frequency=lambda mhz: (calls.append(mhz), next(outcomes))[1],
+                                     reset_frequency=lambda: True)
+    sch.on_step_begin()
+    sch.on_instruction_begin(plan[0][0])
+    assert sch.current_frequency is None and sch.history[-1][2] is False
+    sch.on_instruction_begin(plan[1][0])          # tried again even if the planned value is the same
+    assert len(calls) == 2 and sch.current_frequency == plan[1][1] and sch.history[-1][2] is True
+    assert sch.history[0][2] is False             # the earlier row still says the truth
+
+
+def test_sysfs_node_is_found_by_pci_bus_id_not_by_listing_order(tmp_path):
+    """card10 sorts before card2 as text and a one-GPU lease may be any card: the node is matched by bus id."""
+    from kareus_amd.energy import sysfs_device_dir
+
+    root = tmp_path / "sys"
+    for card, bdf in ((0, "0000:05:00.0"), (2, "0000:15:00.0"), (10, "0000:85:00.0")):
+        real = root / "devices" / "pci0000:00" / bdf
+        real.mkdir(parents=True)
+        (root / "class" / "drm" / f"card{card}").mkdir(parents=True)
+        os.symlink(real, root / "class" / "drm" / f"card{card}" / "device")
+    got = sysfs_device_dir(0, sysfs_root=str(root), bus_id="0000:85:00.0")
+    assert got is not None and os.path.realpath(got).endswith("0000:85:00.0")
+    assert sysfs_device_dir(0, sysfs_root=str(root), bus_id="0000:99:00.0") is None   # no match: nothing is picked
+    (root / "bus" / "pci" / "devices").mkdir(parents=True)
+    os.symlink(root / "devices" / "pci0000:00" / "0000:15:00.0", root / "bus" / "pci" / "devices" / "0000:15:00.0")
+    assert sysfs_device_dir(0, sysfs_root=str(root), bus_id="0000:15:00.0").endswith("bus/pci/devices/0000:15:00.0")
