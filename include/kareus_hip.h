@@ -59,6 +59,31 @@ int kr_gemm_bf16(int layout, int M, int N, int K,
                  void* C, int64_t ldc, int accumulate,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same GEMM with an operation fused into its epilogue and an optional compute-unit budget.
+ * epilogue:
+ *   KR_GEMM_EPI_NONE    plain kr_gemm_bf16.
+ *   KR_GEMM_EPI_ADD     C = bf16(bf16(A.B) + aux), aux [M,N] bf16 with row stride ld_aux: the residual
+ *                       add behind a row-parallel projection (fused_bias_dropout_add_forward with p = 0,
+ *                       no bias, kareus/megatron/core/extensions/ops/bias_dropout_add.py:15-32) done where
+ *                       the projection's output is produced (te_linear.py:188-206 writes that output
+ *                       straight into its consumer's buffer); bit-identical to kr_gemm_bf16 + kr_add.
+ *   KR_GEMM_EPI_SWIGLU  N = 2F, F a multiple of 80, 96, 112 or 128: C = x [M, 2F] as usual and
+ *                       out2 [M, F] (row stride ld_out2) = silu(x[:, :F]) * x[:, F:] computed from the
+ *                       bf16-rounded x (fused_swiglu_forward, bias_swiglu.py:14-20); bit-identical to
+ *                       kr_gemm_bf16 + kr_swiglu_fwd.
+ *   A fused epilogue needs layout TN and accumulate == 0 and is never computed split-K.
+ * max_cus > 0 limits the launch to that many compute units (workgroups are persistent, one per
+ * unit): the compute-unit share a schedule's resource_shape gives a partition
+ * (kareus/megatron/core/partitions/partition_base.py:117-128); 0 = the whole device.             */
+#define KR_GEMM_EPI_NONE 0
+#define KR_GEMM_EPI_ADD 1
+#define KR_GEMM_EPI_SWIGLU 2
+int kr_gemm_bf16_fused(int layout, int M, int N, int K,
+                       const void* A, int64_t lda, const void* B, int64_t ldb,
+                       void* C, int64_t ldc, int accumulate,
+                       int epilogue, const void* aux, int64_t ld_aux, void* out2, int64_t ld_out2,
+                       int max_cus, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- RMSNorm ---------------------------------------------------------------------------
  * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd
  * (kareus/transformer_engine/pytorch/ops/basic/rmsnorm.py:210-219, 256-263).

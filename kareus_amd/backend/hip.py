@@ -27,6 +27,9 @@ _SIGNATURES = {
     "kr_gemm_workspace_bytes_shared": (_c_size_t, [_c_int, _c_int, _c_int, _c_int, _c_float]),
     "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
                               _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
+    "kr_gemm_bf16_fused": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
+                                    _c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
+                                    _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
@@ -75,6 +78,7 @@ class HipBackend:
     def __init__(self) -> None:
         self.lib = load_library()
         self._gemm_ws_bytes: dict = {}  # (layout, m, n, k, split_k) -> workspace bytes
+        self._ws_cache: dict = {}       # (stream, device) -> reusable workspace buffer
 
     # -- plumbing -------------------------------------------------------------------
     # the raw handle of the current stream without building a torch.cuda.Stream object: this is
@@ -112,33 +116,79 @@ class HipBackend:
                 raise RuntimeError(f"the hip backend computes in bf16, got {t.dtype}")
 
     # -- GEMM -------------------------------------------------------------------------
+    def _workspace(self, nbytes: int, device) -> Tensor:
+        """A workspace of at least ``nbytes`` for the current stream.  One buffer per (stream, size
+        class) is kept and reused: kernels on one stream run in order, so consecutive launches may
+        share it, and a fresh ``torch.empty`` per launch costs more host time than the launch."""
+        key = (self._stream(), device.index)
+        buf = self._ws_cache.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+            self._ws_cache[key] = buf
+        return buf
+
     def gemm(self, layout: int, a: Tensor, b: Tensor, m: int, n: int, k: int,
-             out: Tensor = None, accumulate: bool = False, split_k: bool = True) -> Tensor:
+             out: Tensor = None, accumulate: bool = False, split_k: bool = True,
+             residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0) -> Tensor:
         """``split_k=True``: the GEMM has the GPU to itself and splits the contraction of a small
         output for the shortest latency.  ``split_k=False``: kernels of other streams are there
         to use the CUs a small output leaves idle, so the split count is chosen mostly for the
-        least CU-time (often no split at all)."""
+        least CU-time (often no split at all).
+        ``residual`` ([m, n], row-strided): added to the bf16-rounded product in the epilogue.
+        ``swiglu_out`` ([m, n/2]): also receives silu(out[:, :n/2]) * out[:, n/2:] (layout TN).
+        ``max_cus``: compute-unit budget of the launch (0 = the whole device)."""
         self._dev(a, b)
         self._bf16(a, b)
         if a.stride(-1) != 1 or b.stride(-1) != 1:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
             out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-        key = (layout, m, n, k, split_k)
-        ws_bytes = self._gemm_ws_bytes.get(key)
-        if ws_bytes is None:
-            ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
-                        self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
-            self._gemm_ws_bytes[key] = ws_bytes
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-        rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
-                                   out.data_ptr(), out.stride(0), int(accumulate),
-                                   ws.data_ptr() if ws is not None else None, ws_bytes, self._stream())
-        self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k})")
+        epi, aux_ptr, aux_ld, out2_ptr, out2_ld = 0, None, 0, None, 0
+        if residual is not None:
+            self._dev(residual)
+            self._bf16(residual)
+            if tuple(residual.shape) != (m, n) or residual.stride(1) != 1:
+                raise RuntimeError("GEMM residual must be [M, N] with a contiguous last dimension")
+            epi, aux_ptr, aux_ld = 1, residual.data_ptr(), residual.stride(0)
+        if swiglu_out is not None:
+            if residual is not None:
+                raise RuntimeError("one fused epilogue at a time")
+            self._dev(swiglu_out)
+            self._bf16(swiglu_out)
+            if tuple(swiglu_out.shape) != (m, n // 2) or swiglu_out.stride(1) != 1:
+                raise RuntimeError("swiglu_out must be [M, N/2] with a contiguous last dimension")
+            epi, out2_ptr, out2_ld = 2, swiglu_out.data_ptr(), swiglu_out.stride(0)
+        ws_bytes, ws_ptr = 0, None
+        if epi == 0 and split_k is not None:   # split_k=None: never split (no workspace is handed over)
+            key = (layout, m, n, k, split_k)
+            ws_bytes = self._gemm_ws_bytes.get(key)
+            if ws_bytes is None:
+                ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
+                            self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
+                self._gemm_ws_bytes[key] = ws_bytes
+            if ws_bytes:
+                ws_ptr = self._workspace(ws_bytes, a.device).data_ptr()
+        if epi == 0 and max_cus == 0:
+            rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
+                                       out.data_ptr(), out.stride(0), int(accumulate), ws_ptr, ws_bytes,
+                                       self._stream())
+        else:
+            rc = self.lib.kr_gemm_bf16_fused(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(),
+                                             b.stride(0), out.data_ptr(), out.stride(0), int(accumulate),
+                                             epi, aux_ptr, aux_ld, out2_ptr, out2_ld, int(max_cus),
+                                             ws_ptr, ws_bytes, self._stream())
+        self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k}, epilogue={epi})")
         return out
 
-    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
-        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1], split_k=split_k)
+    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True, out: Tensor = None,
+                   residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0) -> Tensor:
+        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1], out=out, split_k=split_k,
+                         residual=residual, swiglu_out=swiglu_out, max_cus=max_cus)
+
+    @staticmethod
+    def can_fuse_swiglu(two_f: int) -> bool:
+        """Whether a projection of this output width can produce the SwiGLU activation in its epilogue."""
+        return two_f % 2 == 0 and any(two_f % (32 * wn) == 0 for wn in (5, 6, 7, 8))
 
     def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
         return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1], split_k=split_k)
@@ -195,7 +245,7 @@ class HipBackend:
             residual_grad = self._rows(residual_grad)
             res_ptr, res_ld = residual_grad.data_ptr(), residual_grad.stride(0)
         dgamma = torch.empty_like(gamma)
-        ws = torch.empty(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), dtype=torch.uint8, device=x.device)
+        ws = self._workspace(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), x.device)
         rc = self.lib.kr_rmsnorm_bwd_add(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
                                          res_ptr, dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols,
                                          dy.stride(0), x.stride(0), res_ld, dx.stride(0), self._stream())
@@ -430,7 +480,7 @@ class HipBackend:
             dk = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
             dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
         nbytes = self.lib.kr_attn_bwd_workspace_bytes(s, b, nq, nkv, hd)
-        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+        ws = self._workspace(max(nbytes, 16), q.device)
         rc = self.lib.kr_attn_bwd(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
                                   lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
                                   s, b, nq, nkv, hd, scale,

@@ -46,6 +46,11 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// SwiGLU on one element, fp32: silu(gate) * up.  One definition for the stand-alone kernel and the
+// GEMM epilogue that fuses it, so that the two produce the same bits.
+__device__ __forceinline__ float kr_sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float kr_swiglu_f(float gate, float up) { return gate * kr_sigmoidf(gate) * up; }
+
 static inline bool kr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static inline int kr_launch_status() {

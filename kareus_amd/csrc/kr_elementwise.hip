@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void add_rows_kernel(const bf16* a, int64
   }
 }
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoidf_(float x) { return kr_sigmoidf(x); }
 
 // x [rows, 2F] -> y [rows, F]; one thread per 8 output columns.
 __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const bf16* __restrict__ x,
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const bf16* __rest
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float x1 = (float)g[e], x2 = (float)u[e];
-      o[e] = (bf16)(x1 * sigmoidf_(x1) * x2);
+      o[e] = (bf16)kr_swiglu_f(x1, x2);
     }
     stg8(y + r * F + c, o);
   }

@@ -98,13 +98,19 @@ __device__ __forceinline__ uint32_t lds_addr(const bf16* p) {
 // clamped to the last valid row; a chunk that would start beyond the contraction range
 // (k_left = elements from the K-step's base to the end, >= 8) is redirected to a valid address —
 // it is zeroed in LDS afterwards, so what it fetches does not matter.
+// gate_up_f > 0 (K-major B of a fused SwiGLU projection, weight rows [gate: 0..F) | up: F..2F)):
+// the first `half_rows` rows of the tile hold the gate rows row0 .., the next `half_rows` the up rows
+// of the same output columns, so that the waves of the tile's left half end up with gate values
+// and the waves of its right half with the matching up values.
 template <bool TRANSPOSED>
 __device__ __forceinline__ uint32_t load_offset(int i, int wave, int lane, int ld, int row0,
-                                                int rows_total, int k_left) {
+                                                int rows_total, int k_left, int gate_up_f = 0,
+                                                int half_rows = 0) {
   if (!TRANSPOSED) {
     const int row = 8 * wave + (lane >> 3) + 32 * i;
     int chunk = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
     int r = row0 + row;
+    if (gate_up_f > 0) r = row < half_rows ? row0 + row : row0 + (row - half_rows) + gate_up_f;
     r = r < rows_total ? r : rows_total - 1;
     chunk = chunk + 8 <= k_left ? chunk : k_left - 8;
     return (uint32_t)(r * ld + chunk);
@@ -191,12 +197,16 @@ struct Count { static constexpr int value = N; };
 // WN: 16-column MFMA tiles per wave along N (5..8): the workgroup's tile is 256 x 32 * WN.  Narrower
 // tiles let the host avoid a mostly empty last round of workgroups or a mostly padded last tile
 // column; a K-major B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
-template <bool A_T, bool B_T, int WN>
+// EPI: the fused epilogue compiled into this instance (KR_GEMM_EPI_*).  A template parameter, not
+// a run-time switch: the plain instances carry none of the extra code or registers.
+template <bool A_T, bool B_T, int WN, int EPI>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
                                                         bf16* __restrict__ C, int ldc, int M,
                                                         int N, int K, int accumulate, int k_per,
-                                                        int splits, float* __restrict__ partial) {
+                                                        int splits, float* __restrict__ partial,
+                                                        const bf16* __restrict__ aux, int ld_aux,
+                                                        bf16* __restrict__ out2, int ld_out2) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -205,7 +215,15 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // transposed tile every load spans all 256 columns
   constexpr int NB_LOADS = B_T ? 8 : WN;
   const int wm = wave >> 1, wn = wave & 1;  // wave tile: rows wm*128.., columns wn*16*WN..
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_ - 1) / BN_;
+  // fused epilogues: ADD: C = bf16(bf16(A.B) + aux), aux [M,N] with row stride ld_aux.
+  // SWIGLU: C = x [M, N = 2F] and out2 = silu(x[:, :F]) * x[:, F:] [M, F]; a tile then covers
+  // 16 * WN columns of out2: its left half (the waves with wn = 0) computes their gate columns,
+  // its right half (wn = 1) the matching up columns of x, and the two meet in the epilogue.
+  static_assert(EPI == KR_GEMM_EPI_NONE || (!A_T && !B_T), "fused epilogues: K-major layout only");
+  constexpr bool epi_add = EPI == KR_GEMM_EPI_ADD;
+  constexpr bool swiglu = EPI == KR_GEMM_EPI_SWIGLU;
+  const int gate_up_f = swiglu ? N / 2 : 0;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = swiglu ? N / BN_ : (N + BN_ - 1) / BN_;
   const int ntiles = tiles_m * tiles_n;
   const bool split_k = partial != nullptr;
   const uint32_t smem_b = lds_addr(smem);
@@ -220,7 +238,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     int tile_m, tile_n;
     remap_block(v - split * ntiles, ntiles, tiles_m, tiles_n, tile_m, tile_n);
     m0 = tile_m * BM;
-    n0 = tile_n * BN_;
+    n0 = swiglu ? tile_n * (16 * WN) : tile_n * BN_;
     if (split_k) {
       // split-K: contraction range [split*k_per, split*k_per + kc), fp32 partial tile out
       // (k_per is a multiple of 64)
@@ -258,7 +276,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       la[i] = 2u * load_offset<A_T>(i, wave, l2, lda, m0, M, k_left);
-      lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left);
+      lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left, gate_up_f, 16 * WN);
     }
   };
   // the first `count` loads of a tile (8 for A, NB_LOADS for B)
@@ -500,13 +518,32 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       // 16-byte chunk rch = eight consecutive columns, 16 lanes per row
       const bool narrow = !to_partial && !add_old;
       const int rch = le & 15;
-      const bool ncols_in = 8 * rch < 16 * WN && n_wave + 8 * rch < N;
+      // first column the wave stores to: n_wave, or with SwiGLU column out_n0 of the gate half
+      // (wn = 0) or of the up half (wn = 1) of x
+      const int n_store = swiglu ? out_n0 + (wn ? gate_up_f : 0) : n_wave;
+      const int ncol = 8 * rch;
+      const bool ncols_in = 8 * rch < 16 * WN && (swiglu || n_wave + 8 * rch < N);
       uint32_t nlo[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) nlo[q] = (uint32_t)((4 * q + quad) * ldc + 8 * rch);
+      for (int q = 0; q < 4; ++q) nlo[q] = (uint32_t)((4 * q + quad) * ldc + ncol);
+      // fused residual: the values to add to a 16-row block are requested one block ahead
+      bf16x8 resv[epi_add ? 2 : 1][epi_add ? 4 : 1];
+      auto fetch_res = [&](int mt) {
+        const bf16* const rb = aux + ((int64_t)(m_wave + mt * 16) * ld_aux + n_wave + 8 * rch);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rr = 4 * q + quad;
+          const bool in = ncols_in && (rows_in || m_wave + mt * 16 + rr < M);
+          resv[mt & 1][q] = in ? ldg8(rb + (int64_t)rr * ld_aux) : zero8();
+        }
+      };
+      if constexpr (epi_add) fetch_res(0);
 #pragma unroll
       for (int mt = 0; mt < WT; ++mt) {
         if (add_old && mt + 1 < WT) fetch_old(mt + 1);
+        if constexpr (epi_add) {
+          if (mt + 1 < WT) fetch_res(mt + 1);
+        }
         f32x4 vals[WN];  // the only place the accumulators are read
 #pragma unroll
         for (int nt = 0; nt < WN; ++nt) {
@@ -514,7 +551,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
           asm volatile("" : "+v"(vals[nt]));  // read here, not once in each branch below
           acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + n_wave;
+        const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + (narrow ? n_store : n_wave);
         if (narrow) {
           const uint32_t buf = stage + (uint32_t)(mt & 1) * 4096u;
 #pragma unroll
@@ -524,12 +561,36 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
             for (int e = 0; e < 4; ++e) o[e] = (bf16)vals[nt][e];
             *(KR_LDS bf16x4*)(buf + row16 * 256 + (((2 * nt + (quad >> 1)) ^ row16) << 4) + (quad & 1) * 8) = o;
           }
-          wave_sync();
+          if constexpr (swiglu) __syncthreads(); else wave_sync();  // SwiGLU reads the neighbour wave's block too
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const int rr = 4 * q + quad;
-            const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
-            if (ncols_in && (rows_in || m_wave + mt * 16 + rr < M)) stg8(C + blk + nlo[q], v);
+            bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
+            const bool in = ncols_in && (rows_in || m_wave + mt * 16 + rr < M);
+            if constexpr (epi_add) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] = (bf16)((float)resv[mt & 1][q][e] + (float)v[e]);
+            }
+            if (in) stg8(C + blk + nlo[q], v);
+          }
+          if constexpr (swiglu) {
+            // the wave beside this one (same rows, other half of the tile) has staged the other
+            // operand of the activation for the same 16 rows: this wave takes rows 4 q + quad
+            // for q = 2 wn, 2 wn + 1 of the block, reads the gate chunk from the left wave's
+            // buffer and the up chunk from the right wave's, and stores out2
+            const uint32_t gbuf = r4 + (uint32_t)(2 * wm) * 8192u + (uint32_t)(mt & 1) * 4096u;
+            const uint32_t ubuf = gbuf + 8192u;
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+              const int rr = 4 * (2 * wn + qq) + quad;
+              const bf16x8 g = *(KR_LDS const bf16x8*)(gbuf + rr * 256 + ((rch ^ rr) << 4));
+              const bf16x8 u = *(KR_LDS const bf16x8*)(ubuf + rr * 256 + ((rch ^ rr) << 4));
+              bf16x8 y;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) y[e] = (bf16)kr_swiglu_f((float)g[e], (float)u[e]);
+              if (ncols_in && (rows_in || m_wave + mt * 16 + rr < M))
+                stg8(out2 + (int64_t)(m_wave + mt * 16 + rr) * ld_out2 + out_n0 + 8 * rch, y);
+            }
           }
         } else {
 #pragma unroll
@@ -650,23 +711,51 @@ inline int choose_wn(int M, int N, int num_cus) {
   return best;
 }
 
-template <bool A_T, bool B_T, int WN>
+struct Fused {
+  int epi = 0;              // KR_GEMM_EPI_*
+  const bf16* aux = nullptr;
+  int64_t ld_aux = 0;
+  bf16* out2 = nullptr;
+  int64_t ld_out2 = 0;
+  int max_cus = 0;          // > 0: use at most this many compute units
+};
+
+// Tile width for a projection with the SwiGLU epilogue: the tiles have to divide the 2F output
+// columns exactly (no partly filled tile column), otherwise as choose_wn.  0: no width fits.
+inline int swiglu_wn(int M, int N, int num_cus) {
+  const int tiles_m = (M + BM - 1) / BM;
+  int best = 0;
+  long best_cost = 0;
+  for (int wn = 8; wn >= 5; --wn) {
+    if (N % (32 * wn)) continue;
+    const int tiles = tiles_m * (N / (32 * wn));
+    const long cost = (long)((tiles + num_cus - 1) / num_cus) * (wn + 1);
+    if (best == 0 || cost < best_cost) {
+      best = wn;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+template <bool A_T, bool B_T, int WN, int EPI = KR_GEMM_EPI_NONE>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
-           hipStream_t stream, int num_cus) {
+           hipStream_t stream, int num_cus, const Fused& fu) {
   constexpr size_t lds_bytes = NSLOTS * TILE * sizeof(bf16);
   // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
   static const hipError_t attr_status =
-      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN>,
+      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN, EPI>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (attr_status != hipSuccess) return KR_ELAUNCH;
+  if (fu.max_cus > 0 && fu.max_cus < num_cus) num_cus = fu.max_cus;
   const int tiles = ((M + BM - 1) / BM) * ((N + 32 * WN - 1) / (32 * WN));
   // the latency-optimal count, capped by what the caller's workspace holds (a caller that wants
   // fewer splits says so by passing the smaller workspace kr_gemm_workspace_bytes_shared sizes)
   int splits = WN == 8 ? choose_splits(M, N, K, 1.f) : 1;
   const size_t one = (size_t)M * N * sizeof(float);
-  if (workspace == nullptr) {
-    splits = 1;
+  if (workspace == nullptr || EPI != KR_GEMM_EPI_NONE) {
+    splits = 1;  // a fused epilogue works on finished sums
   } else if ((size_t)splits * one > workspace_bytes) {
     splits = (int)(workspace_bytes / one);
   }
@@ -685,16 +774,19 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   };
   if (splits == 1) {
     const int grid = grid_for(tiles);
-    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
-                       (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr);
+    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, EPI>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
+                       (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr,
+                       fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2);
     return kr_launch_status();
   }
   int k_per = (K + splits - 1) / splits;
   k_per = (k_per + BK - 1) / BK * BK;
   splits = (K + k_per - 1) / k_per;
   const int items = tiles * splits;
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN>), dim3(grid_for(items)), dim3(NTHREADS),
-                     lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace);
+  if constexpr (EPI != KR_GEMM_EPI_NONE) return KR_EINVAL;  // (not reached: a fused launch never splits)
+  hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE>), dim3(grid_for(items)), dim3(NTHREADS),
+                     lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
+                     (const bf16*)nullptr, 0, (bf16*)nullptr, 0);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream,
@@ -720,9 +812,10 @@ extern "C" size_t kr_gemm_workspace_bytes_shared(int layout, int M, int N, int K
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
-extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int64_t lda,
-                            const void* B, int64_t ldb, void* C, int64_t ldc, int accumulate,
-                            void* workspace, size_t workspace_bytes, void* stream) {
+namespace {
+int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, const void* B,
+                  int64_t ldb, void* C, int64_t ldc, int accumulate, void* workspace,
+                  size_t workspace_bytes, void* stream, const Fused& fu) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return KR_EINVAL;
   if (!kr_aligned16(A) || !kr_aligned16(B) || !kr_aligned16(C)) return KR_EINVAL;
   if (workspace && !kr_aligned16(workspace)) return KR_EINVAL;
@@ -733,6 +826,22 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
   if (a_rows * lda >= (int64_t)1 << 31 || b_rows * ldb >= (int64_t)1 << 31 || ldc >= (int64_t)1 << 26 ||
       N >= 1 << 26)
     return KR_EUNSUPPORTED;
+  if (fu.max_cus < 0) return KR_EINVAL;
+  if (fu.epi != KR_GEMM_EPI_NONE) {
+    if (accumulate) return KR_EINVAL;
+    if (layout != KR_GEMM_TN) return KR_EUNSUPPORTED;  // fused epilogues are built for the forward layout
+    if (fu.epi == KR_GEMM_EPI_ADD) {
+      if (!fu.aux || !kr_aligned16(fu.aux) || fu.ld_aux < N) return KR_EINVAL;
+      if (fu.ld_aux % 8 || fu.ld_aux >= (int64_t)1 << 26) return KR_EUNSUPPORTED;
+    } else if (fu.epi == KR_GEMM_EPI_SWIGLU) {
+      if (!fu.out2 || !kr_aligned16(fu.out2) || fu.ld_out2 < N / 2) return KR_EINVAL;
+      // the tiles must divide the output exactly: F a multiple of 80, 96, 112 or 128
+      if (N % 2 || swiglu_wn(M, N, 256) == 0 || fu.ld_out2 % 8 || fu.ld_out2 >= (int64_t)1 << 26)
+        return KR_EUNSUPPORTED;
+    } else {
+      return KR_EINVAL;
+    }
+  }
   const bf16* a = (const bf16*)A;
   const bf16* b = (const bf16*)B;
   bf16* c = (bf16*)C;
@@ -745,13 +854,34 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
       n = 256;
     return n;
   }();
-  const int wn = choose_wn(M, N, num_cus);
+  const int cus = fu.max_cus > 0 && fu.max_cus < num_cus ? fu.max_cus : num_cus;
+  const int wn = fu.epi == KR_GEMM_EPI_SWIGLU ? swiglu_wn(M, N, cus) : choose_wn(M, N, cus);
+  if (fu.epi != KR_GEMM_EPI_NONE) {
+    if (lda < K || ldb < K || ldc < N) return KR_EINVAL;
+#define KR_GEMM_FUSED(W, E) \
+  return launch<false, false, W, E>(a, lda, b, ldb, c, ldc, M, N, K, 0, ws, workspace_bytes, st, num_cus, fu)
+    if (fu.epi == KR_GEMM_EPI_SWIGLU) {
+      switch (wn) {
+        case 5: KR_GEMM_FUSED(5, KR_GEMM_EPI_SWIGLU);
+        case 6: KR_GEMM_FUSED(6, KR_GEMM_EPI_SWIGLU);
+        case 7: KR_GEMM_FUSED(7, KR_GEMM_EPI_SWIGLU);
+        default: KR_GEMM_FUSED(8, KR_GEMM_EPI_SWIGLU);
+      }
+    }
+    switch (wn) {
+      case 5: KR_GEMM_FUSED(5, KR_GEMM_EPI_ADD);
+      case 6: KR_GEMM_FUSED(6, KR_GEMM_EPI_ADD);
+      case 7: KR_GEMM_FUSED(7, KR_GEMM_EPI_ADD);
+      default: KR_GEMM_FUSED(8, KR_GEMM_EPI_ADD);
+    }
+#undef KR_GEMM_FUSED
+  }
 #define KR_GEMM_LAUNCH(AT, BT)                                                                           \
   switch (wn) {                                                                                          \
-    case 5: return launch<AT, BT, 5>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
-    case 6: return launch<AT, BT, 6>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
-    case 7: return launch<AT, BT, 7>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
-    default: return launch<AT, BT, 8>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus); \
+    case 5: return launch<AT, BT, 5>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
+    case 6: return launch<AT, BT, 6>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
+    case 7: return launch<AT, BT, 7>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
+    default: return launch<AT, BT, 8>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
   }
   switch (layout) {
     case KR_GEMM_TN:  // A [M,K], B [N,K]
@@ -767,4 +897,28 @@ extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int6
       return KR_EINVAL;
   }
 #undef KR_GEMM_LAUNCH
+}
+}  // namespace
+
+extern "C" int kr_gemm_bf16(int layout, int M, int N, int K, const void* A, int64_t lda,
+                            const void* B, int64_t ldb, void* C, int64_t ldc, int accumulate,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  return gemm_dispatch(layout, M, N, K, A, lda, B, ldb, C, ldc, accumulate, workspace, workspace_bytes,
+                       stream, Fused{});
+}
+
+extern "C" int kr_gemm_bf16_fused(int layout, int M, int N, int K, const void* A, int64_t lda,
+                                  const void* B, int64_t ldb, void* C, int64_t ldc, int accumulate,
+                                  int epilogue, const void* aux, int64_t ld_aux, void* out2,
+                                  int64_t ld_out2, int max_cus, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  Fused fu;
+  fu.epi = epilogue;
+  fu.aux = (const bf16*)aux;
+  fu.ld_aux = ld_aux;
+  fu.out2 = (bf16*)out2;
+  fu.ld_out2 = ld_out2;
+  fu.max_cus = max_cus;
+  return gemm_dispatch(layout, M, N, K, A, lda, B, ldb, C, ldc, accumulate, workspace, workspace_bytes,
+                       stream, fu);
 }

@@ -83,3 +83,19 @@ def test_strides_the_kernels_cannot_index_are_refused():
     rope = lambda st: [16, 16, 16, 4, 1, 2, 128] + st + [0, 1, 1, None]
     assert lib.kr_rope(*rope([-256, 256, 128, 256, 256, 128])) == -2
     assert lib.kr_rope(*rope([256, 256, 128, 256, 0, 128])) == -2
+
+
+def test_fused_gemm_argument_checks():
+    lib = hip.load_library()
+    base = [0, 256, 256, 64, 16, 64, 16, 64, 16, 256, 0]
+    call = lambda epi, aux, ld_aux, out2, ld_out2, cus=0, acc=0, layout=0, n=256: lib.kr_gemm_bf16_fused(
+        layout, 256, n, 64, 16, 64, 16, 64, 16, n, acc, epi, aux, ld_aux, out2, ld_out2, cus, None, 0, None)
+    assert call(1, None, 256, None, 0) == -1                 # residual epilogue without a residual
+    assert call(1, 16, 128, None, 0) == -1                   # residual row stride below N
+    assert call(1, 16, 256, None, 0, acc=1) == -1            # a fused epilogue cannot accumulate into C
+    assert call(2, None, 0, None, 0) == -1                   # SwiGLU without its second output
+    assert call(2, None, 0, 16, 128, layout=1) == -2         # fused epilogues are built for the forward layout
+    assert call(1, 16, 256, None, 0, layout=2) == -2
+    assert call(2, None, 0, 16, 136, n=272) == -2            # no tile width divides 2F = 272
+    assert call(7, None, 0, None, 0) == -1                   # unknown epilogue
+    assert call(0, None, 0, None, 0, cus=-3) == -1

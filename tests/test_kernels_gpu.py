@@ -307,3 +307,50 @@ def test_attention_special_cases(be):
         be.attn_fwd(rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), 1.0)  # s % 128 != 0
     with pytest.raises(RuntimeError, match="not supported"):
         be.attn_fwd(rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), 1.0)  # head_dim 64
+
+
+# ------------------------------------------------------------------ fused GEMM epilogues
+@pytest.mark.parametrize("m,n,k", [(512, 768, 512), (264, 520, 200), (4096, 4096, 1024), (1000, 3072, 640),
+                                   (16384, 640, 72)])
+def test_gemm_with_fused_residual_equals_gemm_then_add(be, m, n, k):
+    """C = bf16(bf16(A.B) + R) in the GEMM's epilogue: the same bits as the GEMM followed by the residual add,
+    also with a row-strided residual and a row-strided output (a nanobatch slice of the block's output).
+    (The unfused reference runs without split-K, as a fused launch always does: splitting the contraction
+    changes the order of the sum.)"""
+    x, w = rnd(m, k, seed=80), rnd(n, k, scale=0.05, seed=81)
+    res_wide = rnd(m, 2 * n, seed=82)
+    res = res_wide[:, n // 2: n // 2 + n] if (n // 2) % 8 == 0 else res_wide[:, :n]
+    want = be.add(res.contiguous(), be.linear_fwd(x, w, split_k=None))
+    got = be.linear_fwd(x, w, residual=res)
+    assert torch.equal(got, want)
+    whole = torch.zeros(m, 3 * n, device=DEV, dtype=torch.bfloat16)
+    be.linear_fwd(x, w, residual=res, out=whole[:, n:2 * n])
+    assert torch.equal(whole[:, n:2 * n], want) and not whole[:, :n].any() and not whole[:, 2 * n:].any()
+    assert rel(got, x.float() @ w.float().t() + res.float()) <= TOL
+    with pytest.raises(RuntimeError, match="not supported"):   # fused epilogues exist for the forward layout only
+        be.gemm(1, rnd(m, n, seed=83), w, m, k, n, residual=rnd(m, k, seed=84))
+
+
+@pytest.mark.parametrize("m,f,k", [(512, 128, 256), (264, 384, 200), (4096, 3584, 4096), (1000, 1024, 3072),
+                                   (16384, 320, 72), (8192, 672, 136), (304, 14336, 64)])
+def test_gemm_with_fused_swiglu_equals_gemm_then_swiglu(be, m, f, k):
+    """fc1 with the activation in its epilogue: x = A.W^T [m, 2f] and y = silu(x[:, :f]) * x[:, f:] from one
+    launch, the same bits as the GEMM followed by the SwiGLU kernel."""
+    a, w = rnd(m, k, seed=85), rnd(2 * f, k, scale=0.05, seed=86)
+    x_want = be.linear_fwd(a, w, split_k=None)
+    y_want = be.swiglu_fwd(x_want)
+    y = torch.empty(m, f, device=DEV, dtype=torch.bfloat16)
+    x = be.linear_fwd(a, w, swiglu_out=y)
+    assert torch.equal(x, x_want) and torch.equal(y, y_want)
+    assert rel(y, R.swiglu(a.float() @ w.float().t())) <= TOL
+    assert be.can_fuse_swiglu(2 * f)
+    with pytest.raises(RuntimeError, match="not supported"):   # no tile width divides 2f = 144: the caller keeps the two launches
+        be.linear_fwd(a[:, :k], rnd(2 * 72, k, seed=87), swiglu_out=torch.empty(m, 72, device=DEV, dtype=torch.bfloat16))
+
+
+def test_gemm_compute_unit_budget_changes_nothing_but_the_launch(be):
+    m, n, k = 4096, 3584, 1088
+    x, w = rnd(m, k, seed=88), rnd(n, k, scale=0.05, seed=89)
+    full = be.linear_fwd(x, w, split_k=None)
+    for cus in (1, 64, 200, 256, 1000):
+        assert torch.equal(be.linear_fwd(x, w, split_k=False, max_cus=cus), full)
