@@ -109,6 +109,15 @@ int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd, const v
                        const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
                        int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
 
+/* Weight gradient of one RMSNorm over several nanobatches of a microbatch, summed in fp32 and
+ * rounded once (the reference lets autograd add the per-nanobatch bf16 gradients,
+ * kareus/megatron/core/partitions/autograd_function.py:346-372): call kr_rmsnorm_bwd_add with
+ * dgamma == NULL for every nanobatch — it then only leaves its kr_rmsnorm_bwd_partial_rows(rows, cols)
+ * fp32 partial rows of `cols` columns at `workspace` — with the nanobatches' workspaces back to back in
+ * one buffer, then kr_rmsnorm_dgamma over all `nparts` rows of that buffer.                     */
+int kr_rmsnorm_bwd_partial_rows(int rows, int cols);
+int kr_rmsnorm_dgamma(const float* partial, int nparts, int cols, void* dgamma, void* stream);
+
 /* kr_rmsnorm_bwd_add without a workspace argument, for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  The fp32 partial rows of the weight gradient go to a 16 MiB array

@@ -18,8 +18,22 @@ class EagerBackend:
 
     # y = x . W^T, dx = dy . W, dW = dy^T . x   (reference call sites:
     # kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:571-582, 847-859, 898-909)
-    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
-        return x @ w.t()
+    def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True, out: Tensor = None,
+                   residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0) -> Tensor:
+        y = x @ w.t()
+        if residual is not None:       # rounded product first, then the add: as the two separate ops
+            y = residual + y
+        if swiglu_out is not None:
+            a, b = y.chunk(2, dim=-1)
+            swiglu_out.copy_((torch.nn.functional.silu(a.float()) * b.float()).to(y.dtype))
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+    @staticmethod
+    def can_fuse_swiglu(two_f: int) -> bool:
+        return two_f % 2 == 0
 
     def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
         return dy @ w
@@ -46,8 +60,15 @@ class EagerBackend:
 
     # dx = rs * (g - xhat * mean(g * xhat)), g = gamma * dy ; dgamma = sum_rows dy * xhat
     # (rmsnorm_bwd_kernels.cuh:95-128)
+    def rmsnorm_partial_rows(self, rows: int, cols: int) -> int:
+        return 1
+
+    def rmsnorm_dgamma(self, partials: Tensor, gamma: Tensor) -> Tensor:
+        return partials.sum(dim=0).to(gamma.dtype)
+
     def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor,
-                    residual_grad: Tensor = None, out: Tensor = None) -> Tuple[Tensor, Tensor]:
+                    residual_grad: Tensor = None, out: Tensor = None,
+                    partials_out: Tensor = None) -> Tuple[Tensor, Tensor]:
         xhat = x.float() * rstd[:, None]
         dyf = dy.float()
         g = dyf * gamma.float()
@@ -59,6 +80,9 @@ class EagerBackend:
         if out is not None:
             out.copy_(dx)
             dx = out
+        if partials_out is not None:
+            partials_out.copy_(dgamma.view(1, -1))
+            return dx, None
         return dx, dgamma.to(gamma.dtype)
 
     # y = t cos f + rotate_half(t) sin f, rotate_half([a, b]) = [-b, a]; trig in fp32

@@ -34,6 +34,8 @@ _SIGNATURES = {
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_rmsnorm_bwd_add": (_c_int, [_c_void_p] * 8 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
+    "kr_rmsnorm_bwd_partial_rows": (_c_int, [_c_int, _c_int]),
+    "kr_rmsnorm_dgamma": (_c_int, [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p]),
     "kr_rmsnorm_bwd_add_noalloc": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
     "kr_rope": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int] + [_c_i64] * 6
                 + [_c_int, _c_int, _c_int, _c_void_p]),
@@ -219,11 +221,25 @@ class HipBackend:
         self._check(rc, "kr_rmsnorm_fwd")
         return y, rstd
 
+    def rmsnorm_partial_rows(self, rows: int, cols: int) -> int:
+        """fp32 partial rows of the weight gradient one backward call over [rows, cols] leaves."""
+        return self.lib.kr_rmsnorm_bwd_partial_rows(rows, cols)
+
+    def rmsnorm_dgamma(self, partials: Tensor, gamma: Tensor) -> Tensor:
+        """Sum of the partial rows ([n, cols] fp32) of all nanobatches -> the weight gradient."""
+        dgamma = torch.empty_like(gamma)
+        self._check(self.lib.kr_rmsnorm_dgamma(partials.data_ptr(), partials.shape[0], partials.shape[1],
+                                               dgamma.data_ptr(), self._stream()), "kr_rmsnorm_dgamma")
+        return dgamma
+
     def rmsnorm_bwd(self, dy: Tensor, x: Tensor, rstd: Tensor, gamma: Tensor,
-                    residual_grad: Tensor = None, out: Tensor = None) -> Tuple[Tensor, Tensor]:
+                    residual_grad: Tensor = None, out: Tensor = None,
+                    partials_out: Tensor = None) -> Tuple[Tensor, Tensor]:
         """``residual_grad`` (same shape as ``x``): the gradient of the residual branch forked off
         in front of the norm is added to the norm's input gradient in the same pass.  ``out``: the
-        [rows, cols] tensor (possibly a row-strided slice) the input gradient is written into."""
+        [rows, cols] tensor (possibly a row-strided slice) the input gradient is written into.
+        ``partials_out`` ([rmsnorm_partial_rows, cols] fp32, contiguous): the weight gradient is
+        left there as partial rows for ``rmsnorm_dgamma`` and None is returned in its place."""
         self._dev(dy, x, rstd, gamma)
         self._bf16(dy, x, gamma)
         x, dy = self._rows(x), self._rows(dy)
@@ -244,10 +260,17 @@ class HipBackend:
                 raise RuntimeError("rmsnorm_bwd: residual_grad must have the shape of x")
             residual_grad = self._rows(residual_grad)
             res_ptr, res_ld = residual_grad.data_ptr(), residual_grad.stride(0)
-        dgamma = torch.empty_like(gamma)
-        ws = self._workspace(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), x.device)
+        if partials_out is not None:
+            if (partials_out.dtype != torch.float32 or not partials_out.is_contiguous()
+                    or tuple(partials_out.shape) != (self.rmsnorm_partial_rows(rows, cols), cols)):
+                raise RuntimeError("rmsnorm_bwd: partials_out must be fp32 [partial rows, cols]")
+            dgamma, dg_ptr, ws = None, None, partials_out
+        else:
+            dgamma = torch.empty_like(gamma)
+            dg_ptr = dgamma.data_ptr()
+            ws = self._workspace(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), x.device)
         rc = self.lib.kr_rmsnorm_bwd_add(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-                                         res_ptr, dx.data_ptr(), dgamma.data_ptr(), ws.data_ptr(), rows, cols,
+                                         res_ptr, dx.data_ptr(), dg_ptr, ws.data_ptr(), rows, cols,
                                          dy.stride(0), x.stride(0), res_ld, dx.stride(0), self._stream())
         self._check(rc, "kr_rmsnorm_bwd_add")
         return dx, dgamma

@@ -333,7 +333,7 @@ namespace {
 int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const void* gamma,
                      const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
                      int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream) {
-  if (!dy || !x || !rstd || !gamma || !dx || !dgamma || !workspace || rows <= 0 || cols <= 0 ||
+  if (!dy || !x || !rstd || !gamma || !dx || !workspace || rows <= 0 || cols <= 0 ||
       dy_ld < cols || x_ld < cols || dx_ld < cols || (dres && dres_ld < cols))
     return KR_EINVAL;
   if (cols % 8 || dy_ld % 8 || x_ld % 8 || dx_ld % 8 || (dres && dres_ld % 8) || cols > 8192)
@@ -366,11 +366,26 @@ int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const voi
   }
 #undef KR_RMS_BWD
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+  if (dgamma == nullptr) return KR_OK;  // the caller sums the partial rows later (kr_rmsnorm_dgamma)
   hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 31) / 32), dim3(kDgammaThreads), 0,
                      (hipStream_t)stream, (const float*)workspace, (bf16*)dgamma, blocks, cols);
   return kr_launch_status();
 }
 }  // namespace
+
+extern "C" int kr_rmsnorm_bwd_partial_rows(int rows, int cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return bwd_blocks(rows, cols);
+}
+
+extern "C" int kr_rmsnorm_dgamma(const float* partial, int nparts, int cols, void* dgamma,
+                                 void* stream) {
+  if (!partial || !dgamma || nparts <= 0 || cols <= 0) return KR_EINVAL;
+  if (!kr_aligned16(partial)) return KR_EINVAL;
+  hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3((cols + 31) / 32), dim3(kDgammaThreads), 0,
+                     (hipStream_t)stream, partial, (bf16*)dgamma, nparts, cols);
+  return kr_launch_status();
+}
 
 extern "C" int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
                               void* dx, void* dgamma, void* workspace, int rows, int cols,

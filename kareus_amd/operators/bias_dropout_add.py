@@ -42,6 +42,12 @@ class BiasDropoutAddOp(BasicOperation, PartitionableOperator):
         ctx.has_bias = False
         # the engine may name the tensor the sum belongs in (a slice of the block's output)
         sink = ctx.__dict__.pop("out_sink", None)
+        if getattr(input_, "_kr_residual_added", False):
+            # the projection in front added the residual in its epilogue (and wrote into the
+            # sink if one was named): nothing is left to do here
+            if sink is not None and sink.data_ptr() != input_.data_ptr():
+                raise RuntimeError("BiasDropoutAddOp: fused residual result is not in the output sink")
+            return input_, [()]
         out = get_backend(self._backend_name).add(residual, input_, out=sink)
         return out, [()]
 

@@ -13,6 +13,8 @@ from ..partitions.tensor_graph import Channel, PartitionableOperator
 
 
 class BiasSwigluOp(BasicOperation, PartitionableOperator):
+    forward_is_swiglu = True   # a projection in front may compute this activation in its epilogue
+
     def __init__(self, has_bias: bool = False, fp8_input_store: bool = False, backend="hip") -> None:
         super().__init__()
         if has_bias:

@@ -65,16 +65,89 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         # then the contraction is not split, which costs the least CU-time (set by the block driver)
         self.split_k = True
 
-    def op_forward(self, ctx, input_, *, prev_op=None, next_op=None):
+    # -- what the forward may take along in its epilogue ------------------------------------------
+    # fuse_residual (set by the block driver on row-parallel layers of a one-GPU shard): the layer
+    # also reads the ``residual`` channel and, when the kernels can address the operands, adds it
+    # in the GEMM's epilogue; the result is tagged so that the BiasDropoutAddOp behind the
+    # all-reduce slot passes it on instead of adding again.  With more than one rank the sum over
+    # ranks has to come first, so the flag is only ever set for a world size of one.
+    fuse_residual = False
+    forward_accepts_out_sink = False
+
+    def get_input_channels(self) -> List[Channel]:
+        if self.fuse_residual:
+            return [Channel(0, "main"), Channel(1, "residual")]
+        return [Channel(0, "main")]
+
+    @property
+    def num_extra_inputs(self) -> int:  # type: ignore[override]
+        return 1 if self.fuse_residual else 0
+
+    def can_fuse_forward_with(self, next_operator) -> bool:
+        """The SwiGLU activation behind fc1 can be produced by the projection's epilogue."""
+        if not getattr(next_operator, "forward_is_swiglu", False) or not self.fuse_activation:
+            return False
+        check = getattr(get_backend(self._backend_name), "can_fuse_swiglu", None)
+        return check is not None and check(self.weight.shape[0])
+
+    fuse_activation = True
+
+    @staticmethod
+    def _as_matrix(t, cols):
+        """``t`` as a [rows, cols] matrix with one row stride and no copy, or None."""
+        if t is None or t.shape[-1] != cols:
+            return None
+        try:
+            m = t.view(-1, cols)
+        except RuntimeError:
+            return None
+        return m if m.stride(1) == 1 and m.stride(0) % 8 == 0 and m.stride(0) >= cols else None
+
+    def fuser_forward(self, basic_op_ctxs, input_, *, basic_op_extra_inputs, basic_op_prev_ops,
+                      basic_op_next_ops, basic_op_kwargs):
+        ctx = basic_op_ctxs[0]
         n, k = self.weight.shape
         if input_.shape[-1] != k:
             raise ValueError(f"linear with in_features={k} got input of shape {tuple(input_.shape)}")
+        be = get_backend(self._backend_name)
         x2d = self._rows(input_.reshape(-1, k))
-        y = get_backend(self._backend_name).linear_fwd(x2d, self.weight.detach(), split_k=self.split_k)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d)
             ctx.input_requires_grad = True
-        return y.view(*input_.shape[:-1], n)
+        w = self.weight.detach()
+        if len(basic_op_ctxs) == 2:
+            # [fc1, SwiGLU]: x = input . W^T and y = silu(x[:, :F]) * x[:, F:] from one launch
+            # (kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20 behind basic_linear.py:571-582)
+            act_ctx = basic_op_ctxs[1]
+            y = x2d.new_empty((x2d.shape[0], n // 2))
+            x = be.linear_fwd(x2d, w, split_k=self.split_k, swiglu_out=y)
+            if act_ctx.requires_grad:
+                act_ctx.save_for_backward(x)
+                act_ctx.ori_shape = (*input_.shape[:-1], n)
+            return y.view(*input_.shape[:-1], n // 2), [(), ()]
+        residual = basic_op_extra_inputs[0][0] if (self.fuse_residual and basic_op_extra_inputs) else None
+        sink = ctx.__dict__.pop("out_sink", None)
+        out_shape = (*input_.shape[:-1], n)
+        if residual is not None:
+            res2d = self._as_matrix(residual, n)
+            out2d = self._as_matrix(sink, n) if sink is not None else None
+            if res2d is not None and res2d.shape[0] == x2d.shape[0] and (sink is None or out2d is not None):
+                y = be.linear_fwd(x2d, w, split_k=self.split_k, residual=res2d, out=out2d)
+                y = sink if sink is not None else y.view(out_shape)
+                y._kr_residual_added = True
+                return y, [()]
+        y = be.linear_fwd(x2d, w, split_k=self.split_k)
+        return y.view(out_shape), [()]
+
+    def op_forward(self, ctx, input_, *, prev_op=None, next_op=None):
+        out, _ = self.fuser_forward([ctx], input_, basic_op_extra_inputs=[()], basic_op_prev_ops=[prev_op],
+                                    basic_op_next_ops=[next_op], basic_op_kwargs=[{}])
+        return out
+
+    def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):
+        dx, param_grads = self.op_backward(basic_op_ctxs[0], grad_output)
+        # the residual input passes the incoming gradient through (out = residual + x . W^T)
+        return dx, [param_grads], [(grad_output,)] if self.fuse_residual else [()]
 
     def op_backward(self, ctx, grad_output):
         (x2d,) = ctx.saved_tensors

@@ -8,6 +8,7 @@ import torch
 
 from ..backend import get_backend
 from ..partitions.op_context import BasicOperation
+from ..partitions.streams import stream_api
 from ..partitions.tensor_graph import PartitionableOperator
 
 
@@ -34,9 +35,45 @@ class RMSNorm(BasicOperation):
     def op_backward(self, ctx, grad_output):
         x2d, rstd = ctx.saved_tensors
         dy = grad_output.reshape(x2d.shape)
-        dx, dgamma = get_backend(self._backend_name).rmsnorm_bwd(dy, x2d, rstd, self.weight.detach())
+        dx, dgamma = self._backward(ctx, dy, x2d, rstd, None, None)
         return dx.view(grad_output.shape), (dgamma,)
 
+    def _backward(self, ctx, dy, x2d, rstd, residual_grad, out2d):
+        """Input gradient and weight gradient.  When the engine attached a ``wgrad_sink`` — one
+        dict shared by this norm's contexts of all ``n`` nanobatches of one backward pass — every
+        nanobatch leaves its fp32 partial rows of the weight gradient in one shared buffer and
+        reports ``None``; the last one to get here waits for the others' events, sums all rows
+        in fp32 and reports the gradient, rounded once (the reference lets autograd add the
+        per-nanobatch bf16 gradients, kareus/megatron/core/partitions/autograd_function.py:346-372)."""
+        be = get_backend(self._backend_name)
+        sink = getattr(ctx, "wgrad_sink", None)
+        n = sink.get("n", 0) if sink is not None else 0
+        if n < 2 or not self.weight.requires_grad:
+            return be.rmsnorm_bwd(dy, x2d, rstd, self.weight.detach(), residual_grad=residual_grad, out=out2d)
+        rows, cols = x2d.shape
+        per = be.rmsnorm_partial_rows(rows, cols)
+        buf = sink.get("buf")
+        if buf is None or buf.shape[0] != n * per:
+            buf = sink["buf"] = torch.empty((n * per, cols), dtype=torch.float32, device=x2d.device)
+            sink["done"], sink["events"] = 0, []
+        k = sink["done"]
+        dx, _ = be.rmsnorm_bwd(dy, x2d, rstd, self.weight.detach(), residual_grad=residual_grad, out=out2d,
+                               partials_out=buf[k * per:(k + 1) * per])
+        sink["done"] = k + 1
+        api = stream_api()
+        here = api.current_stream()
+        if here is not None and hasattr(buf, "record_stream") and buf.is_cuda:
+            buf.record_stream(here)   # the buffer is shared by the nanobatch streams
+        if sink["done"] < n:
+            if here is not None:
+                ev = api.new_event()
+                ev.record(here)
+                sink["events"].append(ev)
+            return dx, None
+        if here is not None:
+            for ev in sink["events"]:
+                here.wait_event(ev)
+        return dx, be.rmsnorm_dgamma(buf, self.weight.detach())
 
     # -- fused backward with the residual fork that precedes the norm in the layer ------------
     def can_fuse_backward_with(self, next_operator) -> bool:
@@ -59,8 +96,7 @@ class RMSNorm(BasicOperation):
                 out2d = sink.view(x2d.shape)   # a one-sequence slice is a row-strided matrix
             except RuntimeError:
                 out2d = None
-        dx, dgamma = get_backend(self._backend_name).rmsnorm_bwd(
-            dy, x2d, rstd, self.weight.detach(), residual_grad=grad_residual.reshape(x2d.shape), out=out2d)
+        dx, dgamma = self._backward(norm_ctx, dy, x2d, rstd, grad_residual.reshape(x2d.shape), out2d)
         if sink is not None:
             if out2d is None:
                 sink.copy_(dx.view(sink.shape))

@@ -108,6 +108,15 @@ def _last_compute_op(graph: TensorGraph, capability: str) -> Optional[int]:
     return None
 
 
+def _fused_producer_of_last(graph: TensorGraph) -> Optional[int]:
+    """op_id of the projection in front of the graph's final residual add if it may add the
+    residual in its own epilogue: it is then the op that writes the block's output."""
+    ops = graph.get_compute_ops()
+    if len(ops) >= 2 and getattr(ops[-2].operator, "fuse_residual", False):
+        return ops[-2].op_id
+    return None
+
+
 def _seed_forward(ctxs, hs, rotary, mask, seed: SeedConfig) -> None:
     for ctx, h in zip(ctxs, hs):
         ctx.tensor_store.set(seed.h_tid, h)
@@ -172,8 +181,11 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             last = _last_compute_op(fwd_graph, "forward_accepts_out_sink")
             sinks = _batch_slices(hs) if last is not None else None
             if sinks is not None:
+                producer = _fused_producer_of_last(fwd_graph)
                 for c, sink in zip(ctxs, sinks):
                     c.output_sinks[last] = sink
+                    if producer is not None:
+                        c.output_sinks[producer] = sink
 
         schedule = scheduler.current_schedule if scheduler is not None else None
         _fork(streams)
@@ -253,7 +265,7 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             sinks: Dict[int, dict] = {}
             for c in ctxs:
                 for op_id, op_ctx in c.op_contexts.items():
-                    op_ctx.wgrad_sink = sinks.setdefault(op_id, {})
+                    op_ctx.wgrad_sink = sinks.setdefault(op_id, {"n": n})
 
         if func_ctx.join_in_place:
             last = _last_compute_op(func_ctx.backward_tensor_graph, "backward_accepts_out_sink")

@@ -18,51 +18,81 @@ from .partition_base import PartitionBase, _current_stream
 
 @dataclass
 class ForwardPartition(PartitionBase):
+    # adjacent ops that offer a fused forward (fc1 + the SwiGLU activation behind it) run as one
+    # call; the numbers are those of the separate calls
+    fuse_forward_ops: bool = True
+
     def execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext) -> None:
         with self._on_stream(ctx), self._timed():
             self._execute(ctx, pre_ctx)
+
+    def _fusable_follower(self, idx: int, start: int):
+        """The op after ``idx`` when the two can run as one fused forward: the first op offers it
+        (``can_fuse_forward_with``), the second is a plain one-in/one-out op consuming the
+        first's only output, and the scheduled launch point does not fall between them."""
+        if not self.fuse_forward_ops or idx + 1 >= len(self.comp_ops) or start == idx + 1:
+            return None
+        op, nxt = self.comp_ops[idx], self.comp_ops[idx + 1]
+        offer = getattr(op.operator, "can_fuse_forward_with", None)
+        if offer is None or not offer(nxt.operator):
+            return None
+        outs, nxt_ins = op.get_output_tensor_ids(), nxt.get_input_tensor_ids()
+        if len(outs) != 1 or len(nxt_ins) != 1 or nxt_ins[0] != outs[0] or len(nxt.get_output_tensor_ids()) != 1:
+            return None
+        return nxt
 
     def _execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext) -> None:
         start, _end, sm_num, block_size = self._setup_comm()
         store = ctx.tensor_store
         comm_out, comm_extra = None, []
 
-        for idx, op in enumerate(self.comp_ops):
-            op_ctx = ctx.create_op_context(op.op_id)
+        idx, num_ops = 0, len(self.comp_ops)
+        while idx < num_ops:
+            op = self.comp_ops[idx]
             in_ids = op.get_input_tensor_ids()
             x = store.get(in_ids[0])
             extras = [tuple(store.get(t) for t in in_ids[1:])] if len(in_ids) > 1 else []
+            follower = self._fusable_follower(idx, start)
+            group = [op] if follower is None else [op, follower]
 
             needs_grad = self.is_grad_enabled and (
                 any(store.needs_grad(t) for t in in_ids)
-                or any(p.requires_grad for p in op.operator.parameters())
+                or any(p.requires_grad for member in group for p in member.operator.parameters())
             )
-            op_ctx.requires_grad = needs_grad
-            if ctx.output_sinks and op.op_id in ctx.output_sinks:
-                op_ctx.out_sink = ctx.output_sinks.pop(op.op_id)
+            group_ctxs = []
+            for member in group:
+                op_ctx = ctx.create_op_context(member.op_id)
+                op_ctx.requires_grad = needs_grad
+                if ctx.output_sinks and member.op_id in ctx.output_sinks:
+                    op_ctx.out_sink = ctx.output_sinks.pop(member.op_id)
+                group_ctxs.append(op_ctx)
+            last = idx + len(group) - 1
 
             if start == idx:
                 comm_out, comm_extra = self._launch_comm(pre_ctx, sm_num, block_size)
 
+            k = len(group)
             x, extra_out = op.operator.fuser_forward(
-                [op_ctx],
+                group_ctxs,
                 x,
-                basic_op_extra_inputs=extras,
-                basic_op_prev_ops=[None],
-                basic_op_next_ops=[None],
-                basic_op_kwargs=[{}],
+                basic_op_extra_inputs=extras if k == 1 else [extras[0] if extras else (), ()],
+                basic_op_prev_ops=[None] * k,
+                basic_op_next_ops=[None] * k,
+                basic_op_kwargs=[{} for _ in range(k)],
             )
 
-            self._op_done(idx)
-            if idx == start - 1:
+            for j in range(k):
+                self._op_done(idx + j)
+            if last == start - 1:
                 self.comm_op.event_record(_current_stream())
 
-            out_ids = op.get_output_tensor_ids()
+            out_ids = group[-1].get_output_tensor_ids()
             store.set(out_ids[0], x, needs_grad)
-            for k, tid in enumerate(out_ids[1:]):
-                extra = extra_out[0][k] if extra_out and extra_out[0] else None
+            for j, tid in enumerate(out_ids[1:]):
+                extra = extra_out[-1][j] if extra_out and extra_out[-1] else None
                 if extra is not None:
                     store.set(tid, extra, needs_grad)
+            idx = last + 1
 
         if self.comm_op is not None:
             if start == -1:

@@ -143,6 +143,64 @@ def test_fused_norm_and_fork_backward_changes_nothing(nnb, monkeypatch):
     _check(model, x, go, ref)
 
 
+@pytest.mark.parametrize("nnb", [1, 2, 4])
+@pytest.mark.parametrize("recompute", [False, True])
+def test_forward_epilogue_fusions_change_nothing(nnb, recompute, monkeypatch):
+    """fc1 runs the SwiGLU activation behind it as part of its own call, the out-projection and fc2 add the
+    residual themselves and the BiasDropoutAddOp behind the all-reduce slot passes the sum on; a schedule
+    whose launch point falls between fc1 and the activation switches that pair off.  Same numbers either way."""
+    from kareus_amd.operators.bias_dropout_add import BiasDropoutAddOp
+    from kareus_amd.operators.linear import PartitionableLinear
+
+    x, go, ref = _oracle(layers=2, s=64, b=4)
+    calls = {"pairs": 0, "passed_on": 0}
+    real_linear, real_bda = PartitionableLinear.fuser_forward, BiasDropoutAddOp.fuser_forward
+
+    def spy_linear(self, ctxs, x_, **kw):
+        calls["pairs"] += len(ctxs) == 2
+        return real_linear(self, ctxs, x_, **kw)
+
+    def spy_bda(self, ctxs, x_, **kw):
+        out = real_bda(self, ctxs, x_, **kw)
+        calls["passed_on"] += out[0] is x_
+        return out
+
+    monkeypatch.setattr(PartitionableLinear, "fuser_forward", spy_linear)
+    monkeypatch.setattr(BiasDropoutAddOp, "fuser_forward", spy_bda)
+    results = {}
+    for fuse in (True, False):
+        cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager",
+                          checkpoint_activations=recompute, fuse_forward_epilogues=fuse)
+        model = LayerStack(cfg, seed=1234)
+        calls.update(pairs=0, passed_on=0)
+        y, dx = _run(model, x, go)
+        results[fuse] = (y, dx, [p.grad.clone() for p in model.parameters()])
+        passes = 2 if recompute else 1                       # the recompute runs the forward again
+        assert calls["pairs"] == (2 * nnb * passes if fuse else 0)          # one fc1 per layer and nanobatch
+        # two residual adds per layer; the last one of a nanobatch writes into the block's output, and a
+        # nanobatch of more than one sequence is a slice of it that no single row stride addresses: that add
+        # stays a separate call (the recompute pass has no output to write)
+        kept = nnb if (nnb > 1 and x.shape[1] // nnb > 1) else 0
+        assert calls["passed_on"] == (4 * nnb * passes - kept if fuse else 0)
+    assert torch.allclose(results[True][0], results[False][0], atol=1e-6)
+    assert torch.allclose(results[True][1], results[False][1], atol=1e-6)
+    assert all(torch.allclose(a, c, atol=1e-5) for a, c in zip(results[True][2], results[False][2]))
+    for p in model.parameters():
+        p.grad = None
+    cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager",
+                      checkpoint_activations=recompute)
+    _check(LayerStack(cfg, seed=1234), x, go, ref)
+    # a launch point between fc1 (linear_0 of the MLP partition) and the activation: the pair runs as two calls
+    cfg.kareus_scheduler = None
+    model = LayerStack(cfg, seed=1234)
+    for part in model.forward_partitions:
+        if part.partition_key == "fwd_mlp":
+            part._schedule_config = (("activation_0", "none"), (16, 1024))
+    calls.update(pairs=0, passed_on=0)
+    _check(model, x, go, ref)
+    assert calls["pairs"] == (0 if nnb > 1 else 2 * (2 if recompute else 1))   # (one nanobatch: no launch points)
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")

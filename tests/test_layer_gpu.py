@@ -109,6 +109,33 @@ def test_streams_recompute_and_schedule_do_not_change_results(fixtures_dir):
     assert torch.equal(r1[0], r2[0]) and torch.equal(r1[1], r2[1]) and torch.equal(r1[2][1][4], r2[2][1][4])
 
 
+def test_fused_epilogues_do_not_change_results():
+    """SwiGLU in fc1's epilogue, the residual adds in the epilogues of the out-projection and fc2, and the
+    RMSNorm weight gradient summed over nanobatches in fp32: outputs, input gradients and the linear layers'
+    weight gradients are bit-identical to the engine running every operator as its own kernel (the GEMMs never
+    split the contraction here: a fused epilogue cannot, and splitting changes the order of the sum); only the
+    norm weights' gradients differ, by the one rounding the fp32 sum saves."""
+    dims = R.LayerDims(1024, 8, 2, 128, 896)
+    x, go = _inputs(256, 4, dims.hidden)
+    runs = {}
+    for fuse in (True, False):
+        for nnb in (1, 2, 4):
+            model = _build(dims, 2, nnb, fuse_forward_epilogues=fuse)
+            for layer in model.layers:
+                for op in (layer.linear_qkv, layer.linear_proj, layer.linear_fc1, layer.linear_fc2):
+                    op.split_k = None
+            runs[fuse, nnb] = _run(model, x, go)
+    for nnb in (1, 2, 4):
+        a, b = runs[True, nnb], runs[False, nnb]
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        for la, lb in zip(a[2], b[2]):
+            for (attr, _), ga, gb in zip(PARAMS, la, lb):
+                if "layernorm" in attr:
+                    assert _rel(ga, gb)[0] <= 1e-2
+                else:
+                    assert torch.equal(ga, gb)
+
+
 def test_full_size_properties_config4():
     """Benchmark configuration 4 at full size (h4096, 8q/2kv, ffn 3584, MBS 4 x seq 4096): too large for the CPU
     oracle in test time, so check properties that hold at any size."""
