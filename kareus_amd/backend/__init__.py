@@ -29,3 +29,30 @@ def get_backend(name: str = "hip"):
 
             _CACHE[name] = EagerBackend()
     return _CACHE[name]
+
+
+# ---- compute-unit budget of the launches of the current thread ---------------------------------
+# A schedule gives every partition a resource shape (kareus/megatron/core/partitions/
+# partition_base.py:117-128: ``sm_num``, the compute units the work overlapping the partition is to
+# get).  While a partition runs under such a shape the engine reserves that many units: kernels
+# that would otherwise fill the device (the GEMMs, one persistent workgroup per unit) launch on the
+# rest.  Thread-local because forward and backward run on different host threads.
+import contextlib as _contextlib
+import threading as _threading
+
+_budget = _threading.local()
+
+
+def reserved_compute_units() -> int:
+    """Compute units the current partition leaves to the kernels of other nanobatch streams."""
+    return getattr(_budget, "reserved", 0)
+
+
+@_contextlib.contextmanager
+def reserve_compute_units(count):
+    old = getattr(_budget, "reserved", 0)
+    _budget.reserved = max(int(count or 0), 0)
+    try:
+        yield
+    finally:
+        _budget.reserved = old

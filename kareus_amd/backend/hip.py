@@ -14,6 +14,8 @@ from typing import Tuple
 import torch
 from torch import Tensor
 
+from . import reserved_compute_units
+
 _LIB_NAME = "libkareus_hip.so"
 _c_void_p, _c_int, _c_i64, _c_float, _c_size_t = (
     ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t,
@@ -81,6 +83,7 @@ class HipBackend:
         self.lib = load_library()
         self._gemm_ws_bytes: dict = {}  # (layout, m, n, k, split_k) -> workspace bytes
         self._ws_cache: dict = {}       # (stream, device) -> reusable workspace buffer
+        self._cu_count: dict = {}       # device index -> compute units
 
     # -- plumbing -------------------------------------------------------------------
     # the raw handle of the current stream without building a torch.cuda.Stream object: this is
@@ -118,6 +121,12 @@ class HipBackend:
                 raise RuntimeError(f"the hip backend computes in bf16, got {t.dtype}")
 
     # -- GEMM -------------------------------------------------------------------------
+    def _num_cus(self, device) -> int:
+        n = self._cu_count.get(device.index)
+        if n is None:
+            n = self._cu_count[device.index] = torch.cuda.get_device_properties(device).multi_processor_count
+        return n
+
     def _workspace(self, nbytes: int, device) -> Tensor:
         """A workspace of at least ``nbytes`` for the current stream.  One buffer per (stream, size
         class) is kept and reused: kernels on one stream run in order, so consecutive launches may
@@ -170,6 +179,10 @@ class HipBackend:
                 self._gemm_ws_bytes[key] = ws_bytes
             if ws_bytes:
                 ws_ptr = self._workspace(ws_bytes, a.device).data_ptr()
+        if max_cus == 0:
+            reserved = reserved_compute_units()
+            if reserved:
+                max_cus = max(self._num_cus(a.device) - reserved, 8)
         if epi == 0 and max_cus == 0:
             rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
                                        out.data_ptr(), out.stride(0), int(accumulate), ws_ptr, ws_bytes,

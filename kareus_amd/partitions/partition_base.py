@@ -21,6 +21,8 @@ import contextlib
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional, Tuple, Union
 
+from ..backend import reserve_compute_units
+from ..utils.debug import roctx_enabled, roctx_range
 from .context_manager import NanoBatchContext
 from .streams import stream_api
 from .tensor_graph import CommunicationOp, ComputeOp
@@ -111,6 +113,8 @@ class PartitionBase:
     # With a single nanobatch there is no other nanobatch to overlap with: the
     # hand-over runs after this partition's own compute whatever the schedule says.
     force_no_overlap: bool = False
+    # the schedule's resource shape sets a compute-unit budget for this partition's GEMM launches
+    apply_resource_shape: bool = True
 
     def __post_init__(self) -> None:
         self._overlap_slots: Dict[str, int] = _build_overlap_slots(self.comp_ops)
@@ -213,10 +217,23 @@ class PartitionBase:
             t.op_done(self, idx)
 
     # -- stream scoping -----------------------------------------------------------
-    @staticmethod
-    def _on_stream(ctx: NanoBatchContext):
-        """Context manager making the nanobatch's own stream current (if it has one)."""
-        return stream_api().stream(ctx.stream)
+    def _on_stream(self, ctx: NanoBatchContext):
+        """Context manager making the nanobatch's own stream current (if it has one); with a
+        schedule it also reserves the compute units the partition's resource shape names for
+        the kernels of the other nanobatch streams, and the whole is a named profiler range."""
+        on_stream = stream_api().stream(ctx.stream)
+        sm_num = 0
+        if ctx.stream is not None and self.apply_resource_shape and self._schedule_config and self.comm_op is not None:
+            sm_num = self._schedule_config[1][0] or 0
+        if not sm_num and not roctx_enabled():
+            return on_stream
+        scope = contextlib.ExitStack()
+        scope.enter_context(on_stream)
+        if sm_num:
+            scope.enter_context(reserve_compute_units(sm_num))
+        if roctx_enabled():
+            scope.enter_context(roctx_range(f"{self.partition_key or 'trail'} nb{self.nano_batch_idx}"))
+        return scope
 
     def execute(self, ctx: NanoBatchContext, pre_ctx: NanoBatchContext):
         raise NotImplementedError

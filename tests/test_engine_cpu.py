@@ -374,3 +374,44 @@ def test_stream_protocol_replay():
     for nnb in (1, 4):
         rec = _replay(("norm_0", "none"), nnb=nnb, layers=2)
         assert rec.violations == [] and len(rec.spans) == 2 * nnb * 5
+
+
+def test_resource_shape_reserves_compute_units_for_the_other_streams(monkeypatch):
+    """A schedule's resource shape (sm_num, block_size) acts on the launches: while a partition that carries a
+    hand-over runs on its nanobatch's stream, that many compute units are reserved (GEMM launches take the
+    rest); partitions without a schedule entry, and runs without nanobatch streams, reserve nothing."""
+    from kareus_amd.backend import reserved_compute_units
+    from kareus_amd.backend.eager import EagerBackend
+
+    seen = []
+    real = EagerBackend.linear_fwd
+
+    def spy(self, x, w, **kw):
+        seen.append(reserved_compute_units())
+        return real(self, x, w, **kw)
+
+    monkeypatch.setattr(EagerBackend, "linear_fwd", spy)
+    rec = RecordingStreams()
+    cfg = LayerConfig(hidden_size=64, num_attention_heads=2, num_query_groups=1, kv_channels=32, ffn_hidden_size=64,
+                      num_layers=1, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
+    attn, mlp = CommConfig(("norm_0", "none"), (24, 1024)), CommConfig(("linear_0", "none"), (40, 512))
+
+    class Sch:
+        current_schedule = ScheduleItem(attn, mlp, attn, mlp)
+
+    with use_stream_api(rec):
+        m = LayerStack(cfg, seed=1)
+        cfg.kareus_scheduler = Sch()
+        with torch.no_grad():
+            m(torch.randn(16, 4, 64))
+    # per nanobatch: qkv, proj (fwd_attn), fc1, fc2 (fwd_mlp); the first partition of all carries no hand-over
+    assert sorted(seen) == sorted([0, 0, 24, 24, 40, 40, 40, 40])
+    assert reserved_compute_units() == 0
+    seen.clear()
+    cfg2 = LayerConfig(hidden_size=64, num_attention_heads=2, num_query_groups=1, kv_channels=32, ffn_hidden_size=64,
+                       num_layers=1, num_nanobatches=2, params_dtype=torch.float32, backend="eager", use_streams=False)
+    m2 = LayerStack(cfg2, seed=1)
+    cfg2.kareus_scheduler = Sch()
+    with torch.no_grad():
+        m2(torch.randn(16, 4, 64))
+    assert seen == [0] * 8
