@@ -5,12 +5,22 @@
 
 A step = one forward+backward of the decoder-layer stack over one synthetic batch, inputs
 resident in HBM.  Prints ONE JSON line (metric: layer fwd+bwd tokens/s) that also carries
-  roofline      the dominant kernel (fc1 forward GEMM at nanobatch shape) timed live with HIP
-                events on its stream, against the 2.5 PFLOP/s dense bf16 MFMA peak
+  roofline      the kernel with the largest share of the step's kernel time (the weight-gradient
+                GEMM of fc1 at nanobatch shape), timed live with HIP events on its stream, against
+                the 2.5 PFLOP/s dense bf16 MFMA peak; `roofline_others` has the other two layouts
   cpu_baseline  the CPU oracle (plain PyTorch fp32 layer) timed on the host cores on a bounded
                 sample of the same layer shape
-plus end-to-end MFMA utilisation, speed-up over the serial (1 nanobatch) run, overlap
-efficiency (sum of serially timed partition times / overlapped wall time) and joules/token.
+plus end-to-end MFMA utilisation, the nanobatched run beside the serial (1 nanobatch) run with
+the speed-up between them, overlap efficiency (sum of serially timed partition times / overlapped
+wall time), joules/token and the host's enqueue time per step.
+
+The chip is pre-heated for two seconds before anything is timed, and the three ways of running the
+layer that are compared (nanobatches on their own streams, one nanobatch, the same nanobatches on
+one stream) are timed in interleaved rounds, so that all of them see the same power and thermal
+state.  `value` is the run the engine is configured for; with `--nanobatches auto` that is the
+faster of the workload's nanobatch count and a single nanobatch, picked from those rounds (the
+reference, too, falls back to sequential execution where nanobatching costs more than it gives:
+tests/artifact/README.md:190-196), and `config.nanobatches` names the count that was run.
 """
 
 from __future__ import annotations
@@ -63,22 +73,58 @@ def make_model(w, nnb, device, use_streams=True, schedule=None):
     return LayerStack(cfg, device=device, seed=1234)
 
 
-def run_steps(model, x, go, steps):
-    for _ in range(steps):
-        for p in model.parameters():
+def make_scheduler(path, nnb):
+    """The communication scheduler over a per-microbatch plan file (None without a file or with a
+    single nanobatch, which has nothing to schedule)."""
+    if not path or nnb < 2:
+        return None
+    from kareus_amd.scheduler import PipelineCommScheduler
+    from kareus_amd.scheduler.parser import parse_schedule_file
+
+    stages = parse_schedule_file(path, False, False)
+    return PipelineCommScheduler(path, pp_rank=0, num_microbatches=len(stages[0]))
+
+
+class Stepper:
+    """Runs steps of one model; with a scheduler every step is one microbatch of the plan (forward
+    and backward instruction), and the plan starts over when its microbatches are used up."""
+
+    def __init__(self, model, x, go):
+        self.model, self.x, self.go = model, x, go
+        self.sch = model.config.kareus_scheduler
+        self.left = 0
+
+    def step(self):
+        sch = self.sch
+        if sch is not None:
+            if self.left == 0:
+                sch.on_step_begin()
+                self.left = len(sch._schedule_items)
+            sch.on_instruction_begin("forward")
+        for p in self.model.parameters():
             p.grad = None
-        x.grad = None
-        y = model(x)
-        y.backward(go)
+        self.x.grad = None
+        y = self.model(self.x)
+        if sch is not None:
+            sch.on_instruction_end("forward")
+            sch.on_instruction_begin("backward")
+        y.backward(self.go)
+        if sch is not None:
+            sch.on_instruction_end("backward")
+            self.left -= 1
+            if self.left == 0:
+                sch.on_step_end()
 
+    def run(self, steps):
+        for _ in range(steps):
+            self.step()
 
-def time_steps(model, x, go, steps, warmup):
-    run_steps(model, x, go, warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(model, x, go, steps)
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
+    def timed(self, steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.run(steps)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
 
 
 class EventTimer:
@@ -105,58 +151,191 @@ class EventTimer:
         return out
 
 
-def partition_times(model, x, go, iters=3):
+def partition_times(stepper, iters=3):
     from kareus_amd.partitions.partition_base import PartitionBase
 
-    run_steps(model, x, go, 1)
+    stepper.run(1)
     torch.cuda.synchronize()
     timer = EventTimer()
     PartitionBase.timer = timer
     try:
-        run_steps(model, x, go, iters)
+        stepper.run(iters)
         torch.cuda.synchronize()
     finally:
         PartitionBase.timer = None
     return {k: v / iters for k, v in timer.totals().items()}
 
 
-# HBM-side bytes per launch of the TN GEMM, from hardware counters (FETCH_SIZE and WRITE_SIZE of
-# two profiler runs of `bench.py --roofline-only`, each scaled by what the same counter reads for
-# `bench.py --copy-calibration`: x2.000 and x1.000).  Keyed by (M, N, K); shapes that were not
-# profiled report null.
-MEASURED_TRAFFIC_BYTES = {
-    (4096, 7168, 4096): 369.7e6 + 58.7e6,
+# HBM-side bytes per launch from hardware counters (FETCH_SIZE and WRITE_SIZE of two profiler
+# runs of `bench.py --roofline-only`, each scaled by what the same counter reads for
+# `bench.py --copy-calibration`).  Keyed by (layout, M, N, K); a shape that was not profiled
+# reports null.  A constant read off a profile, not something measured in this run: the entry
+# names the profile it came from.
+MEASURED_TRAFFIC = {
+    ("NT", 7168, 4096, 16384): {"bytes": (833940.0 * 2.000 + 57792.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 16384, 7168, 4096): {"bytes": (725713.1 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 16384, 4096, 7168): {"bytes": (688407.1 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
 }
 
 
-def dominant_kernel_roofline(w, nnb, device, launches=30):
-    """fc1 forward GEMM, y[T_nb, 2F] = x[T_nb, h] . W[2F, h]^T, timed with HIP events on the
-    stream it is launched on (torch's current stream)."""
-    from kareus_amd.backend import get_backend
+def _gemm_operands(layout, m, n, k, device):
+    a = torch.randn((k, m) if layout == "NT" else (m, k), device=device).bfloat16()
+    if layout == "TN":
+        b = (torch.randn(n, k, device=device) * 0.02).bfloat16()
+    elif layout == "NN":
+        b = (torch.randn(k, n, device=device) * 0.02).bfloat16()
+    else:
+        b = torch.randn(k, n, device=device).bfloat16()
+    return a, b
 
-    be = get_backend("hip")
-    m, n, k = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
-    a = torch.randn(m, k, device=device).bfloat16()
-    wt = (torch.randn(n, k, device=device) * 0.02).bfloat16()
+
+def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False):
+    """Average duration of one launch, HIP events on the stream the kernel is launched on."""
+    a, b = _gemm_operands(layout, m, n, k, device)
+    out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
+    y = torch.empty(m, n // 2, device=device, dtype=torch.bfloat16) if fused_swiglu else None
+    r = torch.randn(m, n, device=device).bfloat16() if residual else None
+    code = {"TN": 0, "NN": 1, "NT": 2}[layout]
+
+    def fn():
+        be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=False, swiglu_out=y, residual=r)
+
     for _ in range(5):
-        be.linear_fwd(a, wt)
+        fn()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(launches):
-        be.linear_fwd(a, wt)
+        fn()
     e1.record()
     torch.cuda.synchronize()
-    sec = e0.elapsed_time(e1) * 1e-3 / launches
+    return e0.elapsed_time(e1) * 1e-3 / launches
+
+
+def _roofline_entry(kernel, layout, m, n, k, sec):
     flops = 2.0 * m * n * k
     achieved = flops / sec / 1e12
+    traffic = MEASURED_TRAFFIC.get((layout, m, n, k))
     return {
-        "bound": "mfma", "kernel": "gemm_kernel<TN> (fc1 forward)", "shape": [m, n, k],
+        "bound": "mfma", "kernel": kernel, "shape": [m, n, k],
         "flops_per_launch": flops, "avg_launch_us": sec * 1e6,
         "achieved": achieved, "peak": MFMA_PEAK_BF16 / 1e12, "unit": "TFLOP/s",
         "frac": achieved * 1e12 / MFMA_PEAK_BF16,
-        "traffic": MEASURED_TRAFFIC_BYTES.get((m, n, k)),
+        "traffic": traffic["bytes"] if traffic else None,
+        "traffic_source": traffic["source"] if traffic else None,
     }
+
+
+def dominant_kernel_roofline(w, nnb, device, launches=30):
+    """The GEMM instance with the largest share of the step's kernel time: the weight gradient of
+    fc1, dW[2F, h] = dy[T_nb, 2F]^T . x[T_nb, h] (layout NT), plus the forward (TN, with the SwiGLU
+    epilogue the engine runs it with) and the input gradient (NN) of the same layer."""
+    from kareus_amd.backend import get_backend
+
+    be = get_backend("hip")
+    t, two_f, h = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
+    fuse = be.can_fuse_swiglu(two_f)
+    main = _roofline_entry("gemm_kernel<NT> (fc1 weight gradient)", "NT", two_f, h, t,
+                           time_gemm(be, "NT", two_f, h, t, device, launches))
+    others = [
+        _roofline_entry("gemm_kernel<TN%s> (fc1 forward)" % (", SwiGLU epilogue" if fuse else ""), "TN", t, two_f, h,
+                        time_gemm(be, "TN", t, two_f, h, device, launches, fused_swiglu=fuse)),
+        _roofline_entry("gemm_kernel<NN> (fc1 input gradient)", "NN", t, h, two_f,
+                        time_gemm(be, "NN", t, h, two_f, device, launches)),
+    ]
+    return main, others
+
+
+def gemm_kernels(w, nnb, device, launches=30):
+    """Every GEMM of the layer alone on the GPU at the nanobatch shape, the way the engine launches
+    it (forward of fc1 with the SwiGLU epilogue, of the out-projection and fc2 with the residual
+    epilogue, weight gradients accumulating into an existing buffer): TFLOP/s against the peak."""
+    from kareus_amd.backend import get_backend
+
+    be = get_backend("hip")
+    t, h, f = (w["b"] // nnb) * w["s"], w["h"], w["ffn"]
+    qkv, proj_in = (w["nq"] + 2 * w["nkv"]) * w["hd"], w["nq"] * w["hd"]
+    layers = [("qkv", h, qkv), ("proj", proj_in, h), ("fc1", h, 2 * f), ("fc2", f, h)]
+    rows = []
+    for name, k_in, n_out in layers:
+        variants = [
+            ("forward", "TN", t, n_out, k_in, dict(fused_swiglu=name == "fc1" and be.can_fuse_swiglu(n_out),
+                                                    residual=name in ("proj", "fc2"))),
+            ("input gradient", "NN", t, k_in, n_out, {}),
+            ("weight gradient", "NT", n_out, k_in, t, {}),
+            ("weight gradient, accumulating", "NT", n_out, k_in, t, dict(accumulate=True)),
+        ]
+        for what, layout, m, n, k, kw in variants:
+            sec = time_gemm(be, layout, m, n, k, device, launches, **kw)
+            flops = 2.0 * m * n * k
+            rows.append({"gemm": f"{name} {what}", "layout": layout, "shape": [m, n, k], "epilogue": kw,
+                         "avg_launch_us": sec * 1e6, "TFLOPs": flops / sec / 1e12,
+                         "frac_of_peak": flops / sec / MFMA_PEAK_BF16})
+    return rows
+
+
+def power_trace(w, device, seconds=2.0):
+    """Board power and shader clock (hwmon, 100 Hz) while the GPU idles, runs one GEMM back to back,
+    runs the attention kernels, an HBM-bound kernel, and the layer step with the workload's
+    nanobatch count and with one nanobatch: what the step's time and energy are made of."""
+    from kareus_amd.backend import get_backend
+    from kareus_amd.energy import ClockReader, PowerSampler
+
+    be = get_backend("hip")
+    sampler, clock = PowerSampler(0, hz=100.0), ClockReader(0)
+    t_nb, two_f, h = (w["b"] // w["nnb"]) * w["s"], 2 * w["ffn"], w["h"]
+    a, b = _gemm_operands("TN", t_nb, two_f, h, device)
+    out = torch.empty(t_nb, two_f, device=device, dtype=torch.bfloat16)
+    q = torch.randn(w["s"], w["b"], w["nq"], w["hd"], device=device, dtype=torch.bfloat16)
+    k = torch.randn(w["s"], w["b"], w["nkv"], w["hd"], device=device, dtype=torch.bfloat16)
+    v = torch.randn_like(k)
+    xa = torch.randn(w["b"] * w["s"], h, device=device, dtype=torch.bfloat16)
+    xb = torch.randn_like(xa)
+    gen = torch.Generator().manual_seed(42)
+    x = torch.randn(w["s"], w["b"], h, generator=gen).to(device, torch.bfloat16).requires_grad_(True)
+    go = torch.randn(w["s"], w["b"], h, generator=gen).to(device, torch.bfloat16)
+    steppers = {n: Stepper(make_model(w, n, device), x, go) for n in sorted({w["nnb"], 1})}
+    phases = [
+        ("idle", None, 0.0),
+        ("gemm fc1 forward, back to back", lambda: be.gemm(0, a, b, t_nb, two_f, h, out=out, split_k=False),
+         2.0 * t_nb * two_f * h),
+        ("attention forward, whole microbatch", lambda: be.attn_fwd(q, k, v, w["hd"] ** -0.5),
+         2.0 * w["b"] * w["nq"] * w["s"] ** 2 * w["hd"]),
+        ("residual add (HBM-bound)", lambda: be.add(xa, xb), 0.0),
+    ] + [(f"layer step, {n} nanobatch(es)", steppers[n].step, total_flops(w)) for n in steppers]
+    rows = []
+    for name, fn, flops in phases:
+        calls = 0
+        if fn is not None:
+            for _ in range(3):
+                fn()
+        torch.cuda.synchronize()
+        sampler.start()
+        clock.start()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            if fn is None:
+                time.sleep(0.05)
+            else:
+                for _ in range(8):
+                    fn()
+                calls += 8
+                torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        sampler.stop()
+        clock.stop()
+        joules = sampler.energy_joules(t0, t1) if sampler.available else None
+        mhz = clock.values(t0 + 0.5, t1)
+        rows.append({
+            "phase": name, "seconds": t1 - t0, "calls": calls,
+            "ms_per_call": (t1 - t0) / calls * 1e3 if calls else None,
+            "mean_watts": joules / (t1 - t0) if joules else None,
+            "joules_per_call": joules / calls if joules and calls else None,
+            "sclk_mhz_mean": sum(mhz) / len(mhz) if mhz else None,
+            "sclk_mhz_min": min(mhz) if mhz else None, "sclk_mhz_max": max(mhz) if mhz else None,
+            "TFLOPs": flops * calls / (t1 - t0) / 1e12 if flops and calls else None,
+        })
+    return {"bus_id": sampler.bus_id, "rows": rows}
 
 
 def copy_calibration(device, n=1 << 29, launches=10):
@@ -300,15 +479,89 @@ def cpu_baseline(w, budget_s=25.0):
     }
 
 
+def preheat(stepper, seconds=2.0):
+    """Run the layer until the chip has been busy for `seconds`: clocks and temperature settle at what a
+    training run sees, instead of the first timed window getting a cool chip and the last a hot one."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        stepper.run(4)
+        torch.cuda.synchronize()
+
+
+def interleaved_rounds(steppers, steps_per_turn, rounds):
+    """Time the given ways of running the layer in turn, `rounds` times over (A B C A B C ...), so that
+    all of them see the same chip state; returns name -> median seconds per step."""
+    samples = {name: [] for name in steppers}
+    for _ in range(rounds):
+        for name, st in steppers.items():
+            samples[name].append(st.timed(steps_per_turn))
+    return {name: sorted(v)[len(v) // 2] for name, v in samples.items()}, samples
+
+
+def host_enqueue_ms(stepper, repeats=5):
+    """Host time to enqueue one step (forward and backward calls return once everything is queued);
+    the GPU is idle at the start of each measurement, so nothing here waits for the device."""
+    times = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        stepper.step()
+        times.append(time.perf_counter() - t0)
+        torch.cuda.synchronize()
+    return sorted(times)[len(times) // 2] * 1e3
+
+
+def energy_per_iteration(stepper, tokens, sec_per_step, min_seconds=2.0, min_steps=20):
+    """Board power sampled at 100 Hz on a thread while the layer runs; every iteration ends with a device
+    synchronisation and a timestamp, and the samples are integrated over each iteration's window (the
+    pattern of the reference's per-window energy measurement, tests/bayesian/common/hardware.py:121-132).
+    Iterations shorter than two sampling periods are grouped so that every window holds samples."""
+    from kareus_amd.energy import PowerSampler
+
+    sampler = PowerSampler(0, hz=100.0)
+    if not sampler.available:
+        return {"joules_per_token": None}
+    group = max(1, int(0.03 / sec_per_step) + 1)            # iterations per energy window (>= 30 ms)
+    windows = max(min_steps // group + 1, int(min_seconds / (sec_per_step * group)) + 1)
+    sampler.start()
+    torch.cuda.synchronize()
+    marks = [time.perf_counter()]
+    for _ in range(windows):
+        stepper.run(group)
+        torch.cuda.synchronize()
+        marks.append(time.perf_counter())
+    sampler.stop()
+    per_iter = []
+    for a, b in zip(marks, marks[1:]):
+        e = sampler.energy_joules(a, b)
+        if e is not None:
+            per_iter.append(e / group)
+    total = sampler.energy_joules(marks[0], marks[-1])
+    if total is None or not per_iter:
+        return {"joules_per_token": None}
+    n = windows * group
+    return {
+        "joules_per_token": total / (n * tokens), "mean_watts": total / (marks[-1] - marks[0]),
+        "energy": {"iterations": n, "iterations_per_window": group, "joules_per_iteration_mean": total / n,
+                   "joules_per_iteration_min": min(per_iter), "joules_per_iteration_max": max(per_iter),
+                   "joules_per_iteration": [round(e, 4) for e in per_iter[:32]],
+                   "power_sensor_bus_id": sampler.bus_id},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
-    ap.add_argument("--nanobatches", type=int, default=0, help="override the workload's nanobatch count")
+    ap.add_argument("--nanobatches", default="auto",
+                    help="'auto' (default): the faster of the workload's nanobatch count and one nanobatch, "
+                         "measured; 'workload': the workload's count; or a number")
+    ap.add_argument("--schedule", default=None,
+                    help="per-microbatch plan file for the nanobatched run (default: the shipped plan for c5, none otherwise)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extras", action="store_true", help="skip serial/partition/energy legs")
+    ap.add_argument("--no-extras", action="store_true", help="skip the partition, energy and host-enqueue legs")
     ap.add_argument("--one-stream", action="store_true",
                     help="run every nanobatch on the caller's stream (no overlap; for profiling)")
     ap.add_argument("--roofline-only", action="store_true",
@@ -319,6 +572,10 @@ def main():
                     help="run only the attention forward/backward stand-alone (TFLOP/s against the MFMA peak)")
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
+    ap.add_argument("--gemm-kernels", action="store_true",
+                    help="run only the layer's twelve GEMMs stand-alone at nanobatch shape, as the engine launches them")
+    ap.add_argument("--power-trace", action="store_true",
+                    help="run only the power / shader-clock trace over kernels and layer steps")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs one GPU's shard of the layer; --gpus must be 1 "
@@ -327,12 +584,15 @@ def main():
         sys.exit("bench.py: needs a HIP device")
 
     w = dict(WORKLOADS[args.workload])
-    if args.nanobatches:
-        w["nnb"] = args.nanobatches
+    choice = args.nanobatches
+    if choice not in ("auto", "workload"):
+        w["nnb"] = int(choice)
+        choice = "fixed"
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.roofline_only:
-        print(json.dumps({"roofline": dominant_kernel_roofline(w, w["nnb"], device)}))
+        main_kernel, others = dominant_kernel_roofline(w, w["nnb"], device)
+        print(json.dumps({"roofline": main_kernel, "roofline_others": others}))
         return
     if args.copy_calibration:
         print(json.dumps({"copy_calibration": copy_calibration(device)}))
@@ -343,14 +603,44 @@ def main():
     if args.hbm_kernels:
         print(json.dumps({"hbm_kernels": hbm_kernels(w, w["nnb"], device)}))
         return
+    if args.gemm_kernels:
+        print(json.dumps({"gemm_kernels": gemm_kernels(w, w["nnb"], device)}))
+        return
+    if args.power_trace:
+        print(json.dumps({"power_trace": power_trace(w, device)}))
+        return
     gen = torch.Generator().manual_seed(42)
     x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
     go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
     tokens = w["b"] * w["s"]
     flops = total_flops(w)
 
-    model = make_model(w, w["nnb"], device, use_streams=not args.one_stream)
-    sec = time_steps(model, x, go, args.steps, args.warmup)
+    schedule_path = args.schedule
+    if schedule_path is None and args.workload == "c5":
+        from kareus_amd.plans import plan_path
+
+        schedule_path = plan_path("llama31_8b_4layers_mbs2_seq8192.py")
+    nano = Stepper(make_model(w, w["nnb"], device, use_streams=not args.one_stream,
+                              schedule=make_scheduler(schedule_path, w["nnb"])), x, go)
+    ways = {"nanobatched": nano}
+    if w["nnb"] > 1:
+        ways["serial_1nb"] = Stepper(make_model(w, 1, device, use_streams=False), x, go)
+        if not args.no_extras:
+            ways["same_nb_one_stream"] = Stepper(make_model(w, w["nnb"], device, use_streams=False,
+                                                            schedule=make_scheduler(schedule_path, w["nnb"])), x, go)
+    for st in ways.values():
+        st.run(2)
+    preheat(nano, 2.0)
+    med, samples = interleaved_rounds(ways, max(3, args.steps // 4), 5)
+    picked = "nanobatched"
+    if choice == "auto" and "serial_1nb" in med and med["serial_1nb"] < med["nanobatched"]:
+        picked = "serial_1nb"
+    runner = ways[picked]
+    run_nnb = 1 if picked == "serial_1nb" else w["nnb"]
+
+    # the headline: W warm-up steps, then exactly K timed steps of the chosen configuration
+    runner.run(args.warmup)
+    sec = runner.timed(args.steps)
 
     out = {
         "metric": "layer fwd+bwd tokens/sec on 1 MI355X",
@@ -359,52 +649,40 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['label']}", "hidden": w["h"], "q_heads": w["nq"],
                    "kv_heads": w["nkv"], "head_dim": w["hd"], "ffn": w["ffn"], "layers": w["layers"],
-                   "batch": w["b"], "seq_len": w["s"], "nanobatches": w["nnb"]},
+                   "batch": w["b"], "seq_len": w["s"], "nanobatches": run_nnb,
+                   "nanobatches_of_the_workload": w["nnb"],
+                   "nanobatch_choice": {"auto": "measured: the faster of the workload's count and one nanobatch",
+                                        "workload": "the workload's count", "fixed": "given on the command line"}[choice],
+                   "schedule_file": os.path.relpath(schedule_path, ROOT) if (schedule_path and run_nnb > 1) else None},
         "mfma_util_end_to_end": flops / sec / MFMA_PEAK_BF16,
         "tflops_end_to_end": flops / sec / 1e12,
     }
+    if "serial_1nb" in med:
+        out["overlap"] = {
+            "timing": "interleaved rounds after a 2 s pre-heat, median of 5 rounds per way",
+            "nanobatched_ms": med["nanobatched"] * 1e3,
+            "serial_1nb_ms": med["serial_1nb"] * 1e3,
+            "speedup_vs_serial_1nb": med["serial_1nb"] / med["nanobatched"],
+            "rounds_ms": {k: [round(t * 1e3, 4) for t in v] for k, v in samples.items()},
+        }
+        if "same_nb_one_stream" in med:
+            out["overlap"]["same_nb_one_stream_ms"] = med["same_nb_one_stream"] * 1e3
+            out["overlap"]["speedup_vs_one_stream"] = med["same_nb_one_stream"] / med["nanobatched"]
 
     if not args.no_extras:
-        # energy: keep the layer running for >= 2 s under the power sampler
-        from kareus_amd.energy import PowerSampler
+        out.update(energy_per_iteration(runner, tokens, sec))
+        out["host_enqueue_ms_per_step"] = {name: host_enqueue_ms(st) for name, st in ways.items()
+                                           if name != "same_nb_one_stream"}
+        flat = ways.get("same_nb_one_stream")
+        if flat is not None:
+            # per-partition times: the same nanobatches on one stream, an event pair around each partition
+            parts = partition_times(flat)
+            out["overlap"]["partition_ms"] = parts
+            out["overlap"]["overlap_efficiency"] = sum(parts.values()) * 1e-3 / med["nanobatched"]
 
-        sampler = PowerSampler(0, hz=100.0)
-        if sampler.available:
-            n_e = max(args.steps, int(2.0 / sec) + 1)
-            sampler.start()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            run_steps(model, x, go, n_e)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            sampler.stop()
-            joules = sampler.energy_joules(t0, t1)
-            if joules is not None:
-                out["joules_per_token"] = joules / (n_e * tokens)
-                out["mean_watts"] = joules / (t1 - t0)
-        else:
-            out["joules_per_token"] = None
-
-        # serial baseline: one nanobatch, one stream
-        del model
-        serial = make_model(w, 1, device, use_streams=False)
-        sec_serial = time_steps(serial, x, go, max(3, args.steps // 2), 2)
-        del serial
-        # same nanobatch count, all on one stream (no overlap), with per-partition events
-        flat = make_model(w, w["nnb"], device, use_streams=False)
-        sec_flat = time_steps(flat, x, go, max(3, args.steps // 2), 2)
-        parts = partition_times(flat, x, go)
-        del flat
-        out["overlap"] = {
-            "serial_1nb_ms": sec_serial * 1e3,
-            "same_nb_one_stream_ms": sec_flat * 1e3,
-            "speedup_vs_serial_1nb": sec_serial / sec,
-            "speedup_vs_one_stream": sec_flat / sec,
-            "partition_ms": parts,
-            "overlap_efficiency": sum(parts.values()) * 1e-3 / sec,
-        }
-
-    out["roofline"] = dominant_kernel_roofline(w, w["nnb"], device)
+    ways.clear()
+    del nano, runner
+    out["roofline"], out["roofline_others"] = dominant_kernel_roofline(w, run_nnb, device)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))

@@ -145,3 +145,70 @@ class PowerSampler:
     def mean_watts(self, t0: float, t1: float) -> Optional[float]:
         e = self.energy_joules(t0, t1)
         return None if e is None else e / (t1 - t0)
+
+
+class ClockReader:
+    """Shader clock of the device sampled on a thread; ``values`` are MHz.  Sources, in order:
+    hwmon ``freq1_input`` (Hz), else the starred line of ``pp_dpm_sclk`` (``"S: 1714Mhz *"`` is
+    the clock in force when the driver lists a range instead of levels)."""
+
+    def __init__(self, device_index: int = 0, hz: float = 100.0) -> None:
+        dev = sysfs_device_dir(device_index)
+        paths = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", "freq1_input"))) if dev else []
+        self._hwmon = paths[0] if paths else None
+        dpm = os.path.join(dev, "pp_dpm_sclk") if dev else None
+        self._dpm = dpm if (self._hwmon is None and dpm and os.path.exists(dpm)) else None
+        self.available = self._hwmon is not None or self._dpm is not None
+        self.period = 1.0 / hz
+        self.samples: List[Tuple[float, float]] = []
+        self._stop = threading.Event()
+        self._thread: Optional[threading.Thread] = None
+
+    def read_mhz(self) -> Optional[float]:
+        try:
+            if self._hwmon is not None:
+                with open(self._hwmon) as f:
+                    return int(f.read().strip()) * 1e-6
+            with open(self._dpm) as f:
+                for line in f:
+                    if line.rstrip().endswith("*"):
+                        return parse_dpm_mhz(line)
+        except (OSError, ValueError):
+            pass
+        return None
+
+    def _loop(self) -> None:
+        while not self._stop.is_set():
+            mhz = self.read_mhz()
+            if mhz is not None:
+                self.samples.append((time.perf_counter(), mhz))
+            self._stop.wait(self.period)
+
+    def start(self) -> None:
+        if not self.available:
+            return
+        self.samples = []
+        self._stop.clear()
+        self._thread = threading.Thread(target=self._loop, daemon=True)
+        self._thread.start()
+
+    def stop(self) -> None:
+        if self._thread is not None:
+            self._stop.set()
+            self._thread.join()
+            self._thread = None
+
+    def values(self, t0: float, t1: float) -> List[float]:
+        return [v for t, v in self.samples if t0 <= t <= t1]
+
+
+def parse_dpm_mhz(line: str) -> Optional[float]:
+    """``"1: 2400Mhz *"`` or ``"S: 1714Mhz *"`` -> MHz."""
+    for tok in line.replace("*", " ").split():
+        low = tok.lower()
+        if low.endswith("mhz"):
+            try:
+                return float(low[:-3])
+            except ValueError:
+                return None
+    return None

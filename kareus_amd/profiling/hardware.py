@@ -102,7 +102,8 @@ def available_frequencies_mhz(device_index: int = 0) -> List[int]:
         with open(os.path.join(d, "pp_dpm_sclk")) as f:
             for line in f:
                 parts = line.split()
-                if len(parts) >= 2 and parts[1].lower().endswith("mhz"):
+                # "<level>: <MHz>Mhz [*]"; a line "S: <MHz>Mhz *" is the clock in force, not a level
+                if len(parts) >= 2 and parts[0][:-1].isdigit() and parts[1].lower().endswith("mhz"):
                     out.append(int(float(parts[1][:-3])))
     except OSError:
         return []
