@@ -479,6 +479,43 @@ def cpu_baseline(w, budget_s=25.0):
     }
 
 
+class _FixedSchedule:
+    """A scheduler stand-in that hands every partition the same window and resource shape."""
+
+    def __init__(self, window, reserved_cus):
+        from kareus_amd.scheduler import CommConfig, ScheduleItem
+
+        cc = CommConfig(window, (reserved_cus, 1024))
+        self.current_schedule = ScheduleItem(cc, cc, cc, cc)
+        self._schedule_items = [self.current_schedule]
+
+    def on_step_begin(self): pass
+    def on_step_end(self): pass
+    def on_instruction_begin(self, name): pass
+    def on_instruction_end(self, name=None): pass
+
+
+def cu_budget_sweep(w, device, budgets=(0, 8, 16, 32, 64), rounds=4, steps=6):
+    """The nanobatched layer step under schedules that reserve 0..64 compute units for the other
+    nanobatch streams (every partition's GEMMs launch on the rest), for the earliest release point
+    and for release after the partition; interleaved rounds after a pre-heat, median ms per step."""
+    gen = torch.Generator().manual_seed(42)
+    x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
+    go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
+    ways = {}
+    for window in (("norm_0", "none"), ("none", "none")):
+        for cus in budgets:
+            model = make_model(w, w["nnb"], device, schedule=_FixedSchedule(window, cus))
+            ways[f"release {window[0]}, {cus} units reserved"] = Stepper(model, x, go)
+    ways["no schedule"] = Stepper(make_model(w, w["nnb"], device), x, go)
+    ways["one nanobatch"] = Stepper(make_model(w, 1, device, use_streams=False), x, go)
+    for st in ways.values():
+        st.run(2)
+    preheat(ways["no schedule"], 2.0)
+    med, _ = interleaved_rounds(ways, steps, rounds)
+    return {name: t * 1e3 for name, t in med.items()}
+
+
 def preheat(stepper, seconds=2.0):
     """Run the layer until the chip has been busy for `seconds`: clocks and temperature settle at what a
     training run sees, instead of the first timed window getting a cool chip and the last a hot one."""
@@ -574,6 +611,8 @@ def main():
                     help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
     ap.add_argument("--gemm-kernels", action="store_true",
                     help="run only the layer's twelve GEMMs stand-alone at nanobatch shape, as the engine launches them")
+    ap.add_argument("--cu-budget-sweep", action="store_true",
+                    help="run only the nanobatched step under schedules reserving 0..64 compute units")
     ap.add_argument("--power-trace", action="store_true",
                     help="run only the power / shader-clock trace over kernels and layer steps")
     args = ap.parse_args()
@@ -605,6 +644,9 @@ def main():
         return
     if args.gemm_kernels:
         print(json.dumps({"gemm_kernels": gemm_kernels(w, w["nnb"], device)}))
+        return
+    if args.cu_budget_sweep:
+        print(json.dumps({"cu_budget_sweep_ms_per_step": cu_budget_sweep(w, device)}))
         return
     if args.power_trace:
         print(json.dumps({"power_trace": power_trace(w, device)}))
