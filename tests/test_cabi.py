@@ -99,3 +99,53 @@ def test_fused_gemm_argument_checks():
     assert call(2, None, 0, 16, 136, n=272) == -2            # no tile width divides 2F = 272
     assert call(7, None, 0, None, 0) == -1                   # unknown epilogue
     assert call(0, None, 0, None, 0, cus=-3) == -1
+
+
+def test_swiglu_epilogue_index_model():
+    """A CPU model of the store addresses of the GEMM's SwiGLU epilogue and of its gate / up interleave of
+    the weight rows (kr_gemm.hip), for every tile width: every element of x [M, 2F] and of the activation
+    [M, F] is written exactly once, no address leaves the tensors, and no offset that the kernel keeps in an
+    unsigned register is negative (the mistake that once sent a store 8 GB past the output)."""
+    import numpy as np
+
+    def check(M, F, WN):
+        N = 2 * F
+        assert N % (32 * WN) == 0
+        x_hits, y_hits = np.zeros((M, N), int), np.zeros((M, F), int)
+        for tm in range((M + 255) // 256):
+            for tn in range(N // (32 * WN)):
+                out_m0, out_n0 = tm * 256, tn * 16 * WN
+                for wave in range(4):
+                    wm, wn = wave >> 1, wave & 1
+                    m_wave = out_m0 + wm * 128
+                    rows_in = m_wave + 128 <= M
+                    n_store = out_n0 + (F if wn else 0)
+                    for lane in range(64):
+                        quad, rch = lane >> 4, lane & 15
+                        if 8 * rch >= 16 * WN:
+                            continue
+                        for mt in range(8):
+                            for q in range(4):                      # x: rows 4 q + quad of the block
+                                rr = 4 * q + quad
+                                row = m_wave + mt * 16 + rr
+                                if rows_in or row < M:
+                                    nlo = rr * N + 8 * rch          # kept unsigned in the kernel
+                                    assert nlo >= 0
+                                    r, c = divmod((m_wave + mt * 16) * N + n_store + nlo, N)
+                                    assert 0 <= r < M and c + 8 <= N
+                                    x_hits[r, c:c + 8] += 1
+                            for qq in range(2):                     # activation: this wave's half of the rows
+                                rr = 4 * (2 * wn + qq) + quad
+                                row = m_wave + mt * 16 + rr
+                                if rows_in or row < M:
+                                    c = out_n0 + 8 * rch
+                                    assert c + 8 <= F
+                                    y_hits[row, c:c + 8] += 1
+                for row in range(32 * WN):                          # B tile row -> weight row
+                    r = out_n0 + row if row < 16 * WN else out_n0 + (row - 16 * WN) + F
+                    assert 0 <= r < N and (row < 16 * WN) == (r < F)
+        assert (x_hits == 1).all() and (y_hits == 1).all()
+
+    for M, F, WN in [(512, 128, 8), (264, 384, 8), (264, 384, 6), (1000, 1024, 8), (520, 320, 5), (304, 672, 7),
+                     (304, 672, 6)]:
+        check(M, F, WN)
