@@ -54,6 +54,7 @@ constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
 constexpr uint32_t SLOT_BYTES = TILE * sizeof(bf16);
 constexpr int NSLOTS = 5;          // 5 x 32 KB = the whole 160 KB of LDS
 constexpr int kXcds = 8;
+constexpr int KR_GEMM_EPI_TRANSPOSED_OUT = 3;  // internal: not part of the C ABI's epilogue values
 constexpr int kGroupM = 4;
 
 // ---- LDS layouts (element offsets inside one operand tile) ----------------------------------
@@ -219,7 +220,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // SWIGLU: C = x [M, N = 2F] and out2 = silu(x[:, :F]) * x[:, F:] [M, F]; a tile then covers
   // 16 * WN columns of out2: its left half (the waves with wn = 0) computes their gate columns,
   // its right half (wn = 1) the matching up columns of x, and the two meet in the epilogue.
-  static_assert(EPI == KR_GEMM_EPI_NONE || (!A_T && !B_T), "fused epilogues: K-major layout only");
+  // TRANSPOSED_OUT (internal, layout NT only): the kernel computes the tile of C = A^T . B as
+  // always but stores C^T, i.e. the caller's output is [N, M] with row stride ldc.  The host uses
+  // it with the operands exchanged when the tile grid of the transposed problem fits the device
+  // better (256 x 224 tiles can then be 224 rows x 256 columns of the output).
+  constexpr bool trans_out = EPI == KR_GEMM_EPI_TRANSPOSED_OUT;
+  static_assert(EPI == KR_GEMM_EPI_NONE || trans_out || (!A_T && !B_T), "fused epilogues: K-major layout only");
+  static_assert(!trans_out || (A_T && B_T), "transposed store: layout NT only");
   constexpr bool epi_add = EPI == KR_GEMM_EPI_ADD;
   constexpr bool swiglu = EPI == KR_GEMM_EPI_SWIGLU;
   const int gate_up_f = swiglu ? N / 2 : 0;
@@ -367,9 +374,17 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     for (int g = 0; g < WT; ++g) {
 #pragma unroll
       for (int nt = 0; nt < WN; ++nt) {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
-                     : "+a"(acc[g][nt])
-                     : "v"(cur.b[nt]), "v"(cur.a[g]));
+        if constexpr (trans_out) {
+          // operands not swapped: a lane gets four consecutive rows of one column of C, which are
+          // four consecutive columns of one row of C^T
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                       : "+a"(acc[g][nt])
+                       : "v"(cur.a[g]), "v"(cur.b[nt]));
+        } else {
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                       : "+a"(acc[g][nt])
+                       : "v"(cur.b[nt]), "v"(cur.a[g]));
+        }
         if (nt == 0) nxt.a[g] = read_a(aa, g, h);
         if (nt == 2 && g < WN) nxt.b[g] = read_b(ba, g, h);
         if constexpr (DMA > 0) {
@@ -538,6 +553,39 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         }
       };
       if constexpr (epi_add) fetch_res(0);
+      if constexpr (trans_out) {
+        // C^T leaves in blocks of 16 of its rows (columns nt of the wave tile): the wave's eight
+        // 16 x 16 tiles of that column are 16 rows x 128 columns of C^T, staged and stored like a
+        // block of the plain path with the two tile indices exchanged.
+#pragma unroll
+        for (int nt = 0; nt < WN; ++nt) {
+          f32x4 vals[WT];
+#pragma unroll
+          for (int mt = 0; mt < WT; ++mt) {
+            vals[mt] = acc[mt][nt];
+            asm volatile("" : "+v"(vals[mt]));
+            acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+          const uint32_t buf = stage + (uint32_t)(nt & 1) * 4096u;
+#pragma unroll
+          for (int mt = 0; mt < WT; ++mt) {
+            bf16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (bf16)vals[mt][e];
+            *(KR_LDS bf16x4*)(buf + row16 * 256 + (((2 * mt + (quad >> 1)) ^ row16) << 4) + (quad & 1) * 8) = o;
+          }
+          wave_sync();
+          const bool tcols_in = m_wave + 8 * rch < M;   // M is a multiple of 8: the whole chunk is in or out
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int rr = 4 * q + quad;
+            const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
+            const int n = n_wave + nt * 16 + rr;
+            if (tcols_in && n < N) stg8(C + (int64_t)n * ldc + m_wave + 8 * rch, v);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
 #pragma unroll
       for (int mt = 0; mt < WT; ++mt) {
         if (add_old && mt + 1 < WT) fetch_old(mt + 1);
@@ -614,6 +662,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
           wave_sync();
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the accumulator reads of later blocks below
+      }
       }
     }
     if (!more) break;
@@ -890,9 +939,36 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
     case KR_GEMM_NN:  // A [M,K], B [K,N]
       if (lda < K || ldb < N || ldc < N) return KR_EINVAL;
       KR_GEMM_LAUNCH(false, true)
-    case KR_GEMM_NT:  // A [K,M], B [K,N]
+    case KR_GEMM_NT: {  // A [K,M], B [K,N]
       if (lda < M || ldb < N || ldc < N) return KR_EINVAL;
+      // Both operands of this layout are read the same way, so C^T = B^T . A is the same kernel
+      // with the operands exchanged and a transposing store.  Take that form when its tile grid
+      // needs fewer rounds of workgroups (fc1's weight gradient, 7168 x 4096: 448 tiles of
+      // 256 x 256 are two rounds on 224 units; transposed, 512 tiles of 256 x 224 are two full
+      // rounds of smaller tiles).  Only for a plain store: accumulation and split-K keep the
+      // direct form.
+      if (!accumulate && ((int64_t)M * lda < ((int64_t)1 << 31)) && M <= (1 << 26)) {
+        auto cost = [&](int rows, int cols, int w) {
+          const int tiles = ((rows + BM - 1) / BM) * ((cols + 32 * w - 1) / (32 * w));
+          return (long)((tiles + cus - 1) / cus) * (w + 1);
+        };
+        const int wt = choose_wn(N, M, cus);
+        const int tiles_direct = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        const int tiles_trans = ((N + BM - 1) / BM) * ((M + BN - 1) / BN);
+        if (tiles_direct >= 192 && tiles_trans >= 192 && cost(N, M, wt) < cost(M, N, wn)) {
+#define KR_GEMM_TRANS(W) \
+  return launch<true, true, W, KR_GEMM_EPI_TRANSPOSED_OUT>(b, ldb, a, lda, c, ldc, N, M, K, 0, nullptr, 0, st, num_cus, fu)
+          switch (wt) {
+            case 5: KR_GEMM_TRANS(5);
+            case 6: KR_GEMM_TRANS(6);
+            case 7: KR_GEMM_TRANS(7);
+            default: KR_GEMM_TRANS(8);
+          }
+#undef KR_GEMM_TRANS
+        }
+      }
       KR_GEMM_LAUNCH(true, true)
+    }
     default:
       return KR_EINVAL;
   }

@@ -354,3 +354,21 @@ def test_gemm_compute_unit_budget_changes_nothing_but_the_launch(be):
     full = be.linear_fwd(x, w, split_k=None)
     for cus in (1, 64, 200, 256, 1000):
         assert torch.equal(be.linear_fwd(x, w, split_k=False, max_cus=cus), full)
+
+
+@pytest.mark.parametrize("m,n,k", [(7168, 4096, 256), (7160, 4088, 200), (4096, 7168, 128), (3584, 8192, 72)])
+def test_weight_gradient_with_transposed_store(be, m, n, k):
+    """A weight gradient whose tile grid fits the device better the other way round (fc1 of workload c4:
+    7168 x 4096) is computed as the transposed product with a transposing store; results are those of the
+    direct form (which a call that accumulates still takes) and do not depend on the form bit for bit."""
+    dy, x = rnd(k, m, scale=0.1, seed=90), rnd(k, n, seed=91)
+    ref = dy.float().t() @ x.float()
+    got = be.linear_wgrad(dy, x, split_k=None)
+    assert rel(got, ref) <= TOL
+    direct = be.gemm(2, dy, x, m, n, k, out=torch.zeros(m, n, device=DEV, dtype=torch.bfloat16), accumulate=True,
+                     split_k=None)
+    assert torch.equal(got, direct)
+    wide = torch.zeros(m, n + 64, device=DEV, dtype=torch.bfloat16)        # row-strided output
+    be.gemm(2, dy, x, m, n, k, out=wide[:, :n], split_k=None)
+    assert torch.equal(wide[:, :n], got) and not wide[:, n:].any()
+    assert torch.equal(be.linear_wgrad(dy, x, split_k=None), got)
