@@ -42,8 +42,8 @@ HBM_PEAK = 8.0e12
 
 # name -> (hidden, nq, nkv, hd, ffn, layers, batch, seq, nanobatches)
 WORKLOADS = {
-    "c1gpu": dict(h=512, nq=4, nkv=4, hd=128, ffn=1376, layers=1, b=2, s=256, nnb=2,
-                  label="plumbing-sized layer (h512) in bf16"),
+    "c1gpu": dict(h=512, nq=8, nkv=8, hd=64, ffn=1376, layers=1, b=2, s=256, nnb=2,
+                  label="the CPU plumbing layer (h512, 8 heads of 64, ffn 1376) in bf16 on the device"),
     "c2": dict(h=3072, nq=3, nkv=1, hd=128, ffn=1024, layers=1, b=8, s=4096, nnb=2,
                label="Llama-3.2-3B layer, TP=8 shard, MBS 8 x seq 4096, 2 nanobatches"),
     "c3": dict(h=3072, nq=24, nkv=8, hd=128, ffn=8192, layers=1, b=4, s=4096, nnb=2,

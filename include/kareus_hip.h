@@ -184,7 +184,9 @@ int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* ou
  * straight into a buffer of that layout.
  * lse: [b, nq, s] fp32 contiguous (natural log-sum-exp of the scaled, masked scores).
  * Query head h reads KV head h/per.  Causal, query i sees keys <= i.
- * hd must be 128; s a multiple of 128.  All strides multiples of 8.
+ * hd: a multiple of 8, at most 128; any s.  Head dimension 128 with s a multiple of 128 (the
+ * training workloads) runs on the MFMA kernels; every other shape on general fp32 kernels that
+ * are correct and slow.  All strides multiples of 8.
  * kr_attn_bwd needs a workspace of kr_attn_bwd_workspace_bytes() bytes (16-byte aligned).   */
 int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                 int s, int b, int nq, int nkv, int hd, float scale,

@@ -133,9 +133,13 @@ __device__ __forceinline__ void store_rows_f32(const RowStage& st, const f32x16 
 
 static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
   if (s <= 0 || b <= 0 || nq <= 0 || nkv <= 0) return KR_EINVAL;
-  if (hd != HD || s % BQ || nq % nkv) return KR_EUNSUPPORTED;
+  if (hd <= 0 || hd % 8 || hd > 128 || nq % nkv) return KR_EUNSUPPORTED;
+  if (b > 65535 || nq > 65535) return KR_EUNSUPPORTED;  // grid dimensions of the general kernels
   return KR_OK;
 }
+// The MFMA kernels take head dimension 128 and whole 128-row tiles; everything else that passes
+// check_attn_common goes through the general fp32 kernels.
+static bool attn_fast_path(int s, int hd) { return hd == HD && s % BQ == 0; }
 
 // The kernels keep a sequence stride in 32 bits and build per-lane byte offsets of up to
 // (48 * stride + 128) * 2 from it: strides must be positive and small enough for that.
@@ -1063,6 +1067,269 @@ template __global__ void attn_bwd_dkdv_kernel<false>(KR_ATTN_DKDV_ARGS);
 template __global__ void attn_bwd_dkdv_kernel<true>(KR_ATTN_DKDV_ARGS);
 #undef KR_ATTN_DKDV_ARGS
 
+
+// =============================================================================================
+// General path: any sequence length, head dimensions that are a multiple of 8 up to 128.
+// The kernels above are built for head dimension 128 and sequences of whole 128-row tiles, the
+// shapes of the training workloads.  Everything else (head dimension 64, ragged lengths; the
+// reference's flash-attention call takes both) runs through these plain fp32 kernels: same
+// interface, same tensor layouts, same results to rounding, no MFMA — they exist so that such a
+// shape is computed on the device at all, not to be fast.  A workgroup of 256 threads owns 32
+// query rows (forward, dQ) or 32 keys (dK/dV) and walks 32-row tiles of the other operand through
+// LDS; a thread is (row r = tid / 8, part p = tid % 8): it computes the scores of row r against
+// keys 4 p .. 4 p + 3 of a tile and owns channels p hd/8 .. (p + 1) hd/8 - 1 of row r's
+// accumulators.  Rows beyond the sequence are loaded as zeros and never stored.  No atomics:
+// grouped query heads are summed inside the dK/dV workgroup, in a fixed order.
+// =============================================================================================
+namespace general {
+
+constexpr int GT = 32;          // rows per tile (queries or keys)
+constexpr int GTHREADS = 256;
+constexpr int GHD_MAX = 128;
+constexpr int GLD = GHD_MAX + 8;  // LDS row stride in elements (rows stay 16-byte aligned)
+
+// rows row0 .. row0 + 31 of a [s, hd] matrix with row stride ss -> LDS tile, zeros beyond s
+__device__ __forceinline__ void load_tile(bf16* dst, const bf16* src, int64_t ss, int row0, int s,
+                                          int hd, int tid) {
+  const int vecs = hd / 8;
+  for (int i = tid; i < GT * vecs; i += GTHREADS) {
+    const int r = i / vecs, c = (i - r * vecs) * 8;
+    const bf16x8 v = row0 + r < s ? ldg8(src + (int64_t)(row0 + r) * ss + c) : zero8();
+    *reinterpret_cast<bf16x8*>(dst + r * GLD + c) = v;
+  }
+}
+
+// sum / max over the 8 threads that share a row (consecutive lanes)
+__device__ __forceinline__ float row_sum(float v) {
+  v += __shfl_xor(v, 1, KR_WAVE);
+  v += __shfl_xor(v, 2, KR_WAVE);
+  v += __shfl_xor(v, 4, KR_WAVE);
+  return v;
+}
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 1, KR_WAVE));
+  v = fmaxf(v, __shfl_xor(v, 2, KR_WAVE));
+  v = fmaxf(v, __shfl_xor(v, 4, KR_WAVE));
+  return v;
+}
+
+// dot products of row `r` of tile a with rows 4 p .. 4 p + 3 of tile b over hd channels
+__device__ __forceinline__ void dot4(const bf16* a, const bf16* b, int r, int p, int hd, float (&out)[4]) {
+  out[0] = out[1] = out[2] = out[3] = 0.f;
+  const bf16* ar = a + r * GLD;
+  const bf16* b0 = b + (4 * p) * GLD;
+  for (int d = 0; d < hd; ++d) {
+    const float av = (float)ar[d];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] += av * (float)b0[j * GLD + d];
+  }
+}
+
+__global__ __launch_bounds__(GTHREADS) void attn_general_fwd_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, int hd, float scale,
+    QLayout ql, KLayout kl, KLayout vl, QLayout ol) {
+  __shared__ __attribute__((aligned(16))) bf16 sq[GT * GLD], sk[GT * GLD], sv[GT * GLD];
+  __shared__ float sp[GT][GT + 1];
+  const int tid = threadIdx.x, r = tid >> 3, p = tid & 7;
+  const int q0 = blockIdx.x * GT, head = blockIdx.y, bi = blockIdx.z;
+  const int per = nq / nkv, kvh = head / per, c = hd / 8;
+  const bf16* qb = q + ql.at(bi, head, per);
+  const bf16* kb = k + kl.at(bi, kvh);
+  const bf16* vb = v + vl.at(bi, kvh);
+  load_tile(sq, qb, ql.s_, q0, s, hd, tid);
+  float acc[GHD_MAX / 8];
+#pragma unroll
+  for (int i = 0; i < GHD_MAX / 8; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const int qrow = q0 + r;
+  const int last_key = (q0 + GT - 1 < s ? q0 + GT - 1 : s - 1);
+  for (int k0 = 0; k0 <= last_key; k0 += GT) {
+    __syncthreads();  // the previous tile's K, V and probabilities are no longer read
+    load_tile(sk, kb, kl.s_, k0, s, hd, tid);
+    load_tile(sv, vb, vl.s_, k0, s, hd, tid);
+    __syncthreads();
+    float sc[4];
+    dot4(sq, sk, r, p, hd, sc);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int key = k0 + 4 * p + j;
+      sc[j] = (key <= qrow && key < s) ? sc[j] * scale : -INFINITY;
+      mx = fmaxf(mx, sc[j]);
+    }
+    mx = row_max(mx);
+    const float m_new = fmaxf(m, mx);
+    float pr[4], ps = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      pr[j] = sc[j] == -INFINITY ? 0.f : __expf(sc[j] - m_new);
+      ps += pr[j];
+      sp[r][4 * p + j] = pr[j];
+    }
+    ps = row_sum(ps);
+    const float alpha = m == -INFINITY ? 0.f : __expf(m - m_new);
+    l = l * alpha + ps;
+    m = m_new;
+    __syncthreads();
+    for (int i = 0; i < c; ++i) acc[i] *= alpha;
+    for (int kj = 0; kj < GT; ++kj) {
+      const float pv = sp[r][kj];
+      const bf16* vr = sv + kj * GLD + p * c;
+      for (int i = 0; i < c; ++i) acc[i] += pv * (float)vr[i];
+    }
+  }
+  if (qrow < s) {
+    const float inv = 1.0f / l;
+    bf16* orow = o + ol.at(bi, head, per) + (int64_t)qrow * ol.s_ + p * c;
+    for (int i = 0; i < c; ++i) orow[i] = (bf16)(acc[i] * inv);
+    if (p == 0) lse[((int64_t)bi * nq + head) * s + qrow] = m + __logf(l);
+  }
+}
+
+// delta[b, h, i] = sum_d dO[i, d] O[i, d]
+__global__ __launch_bounds__(GTHREADS) void attn_general_delta_kernel(
+    const bf16* __restrict__ dout, const bf16* __restrict__ o, float* __restrict__ delta, int s,
+    int nq, int nkv, int hd, QLayout dol, QLayout ol) {
+  const int tid = threadIdx.x, r = tid >> 3, p = tid & 7;
+  const int row = blockIdx.x * GT + r, head = blockIdx.y, bi = blockIdx.z;
+  const int per = nq / nkv, c = hd / 8;
+  float sum = 0.f;
+  if (row < s) {
+    const bf16* dr = dout + dol.at(bi, head, per) + (int64_t)row * dol.s_ + p * c;
+    const bf16* orow = o + ol.at(bi, head, per) + (int64_t)row * ol.s_ + p * c;
+    for (int i = 0; i < c; ++i) sum += (float)dr[i] * (float)orow[i];
+  }
+  sum = row_sum(sum);
+  if (row < s && p == 0) delta[((int64_t)bi * nq + head) * s + row] = sum;
+}
+
+// P and dS of one 32 x 32 block: thread (r, p) handles query row r against keys 4 p .. 4 p + 3
+__device__ __forceinline__ void block_p_ds(const bf16* sq, const bf16* sk, const bf16* sv, const bf16* sdo,
+                                           const float* slse, const float* sdelta, int r, int p, int hd,
+                                           int q0, int k0, int s, float scale, float (&pr)[4],
+                                           float (&ds)[4]) {
+  float sc[4], dp[4];
+  dot4(sq, sk, r, p, hd, sc);
+  dot4(sdo, sv, r, p, hd, dp);
+  const int qrow = q0 + r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int key = k0 + 4 * p + j;
+    const bool valid = key <= qrow && key < s && qrow < s;
+    pr[j] = valid ? __expf(sc[j] * scale - slse[r]) : 0.f;
+    ds[j] = pr[j] * (dp[j] - sdelta[r]) * scale;
+  }
+}
+
+__global__ __launch_bounds__(GTHREADS) void attn_general_dkdv_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16* __restrict__ dk, bf16* __restrict__ dv, int s, int nq, int nkv, int hd, float scale,
+    QLayout ql, KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
+  __shared__ __attribute__((aligned(16))) bf16 sq[GT * GLD], sk[GT * GLD], sv[GT * GLD], sdo[GT * GLD];
+  __shared__ float sp[GT][GT + 1], sds[GT][GT + 1], slse[GT], sdelta[GT];
+  const int tid = threadIdx.x, r = tid >> 3, p = tid & 7;
+  const int k0 = blockIdx.x * GT, kvh = blockIdx.y, bi = blockIdx.z;
+  const int per = nq / nkv, c = hd / 8;
+  load_tile(sk, k + kl.at(bi, kvh), kl.s_, k0, s, hd, tid);
+  load_tile(sv, v + vl.at(bi, kvh), vl.s_, k0, s, hd, tid);
+  float adk[GHD_MAX / 8], adv[GHD_MAX / 8];
+#pragma unroll
+  for (int i = 0; i < GHD_MAX / 8; ++i) adk[i] = adv[i] = 0.f;
+  for (int hj = 0; hj < per; ++hj) {
+    const int head = kvh * per + hj;
+    const bf16* qb = q + ql.at(bi, head, per);
+    const bf16* dob = dout + dol.at(bi, head, per);
+    const int64_t stat = ((int64_t)bi * nq + head) * s;
+    for (int q0 = k0; q0 < s; q0 += GT) {  // query tiles at or below the diagonal (k0 is a multiple of 32)
+      __syncthreads();
+      load_tile(sq, qb, ql.s_, q0, s, hd, tid);
+      load_tile(sdo, dob, dol.s_, q0, s, hd, tid);
+      if (tid < GT) {
+        const bool in = q0 + tid < s;
+        slse[tid] = in ? lse[stat + q0 + tid] : 0.f;
+        sdelta[tid] = in ? delta[stat + q0 + tid] : 0.f;
+      }
+      __syncthreads();
+      float pr[4], ds[4];
+      block_p_ds(sq, sk, sv, sdo, slse, sdelta, r, p, hd, q0, k0, s, scale, pr, ds);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sp[r][4 * p + j] = pr[j];
+        sds[r][4 * p + j] = ds[j];
+      }
+      __syncthreads();
+      // this thread now is (key r, channels p c ..): dV += P^T dO, dK += dS^T Q
+      for (int qi = 0; qi < GT; ++qi) {
+        const float pv = sp[qi][r], dsv = sds[qi][r];
+        const bf16* dor = sdo + qi * GLD + p * c;
+        const bf16* qr = sq + qi * GLD + p * c;
+        for (int i = 0; i < c; ++i) {
+          adv[i] += pv * (float)dor[i];
+          adk[i] += dsv * (float)qr[i];
+        }
+      }
+    }
+  }
+  if (k0 + r < s) {
+    bf16* dkr = dk + dkl.at(bi, kvh) + (int64_t)(k0 + r) * dkl.s_ + p * c;
+    bf16* dvr = dv + dvl.at(bi, kvh) + (int64_t)(k0 + r) * dvl.s_ + p * c;
+    for (int i = 0; i < c; ++i) {
+      dkr[i] = (bf16)adk[i];
+      dvr[i] = (bf16)adv[i];
+    }
+  }
+}
+
+__global__ __launch_bounds__(GTHREADS) void attn_general_dq_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16* __restrict__ dq, int s, int nq, int nkv, int hd, float scale, QLayout ql, KLayout kl,
+    KLayout vl, QLayout dol, QLayout dql) {
+  __shared__ __attribute__((aligned(16))) bf16 sq[GT * GLD], sk[GT * GLD], sv[GT * GLD], sdo[GT * GLD];
+  __shared__ float sds[GT][GT + 1], slse[GT], sdelta[GT];
+  const int tid = threadIdx.x, r = tid >> 3, p = tid & 7;
+  const int q0 = blockIdx.x * GT, head = blockIdx.y, bi = blockIdx.z;
+  const int per = nq / nkv, kvh = head / per, c = hd / 8;
+  const int64_t stat = ((int64_t)bi * nq + head) * s;
+  load_tile(sq, q + ql.at(bi, head, per), ql.s_, q0, s, hd, tid);
+  load_tile(sdo, dout + dol.at(bi, head, per), dol.s_, q0, s, hd, tid);
+  if (tid < GT) {
+    const bool in = q0 + tid < s;
+    slse[tid] = in ? lse[stat + q0 + tid] : 0.f;
+    sdelta[tid] = in ? delta[stat + q0 + tid] : 0.f;
+  }
+  const bf16* kb = k + kl.at(bi, kvh);
+  const bf16* vb = v + vl.at(bi, kvh);
+  float adq[GHD_MAX / 8];
+#pragma unroll
+  for (int i = 0; i < GHD_MAX / 8; ++i) adq[i] = 0.f;
+  const int last_key = (q0 + GT - 1 < s ? q0 + GT - 1 : s - 1);
+  for (int k0 = 0; k0 <= last_key; k0 += GT) {
+    __syncthreads();
+    load_tile(sk, kb, kl.s_, k0, s, hd, tid);
+    load_tile(sv, vb, vl.s_, k0, s, hd, tid);
+    __syncthreads();
+    float pr[4], ds[4];
+    block_p_ds(sq, sk, sv, sdo, slse, sdelta, r, p, hd, q0, k0, s, scale, pr, ds);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sds[r][4 * p + j] = ds[j];
+    __syncthreads();
+    for (int kj = 0; kj < GT; ++kj) {
+      const float dsv = sds[r][kj];
+      const bf16* kr = sk + kj * GLD + p * c;
+      for (int i = 0; i < c; ++i) adq[i] += dsv * (float)kr[i];
+    }
+  }
+  if (q0 + r < s) {
+    bf16* dqr = dq + dql.at(bi, head, per) + (int64_t)(q0 + r) * dql.s_ + p * c;
+    for (int i = 0; i < c; ++i) dqr[i] = (bf16)adq[i];
+  }
+}
+
+}  // namespace general
+
 }  // namespace
 
 // The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
@@ -1072,6 +1339,7 @@ static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <=
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
   if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
   size_t bytes = 2 * (size_t)b * nq * s * sizeof(float);  // delta, and -lse in the log2 domain
+  if (!attn_fast_path(s, hd)) return bytes;               // the general kernels only keep delta
   const int qsplit = dkdv_query_split(s, b, nq);
   if (nq != nkv || qsplit > 1)  // fp32 dK, dV partials per (query head, query-tile part)
     bytes += 2 * (size_t)b * nq * qsplit * s * hd * sizeof(float);
@@ -1109,6 +1377,21 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   const KLayout kl{k_ss, k_sb, k_sh}, vl{v_ss, v_sb, v_sh}, dkl{dk_ss, dk_sb, dk_sh},
       dvl{dv_ss, dv_sb, dv_sh};
   float* delta = (float*)workspace;
+  if (!attn_fast_path(s, hd)) {
+    using namespace general;
+    const dim3 qgrid((s + GT - 1) / GT, nq, b), kgrid((s + GT - 1) / GT, nkv, b);
+    hipLaunchKernelGGL(attn_general_delta_kernel, qgrid, dim3(GTHREADS), 0, st, (const bf16*)dout,
+                       (const bf16*)o, delta, s, nq, nkv, hd, dol, ol);
+    if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+    hipLaunchKernelGGL(attn_general_dkdv_kernel, kgrid, dim3(GTHREADS), 0, st, (const bf16*)q,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
+                       (bf16*)dk, (bf16*)dv, s, nq, nkv, hd, scale, ql, kl, vl, dol, dkl, dvl);
+    if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
+    hipLaunchKernelGGL(attn_general_dq_kernel, qgrid, dim3(GTHREADS), 0, st, (const bf16*)q,
+                       (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse, (const float*)delta,
+                       (bf16*)dq, s, nq, nkv, hd, scale, ql, kl, vl, dol, dql);
+    return kr_launch_status();
+  }
   const int64_t rows = (int64_t)b * nq * s;
   float* neg_lse2 = delta + rows;
   float* part_k = neg_lse2 + rows;
@@ -1187,6 +1470,15 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
     const int64_t seq[] = {q_ss, k_ss, v_ss, o_ss};
     if (!attn_strides_ok(seq, {q_sb, q_sg, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sg, o_sh}))
       return KR_EUNSUPPORTED;
+  }
+  if (!attn_fast_path(s, hd)) {
+    using namespace general;
+    const QLayout ql{q_ss, q_sb, q_sg, q_sh}, ol{o_ss, o_sb, o_sg, o_sh};
+    const KLayout kl{k_ss, k_sb, k_sh}, vl{v_ss, v_sb, v_sh};
+    hipLaunchKernelGGL(attn_general_fwd_kernel, dim3((s + GT - 1) / GT, nq, b), dim3(GTHREADS), 0,
+                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
+                       lse, s, nq, nkv, hd, scale, ql, kl, vl, ol);
+    return kr_launch_status();
   }
   // two K and two V tiles of 17 KiB (padded blocks) per half; afterwards the same memory holds
   // the hand-over of half 1 (66 KiB) and, from 68 KiB on, 4 KiB of output staging per wave

@@ -45,7 +45,8 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_gemm_bf16(0, 8, 8, 7, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -2
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1
     assert lib.kr_gemm_bf16(0, 8, 8, 8, 16, 8, 16, 8, 18, 8, 0, None, 0, None) == -1   # misaligned C
-    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 64) == 0  # head_dim 64 unsupported
+    assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 136) == 0  # head dimensions above 128 are unsupported
+    assert lib.kr_attn_bwd_workspace_bytes(250, 1, 4, 2, 64) == 2 * 250 * 4 * 4   # general kernels: delta (+ spare)
     # delta and the rescaled lse, plus fp32 dK/dV partials per query head when heads share KV heads ...
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 32, 128) == 2 * 4 * 32 * 4096 * 4
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 8, 128) == 2 * 4 * 32 * 4096 * 4 + 2 * 4 * 32 * 4096 * 128 * 4

@@ -304,9 +304,32 @@ def test_attention_special_cases(be):
     o2, _ = be.attn_fwd(q, k2, v2, hd ** -0.5)
     assert torch.equal(o2[:200], o[:200])
     with pytest.raises(RuntimeError, match="not supported"):
-        be.attn_fwd(rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), rnd(100, 1, 1, 128), 1.0)  # s % 128 != 0
-    with pytest.raises(RuntimeError, match="not supported"):
-        be.attn_fwd(rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), rnd(128, 1, 1, 64), 1.0)  # head_dim 64
+        be.attn_fwd(rnd(128, 1, 1, 136), rnd(128, 1, 1, 136), rnd(128, 1, 1, 136), 1.0)  # head_dim above 128
+
+
+@pytest.mark.parametrize("s,b,nq,nkv,hd", [(100, 1, 1, 1, 128),    # ragged length at the fast kernels' head dimension
+                                            (256, 2, 8, 8, 64),     # benchmark configuration 1: 8 heads of 64
+                                            (77, 3, 6, 2, 64),      # ragged, grouped queries
+                                            (200, 1, 4, 1, 96), (1, 1, 1, 1, 64), (130, 2, 4, 2, 128), (33, 1, 2, 2, 8)])
+def test_attention_general_shapes(be, s, b, nq, nkv, hd):
+    """Head dimensions other than 128 and sequence lengths that are not whole 128-row tiles run through the
+    general kernels: same interface and layouts (fused QKV views, dense tensors), checked like the fast path."""
+    _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=100)
+    do = rnd(s, b, nq, hd, seed=101)
+    scale = hd ** -0.5
+    o, lse = be.attn_fwd(q, k, v, scale)
+    qf, kf, vf = (t.float().cpu().clone().requires_grad_(True) for t in (q.flatten(2, 3), k, v))
+    ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
+    assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
+    assert torch.equal(o[0], v[0].repeat_interleave(nq // nkv, dim=1))     # one visible key: o = v exactly
+    ro.backward(do.float().cpu())
+    dq, dk, dv = be.attn_bwd(do, q, k, v, o, lse, scale)
+    assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
+    again = be.attn_bwd(do, q, k, v, o, lse, scale)                         # fixed order of every sum: same bits
+    assert all(torch.equal(x, y) for x, y in zip(again, (dq, dk, dv)))
+    qd = q.flatten(2, 3).contiguous()
+    od, lsed = be.attn_fwd(qd, k.contiguous(), v.contiguous(), scale)
+    assert torch.equal(od, o) and torch.equal(lsed, lse)
 
 
 # ------------------------------------------------------------------ fused GEMM epilogues

@@ -57,7 +57,8 @@ def _rel(got, want):
 
 
 @pytest.mark.parametrize("dims,s,b,layers", [
-    (R.LayerDims(512, 4, 4, 128, 1376), 256, 4, 1),     # config-1-sized plumbing layer (head_dim 128 on device)
+    (R.LayerDims(512, 8, 8, 64, 1376), 256, 4, 1),      # benchmark configuration 1's layer exactly (8 heads of 64), in bf16
+    (R.LayerDims(512, 4, 4, 128, 1376), 200, 4, 1),     # the same widths with head_dim 128 and a ragged sequence length
     (R.LayerDims(3072, 3, 1, 128, 1024), 512, 4, 1),    # config 2 widths (3B TP=8 shard), short sequence
     (R.LayerDims(1024, 8, 2, 128, 896), 384, 4, 2),     # config 4 ratios (8 q / 2 kv heads), two layers
 ])
