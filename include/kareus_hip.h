@@ -71,13 +71,19 @@ int kr_gemm_bf16(int layout, int M, int N, int K,
  *                       out2 [M, F] (row stride ld_out2) = silu(x[:, :F]) * x[:, F:] computed from the
  *                       bf16-rounded x (fused_swiglu_forward, bias_swiglu.py:14-20); bit-identical to
  *                       kr_gemm_bf16 + kr_swiglu_fwd.
- *   A fused epilogue needs layout TN and accumulate == 0 and is never computed split-K.
+ *   KR_GEMM_EPI_SWIGLU_BWD  layout NN (an input gradient, N = F): the product g = A.B [M, F] is the gradient
+ *                       of the SwiGLU activation's output and is not stored; aux = x [M, 2F] (row stride ld_aux)
+ *                       is the activation's input and C = dx [M, 2F] (ldc >= 2F) receives
+ *                       fused_swiglu_backward(bf16(g), x) (bias_swiglu.py:34-44); bit-identical to
+ *                       kr_gemm_bf16 + kr_swiglu_bwd.
+ *   ADD and SWIGLU need layout TN, SWIGLU_BWD layout NN; all need accumulate == 0 and are never split-K.
  * max_cus > 0 limits the launch to that many compute units (workgroups are persistent, one per
  * unit): the compute-unit share a schedule's resource_shape gives a partition
  * (kareus/megatron/core/partitions/partition_base.py:117-128); 0 = the whole device.             */
 #define KR_GEMM_EPI_NONE 0
 #define KR_GEMM_EPI_ADD 1
 #define KR_GEMM_EPI_SWIGLU 2
+#define KR_GEMM_EPI_SWIGLU_BWD 4
 int kr_gemm_bf16_fused(int layout, int M, int N, int K,
                        const void* A, int64_t lda, const void* B, int64_t ldb,
                        void* C, int64_t ldc, int accumulate,

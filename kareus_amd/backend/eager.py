@@ -35,8 +35,11 @@ class EagerBackend:
     def can_fuse_swiglu(two_f: int) -> bool:
         return two_f % 2 == 0
 
-    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
-        return dy @ w
+    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True, swiglu_bwd_x: Tensor = None) -> Tensor:
+        g = dy @ w
+        return g if swiglu_bwd_x is None else self.swiglu_bwd(g, swiglu_bwd_x)
+
+    can_fuse_swiglu_bwd = True
 
     def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False,
                      split_k: bool = True) -> Tensor:

@@ -140,21 +140,32 @@ class HipBackend:
 
     def gemm(self, layout: int, a: Tensor, b: Tensor, m: int, n: int, k: int,
              out: Tensor = None, accumulate: bool = False, split_k: bool = True,
-             residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0) -> Tensor:
+             residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0,
+             swiglu_bwd_x: Tensor = None) -> Tensor:
         """``split_k=True``: the GEMM has the GPU to itself and splits the contraction of a small
         output for the shortest latency.  ``split_k=False``: kernels of other streams are there
         to use the CUs a small output leaves idle, so the split count is chosen mostly for the
         least CU-time (often no split at all).
         ``residual`` ([m, n], row-strided): added to the bf16-rounded product in the epilogue.
         ``swiglu_out`` ([m, n/2]): also receives silu(out[:, :n/2]) * out[:, n/2:] (layout TN).
-        ``max_cus``: compute-unit budget of the launch (0 = the whole device)."""
+        ``max_cus``: compute-unit budget of the launch (0 = the whole device).
+        ``swiglu_bwd_x`` ([m, 2n], layout NN): the product is the gradient of a SwiGLU output and
+        is not stored; ``out`` ([m, 2n]) receives the gradient of the activation's input instead."""
         self._dev(a, b)
         self._bf16(a, b)
         if a.stride(-1) != 1 or b.stride(-1) != 1:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
         if out is None:
-            out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+            out = torch.empty((m, 2 * n if swiglu_bwd_x is not None else n), dtype=torch.bfloat16, device=a.device)
         epi, aux_ptr, aux_ld, out2_ptr, out2_ld = 0, None, 0, None, 0
+        if swiglu_bwd_x is not None:
+            if residual is not None or swiglu_out is not None or accumulate:
+                raise RuntimeError("one fused epilogue at a time")
+            self._dev(swiglu_bwd_x)
+            self._bf16(swiglu_bwd_x)
+            if tuple(swiglu_bwd_x.shape) != (m, 2 * n) or swiglu_bwd_x.stride(1) != 1 or tuple(out.shape) != (m, 2 * n):
+                raise RuntimeError("swiglu_bwd_x and out must be [M, 2N] with a contiguous last dimension")
+            epi, aux_ptr, aux_ld = 4, swiglu_bwd_x.data_ptr(), swiglu_bwd_x.stride(0)
         if residual is not None:
             self._dev(residual)
             self._bf16(residual)
@@ -205,8 +216,13 @@ class HipBackend:
         """Whether a projection of this output width can produce the SwiGLU activation in its epilogue."""
         return two_f % 2 == 0 and any(two_f % (32 * wn) == 0 for wn in (5, 6, 7, 8))
 
-    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True) -> Tensor:
-        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1], split_k=split_k)
+    def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True, swiglu_bwd_x: Tensor = None) -> Tensor:
+        """``dy . W``; with ``swiglu_bwd_x`` (the input of the SwiGLU activation that fed this layer) the
+        result is the gradient of that input, [rows, 2 * in_features], computed in the GEMM's epilogue."""
+        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1], split_k=split_k,
+                         swiglu_bwd_x=swiglu_bwd_x)
+
+    can_fuse_swiglu_bwd = True
 
     def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False,
                      split_k: bool = True) -> Tensor:

@@ -72,8 +72,9 @@ class LayerConfig:
     # nanobatch outputs (and input gradients) are written into slices of one tensor by the ops
     # that produce them, so joining the nanobatches needs no concatenation
     join_nanobatches_in_place: bool = True
-    # HBM passes folded into GEMM epilogues: the SwiGLU activation into fc1, and (one GPU only: no
-    # sum over ranks has to come first) the residual adds into the out-projection and fc2
+    # HBM passes folded into GEMM epilogues: the SwiGLU activation into fc1, its backward into fc2's
+    # input-gradient GEMM, and (one GPU only: no sum over ranks has to come first) the residual adds
+    # into the out-projection and fc2
     fuse_forward_epilogues: bool = True
     hidden_dropout: float = 0.0
     attention_dropout: float = 0.0
@@ -194,7 +195,8 @@ class DecoderLayer(torch.nn.Module):
         self.linear_fc2 = TERowParallelLinearOp(c.ffn_hidden_size, c.hidden_size, skip_bias_add=True, **lin)
         self.mlp_bda = BiasDropoutAddOp(has_bias=c.add_bias_linear, dropout_prob=c.hidden_dropout, backend=be)
         fuse = bool(getattr(c, "fuse_forward_epilogues", False))
-        self.linear_fc1.fuse_activation = fuse
+        self.linear_fc1.fuse_activation = fuse    # SwiGLU forward in fc1's epilogue
+        self.linear_fc2.fuse_activation = fuse    # SwiGLU backward in the epilogue of fc2's input gradient
         for row_parallel in (self.linear_proj, self.linear_fc2):
             row_parallel.fuse_residual = fuse
             row_parallel.forward_accepts_out_sink = fuse

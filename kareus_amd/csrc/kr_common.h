@@ -51,6 +51,13 @@ __device__ __forceinline__ float wave_max(float v) {
 __device__ __forceinline__ float kr_sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float kr_swiglu_f(float gate, float up) { return gate * kr_sigmoidf(gate) * up; }
 
+// SwiGLU backward on one element: upstream gradient gy, forward inputs (gate, up) -> gradients.
+__device__ __forceinline__ void kr_swiglu_bwd_f(float gy, float gate, float up, float& d_gate, float& d_up) {
+  const float sg = kr_sigmoidf(gate);
+  d_gate = gy * sg * (1.0f + gate * (1.0f - sg)) * up;
+  d_up = gy * gate * sg;
+}
+
 static inline bool kr_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static inline int kr_launch_status() {

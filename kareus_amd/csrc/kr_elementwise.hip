@@ -78,10 +78,10 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16* __rest
     bf16x8 g = ldg8(xr + c), u = ldg8(xr + F + c), d = ldg8(dy + r * F + c), d1, d2;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      float x1 = (float)g[e], x2 = (float)u[e], gy = (float)d[e];
-      float sg = sigmoidf_(x1);
-      d1[e] = (bf16)(gy * sg * (1.0f + x1 * (1.0f - sg)) * x2);
-      d2[e] = (bf16)(gy * x1 * sg);
+      float dg, du;
+      kr_swiglu_bwd_f((float)d[e], (float)g[e], (float)u[e], dg, du);
+      d1[e] = (bf16)dg;
+      d2[e] = (bf16)du;
     }
     stg8(dx + r * 2 * F + c, d1);
     stg8(dx + r * 2 * F + F + c, d2);

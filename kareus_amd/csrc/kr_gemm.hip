@@ -54,7 +54,7 @@ constexpr int TILE = 256 * BK;  // elements of one operand tile (either layout)
 constexpr uint32_t SLOT_BYTES = TILE * sizeof(bf16);
 constexpr int NSLOTS = 5;          // 5 x 32 KB = the whole 160 KB of LDS
 constexpr int kXcds = 8;
-constexpr int KR_GEMM_EPI_TRANSPOSED_OUT = 3;  // internal: not part of the C ABI's epilogue values
+constexpr int KR_GEMM_EPI_TRANSPOSED_OUT = 100;  // internal: not part of the C ABI's epilogue values
 constexpr int kGroupM = 4;
 
 // ---- LDS layouts (element offsets inside one operand tile) ----------------------------------
@@ -225,7 +225,13 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // it with the operands exchanged when the tile grid of the transposed problem fits the device
   // better (256 x 224 tiles can then be 224 rows x 256 columns of the output).
   constexpr bool trans_out = EPI == KR_GEMM_EPI_TRANSPOSED_OUT;
-  static_assert(EPI == KR_GEMM_EPI_NONE || trans_out || (!A_T && !B_T), "fused epilogues: K-major layout only");
+  // SWIGLU_BWD (layout NN, an input gradient): the product is the gradient of the activation's
+  // output; the epilogue reads the activation's input x = [gate | up] for the same rows and
+  // columns and stores the gradient of x instead of the product.
+  constexpr bool swiglu_bwd = EPI == KR_GEMM_EPI_SWIGLU_BWD;
+  static_assert(!swiglu_bwd || (!A_T && B_T), "SwiGLU backward epilogue: layout NN only");
+  static_assert(EPI == KR_GEMM_EPI_NONE || trans_out || swiglu_bwd || (!A_T && !B_T),
+                "residual / SwiGLU epilogues: K-major layout only");
   static_assert(!trans_out || (A_T && B_T), "transposed store: layout NT only");
   constexpr bool epi_add = EPI == KR_GEMM_EPI_ADD;
   constexpr bool swiglu = EPI == KR_GEMM_EPI_SWIGLU;
@@ -542,6 +548,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
       for (int q = 0; q < 4; ++q) nlo[q] = (uint32_t)((4 * q + quad) * ldc + ncol);
       // fused residual: the values to add to a 16-row block are requested one block ahead
+      // SwiGLU backward: gate and up values of a 16-row block, requested one block ahead
+      bf16x8 xg[swiglu_bwd ? 2 : 1][swiglu_bwd ? 4 : 1], xu[swiglu_bwd ? 2 : 1][swiglu_bwd ? 4 : 1];
+      auto fetch_x = [&](int mt) {
+        const bf16* const xb = aux + ((int64_t)(m_wave + mt * 16) * ld_aux + n_wave + 8 * rch);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int rr = 4 * q + quad;
+          const bool in = ncols_in && (rows_in || m_wave + mt * 16 + rr < M);
+          xg[mt & 1][q] = in ? ldg8(xb + (int64_t)rr * ld_aux) : zero8();
+          xu[mt & 1][q] = in ? ldg8(xb + (int64_t)rr * ld_aux + N) : zero8();
+        }
+      };
+      if constexpr (swiglu_bwd) fetch_x(0);
       bf16x8 resv[epi_add ? 2 : 1][epi_add ? 4 : 1];
       auto fetch_res = [&](int mt) {
         const bf16* const rb = aux + ((int64_t)(m_wave + mt * 16) * ld_aux + n_wave + 8 * rch);
@@ -592,6 +611,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         if constexpr (epi_add) {
           if (mt + 1 < WT) fetch_res(mt + 1);
         }
+        if constexpr (swiglu_bwd) {
+          if (mt + 1 < WT) fetch_x(mt + 1);
+        }
         f32x4 vals[WN];  // the only place the accumulators are read
 #pragma unroll
         for (int nt = 0; nt < WN; ++nt) {
@@ -619,7 +641,22 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
               for (int e = 0; e < 8; ++e) v[e] = (bf16)((float)resv[mt & 1][q][e] + (float)v[e]);
             }
-            if (in) stg8(C + blk + nlo[q], v);
+            if constexpr (swiglu_bwd) {
+              bf16x8 d1, d2;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                float dg, du;
+                kr_swiglu_bwd_f((float)v[e], (float)xg[mt & 1][q][e], (float)xu[mt & 1][q][e], dg, du);
+                d1[e] = (bf16)dg;
+                d2[e] = (bf16)du;
+              }
+              if (in) {
+                stg8(C + blk + nlo[q], d1);
+                stg8(C + blk + nlo[q] + N, d2);
+              }
+            } else {
+              if (in) stg8(C + blk + nlo[q], v);
+            }
           }
           if constexpr (swiglu) {
             // the wave beside this one (same rows, other half of the tile) has staged the other
@@ -878,8 +915,13 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   if (fu.max_cus < 0) return KR_EINVAL;
   if (fu.epi != KR_GEMM_EPI_NONE) {
     if (accumulate) return KR_EINVAL;
-    if (layout != KR_GEMM_TN) return KR_EUNSUPPORTED;  // fused epilogues are built for the forward layout
-    if (fu.epi == KR_GEMM_EPI_ADD) {
+    if (fu.epi == KR_GEMM_EPI_SWIGLU_BWD) {
+      if (layout != KR_GEMM_NN) return KR_EUNSUPPORTED;
+      if (!fu.aux || !kr_aligned16(fu.aux) || fu.ld_aux < 2 * (int64_t)N || ldc < 2 * (int64_t)N) return KR_EINVAL;
+      if (fu.ld_aux % 8 || fu.ld_aux >= (int64_t)1 << 26) return KR_EUNSUPPORTED;
+    } else if (layout != KR_GEMM_TN) {
+      return KR_EUNSUPPORTED;  // the other fused epilogues are built for the forward layout
+    } else if (fu.epi == KR_GEMM_EPI_ADD) {
       if (!fu.aux || !kr_aligned16(fu.aux) || fu.ld_aux < N) return KR_EINVAL;
       if (fu.ld_aux % 8 || fu.ld_aux >= (int64_t)1 << 26) return KR_EUNSUPPORTED;
     } else if (fu.epi == KR_GEMM_EPI_SWIGLU) {
@@ -905,6 +947,18 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   }();
   const int cus = fu.max_cus > 0 && fu.max_cus < num_cus ? fu.max_cus : num_cus;
   const int wn = fu.epi == KR_GEMM_EPI_SWIGLU ? swiglu_wn(M, N, cus) : choose_wn(M, N, cus);
+  if (fu.epi == KR_GEMM_EPI_SWIGLU_BWD) {
+    if (lda < K || ldb < N) return KR_EINVAL;
+#define KR_GEMM_SWIGLU_BWD(W) \
+  return launch<false, true, W, KR_GEMM_EPI_SWIGLU_BWD>(a, lda, b, ldb, c, ldc, M, N, K, 0, ws, workspace_bytes, st, num_cus, fu)
+    switch (wn) {
+      case 5: KR_GEMM_SWIGLU_BWD(5);
+      case 6: KR_GEMM_SWIGLU_BWD(6);
+      case 7: KR_GEMM_SWIGLU_BWD(7);
+      default: KR_GEMM_SWIGLU_BWD(8);
+    }
+#undef KR_GEMM_SWIGLU_BWD
+  }
   if (fu.epi != KR_GEMM_EPI_NONE) {
     if (lda < K || ldb < K || ldc < N) return KR_EINVAL;
 #define KR_GEMM_FUSED(W, E) \

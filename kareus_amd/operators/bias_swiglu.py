@@ -14,6 +14,7 @@ from ..partitions.tensor_graph import Channel, PartitionableOperator
 
 class BiasSwigluOp(BasicOperation, PartitionableOperator):
     forward_is_swiglu = True   # a projection in front may compute this activation in its epilogue
+    backward_is_swiglu = True  # ... and the projection behind it its backward, in the input-gradient GEMM
 
     def __init__(self, has_bias: bool = False, fp8_input_store: bool = False, backend="hip") -> None:
         super().__init__()

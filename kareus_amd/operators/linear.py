@@ -144,10 +144,30 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
                                     basic_op_next_ops=[next_op], basic_op_kwargs=[{}])
         return out
 
+    def can_fuse_backward_with(self, next_operator) -> bool:
+        """The backward of the SwiGLU activation that feeds this layer can run in the epilogue of
+        the input-gradient GEMM (the product itself is then never written)."""
+        if not getattr(next_operator, "backward_is_swiglu", False) or not self.fuse_activation:
+            return False
+        return bool(getattr(get_backend(self._backend_name), "can_fuse_swiglu_bwd", False))
+
     def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):
-        dx, param_grads = self.op_backward(basic_op_ctxs[0], grad_output)
-        # the residual input passes the incoming gradient through (out = residual + x . W^T)
-        return dx, [param_grads], [(grad_output,)] if self.fuse_residual else [()]
+        extra = (grad_output,) if self.fuse_residual else ()
+        if len(basic_op_ctxs) == 1:
+            dx, param_grads = self.op_backward(basic_op_ctxs[0], grad_output)
+            # the residual input passes the incoming gradient through (out = residual + x . W^T)
+            return dx, [param_grads], [extra]
+        # [this layer, SwiGLU]: d(activation input) = swiglu_backward(dy . W, x) in one launch
+        # (kareus/megatron/core/extensions/ops/bias_swiglu.py:34-44 behind basic_linear.py:847-859)
+        ctx, act_ctx = basic_op_ctxs
+        (x2d,) = ctx.saved_tensors
+        (act_in,) = act_ctx.saved_tensors
+        n, _k = self.weight.shape
+        dy = self._rows(grad_output.reshape(-1, n))
+        be = get_backend(self._backend_name)
+        dx = be.linear_dgrad(dy, self.weight.detach(), split_k=self.split_k, swiglu_bwd_x=act_in)
+        dw = self._weight_grad(be, ctx, dy, x2d, self.split_k) if self.weight.requires_grad else None
+        return dx.view(act_ctx.ori_shape), [(dw,), ()], [extra, ()]
 
     def op_backward(self, ctx, grad_output):
         (x2d,) = ctx.saved_tensors

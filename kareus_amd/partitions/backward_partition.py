@@ -45,7 +45,7 @@ class BackwardPartition(PartitionBase):
         if offer is None or not offer(nxt.operator):
             return None
         outs, nxt_ins = op.get_output_tensor_ids(), nxt.get_input_tensor_ids()
-        if len(outs) != 1 or not nxt_ins or nxt_ins[0] != outs[0]:
+        if not outs or not nxt_ins or nxt_ins[0] != outs[0]:
             return None
         if not ctx.get_op_context(nxt.op_id).requires_grad:
             return None
@@ -100,11 +100,14 @@ class BackwardPartition(PartitionBase):
             if last == start - 1:
                 self.comm_op.event_record(_current_stream())
 
-            out_ids = group[-1].get_output_tensor_ids()
-            store.set(out_ids[0], dx)
-            if grad_extra_in and grad_extra_in[-1]:
-                for k, tid in enumerate(out_ids[1:]):
-                    g = grad_extra_in[-1][k]
+            store.set(group[-1].get_output_tensor_ids()[0], dx)
+            # gradients of extra inputs: every member of a fused group may have some (a projection
+            # that adds the residual in its epilogue hands the residual's gradient on)
+            for k, member in enumerate(group):
+                extras_k = grad_extra_in[k] if (grad_extra_in and len(grad_extra_in) == len(group)) else (
+                    grad_extra_in[-1] if (grad_extra_in and k == len(group) - 1) else ())
+                for j, tid in enumerate(member.get_output_tensor_ids()[1:]):
+                    g = extras_k[j] if j < len(extras_k) else None
                     if g is not None:
                         store.set(tid, g)
             idx = last + 1

@@ -99,6 +99,11 @@ def test_fused_gemm_argument_checks():
     assert call(1, 16, 256, None, 0, layout=2) == -2
     assert call(2, None, 0, 16, 136, n=272) == -2            # no tile width divides 2F = 272
     assert call(7, None, 0, None, 0) == -1                   # unknown epilogue
+    assert call(4, 16, 512, None, 0, layout=0) == -2         # the SwiGLU backward epilogue belongs to the NN layout
+    assert call(4, None, 512, None, 0, layout=1) == -1       # ... and needs the activation's input
+    assert call(4, 16, 256, None, 0, layout=1) == -1         # ... of twice the product's width
+    assert lib.kr_gemm_bf16_fused(1, 256, 256, 64, 16, 64, 16, 256, 16, 256, 0, 4, 16, 512, None, 0, 0, None, 0,
+                                  None) == -1                # ... and an output of that width
     assert call(0, None, 0, None, 0, cus=-3) == -1
 
 

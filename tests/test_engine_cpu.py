@@ -153,8 +153,15 @@ def test_forward_epilogue_fusions_change_nothing(nnb, recompute, monkeypatch):
     from kareus_amd.operators.linear import PartitionableLinear
 
     x, go, ref = _oracle(layers=2, s=64, b=4)
-    calls = {"pairs": 0, "passed_on": 0}
+    calls = {"pairs": 0, "passed_on": 0, "bwd_pairs": 0}
     real_linear, real_bda = PartitionableLinear.fuser_forward, BiasDropoutAddOp.fuser_forward
+    real_linear_bwd = PartitionableLinear.fuser_backward
+
+    def spy_linear_bwd(self, ctxs, dy, **kw):
+        calls["bwd_pairs"] += len(ctxs) == 2
+        return real_linear_bwd(self, ctxs, dy, **kw)
+
+    monkeypatch.setattr(PartitionableLinear, "fuser_backward", spy_linear_bwd)
 
     def spy_linear(self, ctxs, x_, **kw):
         calls["pairs"] += len(ctxs) == 2
@@ -172,9 +179,10 @@ def test_forward_epilogue_fusions_change_nothing(nnb, recompute, monkeypatch):
         cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager",
                           checkpoint_activations=recompute, fuse_forward_epilogues=fuse)
         model = LayerStack(cfg, seed=1234)
-        calls.update(pairs=0, passed_on=0)
+        calls.update(pairs=0, passed_on=0, bwd_pairs=0)
         y, dx = _run(model, x, go)
         results[fuse] = (y, dx, [p.grad.clone() for p in model.parameters()])
+        assert calls["bwd_pairs"] == (2 * nnb if fuse else 0)     # fc2's backward takes the activation's along
         passes = 2 if recompute else 1                       # the recompute runs the forward again
         assert calls["pairs"] == (2 * nnb * passes if fuse else 0)          # one fc1 per layer and nanobatch
         # two residual adds per layer; the last one of a nanobatch writes into the block's output, and a
@@ -196,7 +204,7 @@ def test_forward_epilogue_fusions_change_nothing(nnb, recompute, monkeypatch):
     for part in model.forward_partitions:
         if part.partition_key == "fwd_mlp":
             part._schedule_config = (("activation_0", "none"), (16, 1024))
-    calls.update(pairs=0, passed_on=0)
+    calls.update(pairs=0, passed_on=0, bwd_pairs=0)
     _check(model, x, go, ref)
     assert calls["pairs"] == (0 if nnb > 1 else 2 * (2 if recompute else 1))   # (one nanobatch: no launch points)
 

@@ -395,3 +395,19 @@ def test_weight_gradient_with_transposed_store(be, m, n, k):
     be.gemm(2, dy, x, m, n, k, out=wide[:, :n], split_k=None)
     assert torch.equal(wide[:, :n], got) and not wide[:, n:].any()
     assert torch.equal(be.linear_wgrad(dy, x, split_k=None), got)
+
+
+@pytest.mark.parametrize("m,f,h", [(512, 128, 256), (264, 520, 200), (4096, 3584, 1024), (1000, 1024, 640), (16384, 72, 3072)])
+def test_input_gradient_with_fused_swiglu_backward_equals_the_two_kernels(be, m, f, h):
+    """fc2's input-gradient GEMM with the SwiGLU backward in its epilogue: dy . W is never written, the
+    gradient of the activation's input comes out of the one launch with the bits of the GEMM followed by
+    kr_swiglu_bwd."""
+    dy, w = rnd(m, h, seed=110), rnd(h, f, scale=0.05, seed=111)        # W_fc2 [hidden, ffn]
+    x = rnd(m, 2 * f, seed=112)                                         # the activation's input (fc1's output)
+    want = be.swiglu_bwd(be.linear_dgrad(dy, w, split_k=None), x)
+    got = be.linear_dgrad(dy, w, swiglu_bwd_x=x)
+    assert got.shape == (m, 2 * f) and torch.equal(got, want)
+    assert rel(got, R.swiglu_bwd_formula(dy.float() @ w.float(), x.float())) <= TOL
+    wide = rnd(m, 2 * f + 16, seed=113)                                 # row-strided activation input
+    assert torch.equal(be.linear_dgrad(dy, w, swiglu_bwd_x=wide[:, :2 * f]),
+                       be.swiglu_bwd(be.linear_dgrad(dy, w, split_k=None), wide[:, :2 * f].contiguous()))

@@ -27,11 +27,12 @@ def _build(dims, layers, nnb, **kw):
                       kv_channels=dims.hd, ffn_hidden_size=dims.ffn, num_layers=layers, num_nanobatches=nnb,
                       backend="hip", **kw)
     model = LayerStack(cfg, device="cuda", seed=1234)
-    # split-K changes the order of the contraction sum; the driver switches it off when nanobatch
-    # streams run side by side, so for bit-exact comparisons across modes it is off everywhere
+    # split-K changes the order of the contraction sum, and which GEMMs split depends on the mode (alone on
+    # the GPU, beside other nanobatch streams, with a fused epilogue — which never splits): for bit-exact
+    # comparisons across modes no GEMM splits
     for layer in model.layers:
         for op in (layer.linear_qkv, layer.linear_proj, layer.linear_fc1, layer.linear_fc2):
-            op.split_k = False
+            op.split_k = None
     return model
 
 
