@@ -218,3 +218,31 @@ def generate_profile_csv(
     fwd, bwd = candidate_points(logs, stage_layers, nanobatches, use_activation_checkpointing,
                                 scale_time_energy, nonpartition)
     return write_profile_csv(output_path, fwd, bwd, P2P_POWER_W[gpu_type], use_activation_checkpointing)
+
+
+def main(argv=None) -> int:
+    """``python -m kareus_amd.profiling.profile_csv --log-dir logs --output profile.csv --num-layers 1``"""
+    import argparse
+
+    ap = argparse.ArgumentParser(prog="python -m kareus_amd.profiling.profile_csv")
+    ap.add_argument("--log-dir", required=True, help="directory with the four partitions' eval logs")
+    ap.add_argument("--output", required=True)
+    ap.add_argument("--num-layers", type=int, required=True)
+    ap.add_argument("--pipeline-parallel-size", type=int, default=1)
+    ap.add_argument("--num-layers-in-first-pipeline-stage", type=int, default=0)
+    ap.add_argument("--num-layers-in-last-pipeline-stage", type=int, default=0)
+    ap.add_argument("--nanobatches", type=int, default=2)
+    ap.add_argument("--gpu-type", default="MI355X")
+    ap.add_argument("--no-activation-checkpointing", action="store_true")
+    ap.add_argument("--no-scale", action="store_true", help="do not multiply time and energy by 1.15")
+    args = ap.parse_args(argv)
+    kept = generate_profile_csv(args.log_dir, args.output, args.num_layers, args.pipeline_parallel_size,
+                                args.num_layers_in_first_pipeline_stage, args.num_layers_in_last_pipeline_stage,
+                                args.nanobatches, args.gpu_type, not args.no_activation_checkpointing,
+                                not args.no_scale)
+    print(f"{args.output}: {kept['forward']} forward and {kept['backward']} backward candidates")
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
