@@ -48,7 +48,9 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // SwiGLU on one element, fp32: silu(gate) * up.  One definition for the stand-alone kernel and the
 // GEMM epilogue that fuses it, so that the two produce the same bits.
-__device__ __forceinline__ float kr_sigmoidf(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// one v_exp_f32 and one v_rcp_f32 (1 ulp each): an IEEE division here is ten instructions per
+// element, which is what a GEMM epilogue that applies the activation spends its time on
+__device__ __forceinline__ float kr_sigmoidf(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 __device__ __forceinline__ float kr_swiglu_f(float gate, float up) { return gate * kr_sigmoidf(gate) * up; }
 
 // SwiGLU backward on one element: upstream gradient gy, forward inputs (gate, up) -> gradients.
