@@ -349,6 +349,15 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
     request(vreq, v_rows4, v_lane_off, tile, VBLK);
     vreq += v_tiles2;
   };
+  // one of a tile's four requests of this wave (i = 0..3); the last one moves on to the next tile
+  auto request_k_part = [&](uint32_t tile, int i) {
+    dma_b128(kreq + i * k_rows4, k_lane_off, tile + (wave + 4 * i) * KBLK);
+    if (i == 3) kreq += k_tiles2;
+  };
+  auto request_v_part = [&](uint32_t tile, int i) {
+    dma_b128(vreq + i * v_rows4, v_lane_off, tile + (wave + 4 * i) * VBLK);
+    if (i == 3) vreq += v_tiles2;
+  };
 
   request_k(kbuf);
   if (nsteps > 1) request_k(kbuf + KTILE);
@@ -426,10 +435,12 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();
 
-    // ---- vector period of tile j: request K(j+2) and V(j+1) (their buffers were last read in
-    // the matrix period that just ended), then the softmax
-    if (j + 2 < nsteps) request_k(kbuf + (j & 1) * KTILE);
-    if (j + 1 < nsteps) request_v(vbuf + ((j + 1) & 1) * VTILE);
+    // ---- vector period of tile j: the softmax, and between its eight groups of exponentials
+    // the eight requests for K(j+2) and V(j+1) (their buffers were last read in the matrix period
+    // that just ended).  Issued back to back the requests hold the wave until the address path
+    // has taken them, which is as long as the softmax itself.
+    const bool want_k = j + 2 < nsteps, want_v = j + 1 < nsteps;
+    const uint32_t k_dst = kbuf + (j & 1) * KTILE, v_dst = vbuf + ((j + 1) & 1) * VTILE;
     {
       const int key0 = key_of(j);
       if (key0 + BKV - 1 > qw0) {
@@ -463,7 +474,13 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
           pb[t][e >> 3][e & 7] = (bf16)pe;
           // eight elements at a time: scheduled freely, all 32 exponent arguments and results
           // would be alive together
-          if ((e & 7) == 7) __builtin_amdgcn_sched_barrier(0);
+          if ((e & 7) == 7) {
+            __builtin_amdgcn_sched_barrier(0);
+            const int c = t * 2 + (e >> 3);   // 0..3
+            if (want_k) request_k_part(k_dst, c);
+            if (want_v) request_v_part(v_dst, c);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       l_run = l_run * alpha + psum;
       if (__any(moved)) {
