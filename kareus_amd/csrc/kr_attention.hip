@@ -36,6 +36,21 @@ __device__ __forceinline__ int xcd_contiguous_id(int pid, int nblocks) {
   return xcd * q + (xcd < r ? xcd : r) + pid / kXcds;
 }
 
+// Workgroup -> (query tile, (batch, head) pair), longest causal rows first.  With fewer than 32
+// tiles per pair an XCD starts its 32 compute units on the longest tiles of `grp` pairs at once,
+// and the short tiles that follow land on the units that finish first.
+__device__ __forceinline__ void longest_first(int lid, int nqt, int total_pairs, int& qt, int& pair) {
+  const int grp = (nqt < 32 && 32 % nqt == 0) ? 32 / nqt : 1;
+  const int span = grp * nqt, base = lid / span, i = lid % span;
+  if ((base + 1) * grp <= total_pairs) {
+    qt = nqt - 1 - i / grp;
+    pair = base * grp + i % grp;
+  } else {  // a last, incomplete group keeps the plain order
+    qt = nqt - 1 - (lid % nqt);
+    pair = lid / nqt;
+  }
+}
+
 // Output staging.  After the MFMAs a lane holds, for its row (lane % 32), groups of four
 // consecutive channels; stored from there an instruction scatters 64 small pieces over 32 rows
 // and the texture-address path takes them one at a time.  Each wave therefore passes its
@@ -140,6 +155,17 @@ static int check_attn_common(int s, int b, int nq, int nkv, int hd) {
 // The MFMA kernels take head dimension 128 and whole 128-row tiles; everything else that passes
 // check_attn_common goes through the general fp32 kernels.
 static bool attn_fast_path(int s, int hd) { return hd == HD && s % BQ == 0; }
+
+static int kr_compute_units() {
+  static const int num_cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return num_cus;
+}
 
 // The kernels keep a sequence stride in 32 bits and build per-lane byte offsets of up to
 // (48 * stride + 128) * 2 from it: strides must be positive and small enough for that.
@@ -549,6 +575,243 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
         (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
+// Ping-pong forward over shared tiles, for launches with enough 256-query tiles to fill the GPU.
+// The two halves of four waves own *different* queries (rows 0..127 and 128..255 of the tile) and
+// walk the *same* 64-key tiles, half 1 one period behind half 0: a K / V tile is fetched once for
+// 256 queries instead of once for 128, there are half as many workgroups to start and to finish,
+// and the halves never have to merge anything.  Periods as above: in each, one half feeds the
+// matrix pipe (P.V of its previous tile, S = Q.K^T of its next) and the other does its softmax;
+// half 0 requests the K tiles during its softmax (K(j+2) while it works on tile j), half 1 the V
+// tiles (V(j+2)).  K(j) is read in periods 2j (half 0) and 2j+1 (half 1), V(j) in 2j+2 and 2j+3;
+// rings of three tiles each give every request three to four periods to land.  Half 0 needs two
+// tiles fewer than half 1 (its rows end 128 earlier) and idles through the last two steps.
+__global__ __launch_bounds__(512, 1) void attn_fwd_sh_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    bf16* __restrict__ o, float* __restrict__ lse, int s, int nq, int nkv, float scale_log2,
+    int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+    int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+    int64_t o_sg, int64_t o_sh) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  constexpr int BQ2 = 256;
+
+  const int half = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+  const int tid = threadIdx.x & 255;
+  const int lane = tid & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nqt = s / BQ2;
+  int qt, pair;
+  longest_first(xcd_contiguous_id(blockIdx.x, gridDim.x), nqt, gridDim.x / nqt, qt, pair);
+  const int head = pair % nq;
+  const int bi = pair / nq;
+  const int per = nq / nkv;
+  const int kvh = head / per, hj = head % per;
+
+  const int q0 = qt * BQ2;
+  const int qw0 = q0 + half * 128 + wave * 32;
+  const int qrow = qw0 + (lane & 31);
+  const bf16* qp = q + (int64_t)bi * q_sb + kvh * q_sg + hj * q_sh + (int64_t)qrow * q_ss;
+  const bf16* kb = k + (int64_t)bi * k_sb + (int64_t)kvh * k_sh;
+  const bf16* vb = v + (int64_t)bi * v_sb + (int64_t)kvh * v_sh;
+
+  bf16x8 qf[HD / 16];
+#pragma unroll
+  for (int kk = 0; kk < HD / 16; ++kk) qf[kk] = ldg8(qp + kk * 16 + h * 8);
+
+  f32x16 oacc[HD / 32];
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int ntiles = (q0 + BQ2) / BKV;                // tiles the workgroup walks (>= 4)
+  const int nmine = (q0 + half * 128 + 128) / BKV;    // tiles with keys this half's rows see
+  constexpr uint32_t KBLK = 1024 + 16, VBLK = 1024 + 64, KTILE = 16 * KBLK, VTILE = 16 * VBLK;
+  const uint32_t kring = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
+  const uint32_t vring = kring + 3 * KTILE;
+  const uint32_t kfrag_lane = (uint32_t)((lane & 15) * KBLK + ((lane >> 4) & 1) * 256 + h * 16);
+  const uint32_t vfrag_lane = (uint32_t)((4 * h + ((lane & 15) >> 2)) * VBLK + ((lane >> 4) & 1) * 32 +
+                                         ((lane & 3) >> 1) * 16 + (lane & 1) * 8);
+
+  // This half's requests: half 0 brings in K tiles, half 1 V tiles; block b of a tile holds its
+  // rows b, b + 16, b + 32, b + 48 and wave w fills blocks w + 4 i.  `req` points at row w of the
+  // next tile to ask for.
+  const int64_t r_ss = half ? v_ss : k_ss;
+  const uint32_t r_blk = half ? VBLK : KBLK, r_tile = half ? VTILE : KTILE;
+  const uint32_t r_ring = half ? vring : kring;
+  const bf16* req = (half ? vb : kb) + (int64_t)wave * r_ss;
+  const int64_t r_next = (int64_t)BKV * r_ss, r_rows4 = 4 * r_ss;
+  const uint32_t r_lane_off = (uint32_t)((lane >> 4) * 16 * (int)r_ss + (lane & 15) * 8) * 2u;
+  auto request_part = [&](uint32_t tile, int i) {
+    dma_b128(req + i * r_rows4, r_lane_off, tile + (wave + 4 * i) * r_blk);
+    if (i == 3) req += r_next;
+  };
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) request_part(r_ring + t * r_tile, i);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  if (half == 1) __syncthreads();  // half 1 starts one period late
+
+  bf16x8 pb[2][2];
+
+  // O^T += V^T . P^T for the tile in ring slot `slot` (pb holds its probabilities)
+  auto pv_step = [&](int slot) {
+    uint32_t va = vring + slot * VTILE + vfrag_lane;
+    asm volatile("" : "+v"(va));
+    auto vfrag = [&](int g, int dt) {
+      union {
+        struct { s16x4 lo, hi; } s;
+        bf16x8 v;
+      } u;
+      const uint32_t a = va + g * 256 + dt * 64;
+      u.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a));
+      u.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((KR_LDS s16x4*)(a + 8 * VBLK));
+      return u.v;
+    };
+    bf16x8 fr[2][HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt) fr[0][dt] = vfrag(0, dt);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if (g + 1 < 4) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) fr[(g + 1) & 1][dt] = vfrag(g + 1, dt);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int dt = 0; dt < HD / 32; ++dt)
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[g & 1][dt], pb[g >> 1][g & 1],
+                                                           oacc[dt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  int slot = 0, slot_prev = 2, slot_req = 2;  // j % 3, (j - 1) % 3, (j + 2) % 3
+  for (int j = 0; j < ntiles; ++j) {
+    // ---- matrix period: O^T += V^T . P^T of tile j-1, then S^T = K . Q^T of tile j
+    f32x16 sacc[2];
+    const bool mine = j < nmine;
+    __builtin_amdgcn_s_setprio(1);
+    if (j > 0 && j - 1 < nmine) pv_step(slot_prev);
+    if (mine) {
+      uint32_t ka = kring + slot * KTILE + kfrag_lane;
+      asm volatile("" : "+v"(ka));
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[t][e] = 0.f;
+      auto kfrag = [&](int t, int kk) { return *(KR_LDS const bf16x8*)(ka + t * 512 + kk * 32); };
+      bf16x8 fr[2][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) fr[0][u] = kfrag(u & 1, u >> 1);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g + 1 < 4) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) fr[(g + 1) & 1][u] = kfrag(u & 1, 2 * (g + 1) + (u >> 1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          sacc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[g & 1][u], qf[2 * g + (u >> 1)],
+                                                                sacc[u & 1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();
+
+    // ---- vector period of tile j: the softmax, and between its four groups of exponentials
+    // this wave's four requests for tile j+2 of its operand (the ring slot was last read two
+    // periods ago).  Half 0 has no request left once it has run out of tiles of its own.
+    const bool want = j + 2 < ntiles;
+    const uint32_t r_dst = r_ring + slot_req * r_tile;
+    if (mine) {
+      const int key0 = j * BKV;
+      if (key0 + BKV - 1 > qw0) {
+        asm volatile("" ::: "memory");  // keeps this a branch: off the diagonal no mask code runs
+        const int lim = qrow - key0 - 4 * h;  // element offsets beyond it are keys after the query
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            if (t * 32 + 8 * (e >> 2) + (e & 3) > lim) sacc[t][e] = -INFINITY;
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);
+      const bool moved = m_new != m_run;
+      m_run = m_new;
+      const float neg_m = -m_ref * scale_log2;
+      float psum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][e], scale_log2, neg_m));
+          psum += pe;
+          pb[t][e >> 3][e & 7] = (bf16)pe;
+          if ((e & 7) == 7) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (want) request_part(r_dst, t * 2 + (e >> 3));
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      l_run = l_run * alpha + psum;
+      if (__any(moved)) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[dt][e] *= alpha;
+      }
+    } else if (want) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) request_part(r_dst, i);
+    }
+    // tile j+1 of this half's operand (requested one step ago) is read from the next period on;
+    // only this period's four requests may stay in flight
+    if (want)
+      __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    __syncthreads();
+    slot_prev = slot;
+    slot = slot == 2 ? 0 : slot + 1;
+    slot_req = slot_req == 2 ? 0 : slot_req + 1;
+  }
+  // last matrix period: the product of the final tile (half 1; half 0 finished two steps ago)
+  if (ntiles - 1 < nmine) {
+    __builtin_amdgcn_s_setprio(1);
+    pv_step(slot_prev);
+    __builtin_amdgcn_s_setprio(0);
+  }
+  if (half == 0) __syncthreads();  // the barrier half 1 spent on starting late
+
+  // No tile is requested any more and K tiles are no longer read: each wave stages its output
+  // rows through 4 KiB of the K ring.
+  const float l_tot = l_run + __shfl_xor(l_run, 32, KR_WAVE);
+  const float inv_l = 1.0f / l_tot;
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + (half * 4 + wave) * 4096, lane);
+  bf16* op = o + (int64_t)bi * o_sb + kvh * o_sg + hj * o_sh + (int64_t)qw0 * o_ss;
+#pragma unroll
+  for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[dt][e] *= inv_l;
+  store_rows_bf16(rs, oacc, 1.0f, op, o_ss);
+  if (h == 0)
+    lse[((int64_t)bi * nq + head) * s + qrow] =
+        (m_run * scale_log2 + __builtin_amdgcn_logf(l_tot)) * kLn2;
+}
+
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* __restrict__ dout,
                                                          const bf16* __restrict__ o,
                                                          const float* __restrict__ lse,
@@ -935,7 +1198,11 @@ __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
 // HALVES = 2: as in the forward kernel, two halves of an 8-wave workgroup own the same 128
 // queries and walk the even / odd key tiles; half 1's dQ partial is added to half 0's through
 // LDS at the end.  Chosen by the host when there are few workgroups.
-template <int HALVES>
+// SHARED (with two halves): the halves own different queries (rows 0..127 and 128..255 of a
+// 256-query tile) and walk the same key tiles, which all eight waves bring in together — half
+// the K / V traffic and half the workgroups of the split form, and nothing to merge.  Chosen
+// when there is such a tile for every compute unit.
+template <int HALVES, bool SHARED>
 __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
@@ -947,15 +1214,23 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
   const int half = HALVES == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
   const int tid = threadIdx.x & 255, lane = tid & 63, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nqt = s / BQ;
+  static_assert(!SHARED || HALVES == 2, "shared tiles need two halves");
+  constexpr int ROWS = SHARED ? 2 * BQ : BQ;  // queries per workgroup
+  const int nqt = s / ROWS;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  const int qt = nqt - 1 - (lid % nqt);
-  const int head = (lid / nqt) % nq;
-  const int bi = lid / (nqt * nq);
+  int qt, pair;
+  if (SHARED) {
+    longest_first(lid, nqt, gridDim.x / nqt, qt, pair);
+  } else {
+    qt = nqt - 1 - (lid % nqt);
+    pair = lid / nqt;
+  }
+  const int head = pair % nq;
+  const int bi = pair / nq;
   const int per = nq / nkv;
   const int kvh = head / per;
-  const int q0 = qt * BQ;
-  const int qw0 = q0 + wave * 32;
+  const int q0 = qt * ROWS;
+  const int qw0 = q0 + (SHARED ? half * BQ : 0) + wave * 32;
   const int qrow = qw0 + (lane & 31);
 
   const bf16* qp = q + ql.at(bi, head, per) + (int64_t)qrow * ql.s_;
@@ -978,13 +1253,17 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
 #pragma unroll
     for (int e = 0; e < 16; ++e) dqacc[dt][e] = 0.f;
 
-  const int ntiles = (q0 + BQ) / (HALVES * BKV);  // key tiles per half (the tile count is even)
-  // K and V tiles go straight from global memory into this half's two LDS stages
-  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + half * 2 * STAGE;
+  // key tiles per half (the tile count is even), or all tiles up to the workgroup's last row
+  const int ntiles = SHARED ? (q0 + ROWS) / BKV : (q0 + BQ) / (HALVES * BKV);
+  auto key_of = [&](int j) { return SHARED ? j * BKV : (HALVES * j + half) * BKV; };
+  // K and V tiles go straight from global memory into two LDS stages: this half's own, or with
+  // shared tiles the workgroup's, half 0 bringing in the K tile and half 1 the V tile
+  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + (SHARED ? 0 : half * 2 * STAGE);
   auto stage_request = [&](int j, int buf) {
-    const int key0 = (HALVES * j + half) * BKV;
-    bt_request(kb + (int64_t)key0 * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
-    bt_request(vb + (int64_t)key0 * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
+    const int key0 = key_of(j);
+    if (!SHARED || half == 0) bt_request(kb + (int64_t)key0 * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
+    if (!SHARED || half == 1)
+      bt_request(vb + (int64_t)key0 * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
   };
   stage_request(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
@@ -993,7 +1272,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
   for (int j = 0; j < ntiles; ++j) {
     const int cur = j & 1;
     if (j + 1 < ntiles) stage_request(j + 1, cur ^ 1);
-    const int key0 = (HALVES * j + half) * BKV;
+    const int key0 = key_of(j);
     if (key0 <= qw0 + 31) {
       // one base register per tile and read direction; everything else is an immediate
       uint32_t k_rows = area + cur * STAGE + bt_rows_lane(lane);
@@ -1046,7 +1325,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     __syncthreads();
   }
 
-  if (HALVES == 2) {  // half 1 -> LDS -> half 0 ([value][wave][lane]; the staging areas are free)
+  if (HALVES == 2 && !SHARED) {  // half 1 -> LDS -> half 0 ([value][wave][lane]; the staging areas are free)
     float* xch = reinterpret_cast<float*>(smem);
     const int slot = wave * 64 + lane;
     if (half == 1) {
@@ -1065,15 +1344,16 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
 
   // output transposition through LDS (behind the 64 KiB hand-over buffer when there are two halves)
   RowStage rs;
-  rs.init(reinterpret_cast<char*>(smem) + (HALVES == 2 ? 64 * 1024 : 0) + wave * 4096, lane);
+  rs.init(reinterpret_cast<char*>(smem) + (SHARED ? half * 16384 : HALVES == 2 ? 64 * 1024 : 0) + wave * 4096, lane);
   store_rows_bf16(rs, dqacc, scale, dq + dql.at(bi, head, per) + (int64_t)qw0 * dql.s_, dql.s_);
 }
 
 #define KR_ATTN_DQ_ARGS                                                                          \
   const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, int, int, \
       int, float, float, QLayout, KLayout, KLayout, QLayout, QLayout
-template __global__ void attn_bwd_dq_kernel<1>(KR_ATTN_DQ_ARGS);
-template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<1, false>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<2, false>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<2, true>(KR_ATTN_DQ_ARGS);
 #undef KR_ATTN_DQ_ARGS
 
 #define KR_ATTN_DKDV_ARGS                                                                          \
@@ -1351,6 +1631,9 @@ __global__ __launch_bounds__(GTHREADS) void attn_general_dq_kernel(
 
 // The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
 // set by the first key tiles (they see every query): two workgroups then share each key tile.
+#ifndef KR_DQ_SHARED_MAX
+#define KR_DQ_SHARED_MAX (1 << 30)
+#endif
 static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <= 2 * 256 ? 2 : 1; }
 
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
@@ -1424,11 +1707,14 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
       e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1>,
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1, false>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2>,
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2, false>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds_dq));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2, true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
     return e;
   }();
   if (attr_status != hipSuccess) return KR_ELAUNCH;
@@ -1457,13 +1743,19 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
 #undef KR_DKDV_LAUNCH
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int dq_blocks = (s / BQ) * nq * b;
-  if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
-    hipLaunchKernelGGL(attn_bwd_dq_kernel<2>, dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
+  if (s % 256 == 0 && dq_blocks / 2 >= kr_compute_units() && dq_blocks <= KR_DQ_SHARED_MAX) {
+    // a 256-query tile for every compute unit: the halves share their K / V tiles
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<2, true>), dim3(dq_blocks / 2), dim3(512), lds_dq, st,
+                       (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
+                       (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
+                       dql);
+  } else if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<2, false>), dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
                        dql);
   } else {
-    hipLaunchKernelGGL(attn_bwd_dq_kernel<1>, dim3(dq_blocks), dim3(256), lds_dq, st,
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<1, false>), dim3(dq_blocks), dim3(256), lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
                        dql);
@@ -1495,6 +1787,18 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
     hipLaunchKernelGGL(attn_general_fwd_kernel, dim3((s + GT - 1) / GT, nq, b), dim3(GTHREADS), 0,
                        (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
                        lse, s, nq, nkv, hd, scale, ql, kl, vl, ol);
+    return kr_launch_status();
+  }
+  if (s % 256 == 0 && (s / 256) * nq * b >= kr_compute_units()) {
+    // enough 256-query tiles for every compute unit: the halves share their K / V tiles
+    constexpr size_t lds_sh = 3 * 16 * ((1024 + 16) + (1024 + 64));  // 100 KiB
+    static const hipError_t attr_sh = hipFuncSetAttribute(
+        (const void*)attn_fwd_sh_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_sh);
+    if (attr_sh != hipSuccess) return KR_ELAUNCH;
+    hipLaunchKernelGGL(attn_fwd_sh_kernel, dim3((s / 256) * nq * b), dim3(512), lds_sh,
+                       (hipStream_t)stream, (const bf16*)q, (const bf16*)k, (const bf16*)v, (bf16*)o,
+                       lse, s, nq, nkv, scale * kLog2e, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh);
     return kr_launch_status();
   }
   // two K and two V tiles of 17 KiB (padded blocks) per half; afterwards the same memory holds
