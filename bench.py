@@ -189,16 +189,22 @@ def _gemm_operands(layout, m, n, k, device):
     return a, b
 
 
-def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False):
+def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False,
+              fused_swiglu_backward=False):
     """Average duration of one launch, HIP events on the stream the kernel is launched on."""
     a, b = _gemm_operands(layout, m, n, k, device)
     out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
     y = torch.empty(m, n // 2, device=device, dtype=torch.bfloat16) if fused_swiglu else None
     r = torch.randn(m, n, device=device).bfloat16() if residual else None
+    # fc1's saved output (gate | up): the epilogue turns the product into its gradient
+    hx = torch.randn(m, 2 * n, device=device).bfloat16() if fused_swiglu_backward else None
     code = {"TN": 0, "NN": 1, "NT": 2}[layout]
 
     def fn():
-        be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=False, swiglu_out=y, residual=r)
+        if hx is not None:
+            be.gemm(code, a, b, m, n, k, split_k=None, swiglu_bwd_x=hx)
+        else:
+            be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=False, swiglu_out=y, residual=r)
 
     for _ in range(5):
         fn()
@@ -249,7 +255,8 @@ def dominant_kernel_roofline(w, nnb, device, launches=30):
 def gemm_kernels(w, nnb, device, launches=30):
     """Every GEMM of the layer alone on the GPU at the nanobatch shape, the way the engine launches
     it (forward of fc1 with the SwiGLU epilogue, of the out-projection and fc2 with the residual
-    epilogue, weight gradients accumulating into an existing buffer): TFLOP/s against the peak."""
+    epilogue, fc2's input gradient with the SwiGLU-backward epilogue, weight gradients also
+    accumulating into an existing buffer): TFLOP/s against the peak."""
     from kareus_amd.backend import get_backend
 
     be = get_backend("hip")
@@ -261,7 +268,7 @@ def gemm_kernels(w, nnb, device, launches=30):
         variants = [
             ("forward", "TN", t, n_out, k_in, dict(fused_swiglu=name == "fc1" and be.can_fuse_swiglu(n_out),
                                                     residual=name in ("proj", "fc2"))),
-            ("input gradient", "NN", t, k_in, n_out, {}),
+            ("input gradient", "NN", t, k_in, n_out, dict(fused_swiglu_backward=True) if name == "fc2" else {}),
             ("weight gradient", "NT", n_out, k_in, t, {}),
             ("weight gradient, accumulating", "NT", n_out, k_in, t, dict(accumulate=True)),
         ]
