@@ -195,7 +195,7 @@ struct Frags {
 template <int N>
 struct Count { static constexpr int value = N; };
 
-// WN: 16-column MFMA tiles per wave along N (5..8): the workgroup's tile is 256 x 32 * WN.  Narrower
+// WN: 16-column MFMA tiles per wave along N (4..8): the workgroup's tile is 256 x 32 * WN.  Narrower
 // tiles let the host avoid a mostly empty last round of workgroups or a mostly padded last tile
 // column; a K-major B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
 // EPI: the fused epilogue compiled into this instance (KR_GEMM_EPI_*).  A template parameter, not
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
         if (nt == 0) nxt.a[g] = read_a(aa, g, h);
         if (nt == 2 && g < WN) nxt.b[g] = read_b(ba, g, h);
         if constexpr (DMA > 0) {
-          if (nt == 4 && g < DMA) {
+          if (nt == (WN > 4 ? 4 : 3) && g < DMA) {
             if (g == 0) dma_b128<0 * 4096>(dbase, doff[0], dst);
             if (g == 1) dma_b128<1 * 4096>(dbase, doff[1], dst);
             if (g == 2) dma_b128<2 * 4096>(dbase, doff[2], dst);
@@ -740,50 +740,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   stg8(dst, o);
 }
 
-// How many ways to cut the contraction when the output has too few tiles to occupy the GPU.
-// 1 = no split.  Two estimates, in units of one K-step of one workgroup (~1.5 us):
-//   latency  rounds of work items over the CUs, each item paying its K-steps plus a fixed
-//            prologue/epilogue, plus the traffic of the fp32 partial tiles (written once, read
-//            once by the reduce kernel at ~5 TB/s);
-//   CU-time  the same work summed over the CUs it occupies, per CU of the device.
-// A GEMM that has the GPU to itself wants the smallest latency (latency_weight 1); one that
-// runs beside kernels of other streams, which can use the CUs it leaves idle, should mostly
-// keep its CU-time small (latency_weight ~0.3).
-inline int choose_splits(int M, int N, int K, float latency_weight) {
-  constexpr int kCus = 256, kItemOverhead = 4;
-  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  if (tiles >= 192) return 1;
-  const double w = latency_weight < 0.f ? 0.0 : (latency_weight > 1.f ? 1.0 : (double)latency_weight);
-  const int nk = (K + BK - 1) / BK;
-  const double reduce_per_split = (double)M * N * 8.0 / 5.0e12 / 1.5e-6;
-  auto cost = [&](int sp) {
-    const int items = tiles * sp, rounds = (items + kCus - 1) / kCus;
-    const int per_item = (nk + sp - 1) / sp + kItemOverhead;
-    const double reduce = sp > 1 ? sp * reduce_per_split : 0.0;
-    const double latency = (double)rounds * per_item + reduce;
-    const double cu_time = (double)items * per_item / kCus + reduce;
-    return w * latency + (1.0 - w) * cu_time;
-  };
-  int best = 1;
-  double best_cost = cost(1);
-  for (int sp = 2; sp <= 16 && nk / sp >= 8; ++sp) {
-    const double c = cost(sp);
-    if (c < best_cost * 0.95) {  // a split must pay for itself clearly
-      best_cost = c;
-      best = sp;
-    }
-  }
-  return best;
-}
-
-// Tile width for an output that is not split along K: 32 * WN columns, WN in 5..8.  The estimate is
-// the launch's own latency — rounds of tiles over the CUs times the cost of a tile (WN units of
-// MFMA work plus about one unit of prologue and epilogue); ties go to the wider tile, which reads
-// less from LDS per FLOP.  Outputs with fewer than 192 full-width tiles keep the full width (they
-// are candidates for split-K, whose cost model assumes it).
+// Tile width for an output with enough tiles to occupy the GPU without a split: 32 * WN columns,
+// WN in 5..8.  The estimate is the launch's own latency — rounds of tiles over the CUs times the
+// cost of a tile (WN units of MFMA work plus about one unit of prologue and epilogue); ties go to
+// the wider tile, which reads less from LDS per FLOP.
 inline int choose_wn(int M, int N, int num_cus) {
   const int tiles_m = (M + BM - 1) / BM;
-  if (tiles_m * ((N + BN - 1) / BN) < 192) return 8;
   int best = 8;
   long best_cost = 0;
   for (int wn = 8; wn >= 5; --wn) {
@@ -794,6 +756,59 @@ inline int choose_wn(int M, int N, int num_cus) {
       best_cost = cost;
     }
   }
+  return best;
+}
+
+// Tile width and number of cuts of the contraction.  An output of at least 192 full-width tiles is
+// never cut and takes the width of choose_wn.  A smaller one has too few tiles to occupy the GPU:
+// narrower tiles (down to 128 columns; 160 with a fused epilogue) and cuts of the contraction both
+// make more work items, and the pair with the least estimated cost wins.  Two estimates, in units of one K-step of a full-width tile (~1.3 us;
+// a tile of WN columns takes (WN + 2) / 10 of it):
+//   latency  rounds of work items over the CUs, each item paying its K-steps plus a fixed
+//            prologue/epilogue, plus the traffic of the fp32 partial tiles (written once, read
+//            once by the reduce kernel at ~5 TB/s);
+//   CU-time  the same work summed over the CUs it occupies, per CU of the device.
+// A GEMM that has the GPU to itself wants the smallest latency (latency_weight 1); one that
+// runs beside kernels of other streams, which can use the CUs it leaves idle, should mostly
+// keep its CU-time small (latency_weight ~0.3).  `max_splits` is what the caller's workspace holds.
+struct Plan {
+  int wn, splits;
+};
+inline Plan choose_plan(int M, int N, int K, float latency_weight, int num_cus, int max_splits,
+                        int min_wn = 4) {
+  constexpr int kItemOverhead = 4;
+  const int tiles_m = (M + BM - 1) / BM;
+  if (tiles_m * ((N + BN - 1) / BN) >= 192) return {choose_wn(M, N, num_cus), 1};
+  const double w = latency_weight < 0.f ? 0.0 : (latency_weight > 1.f ? 1.0 : (double)latency_weight);
+  const int nk = (K + BK - 1) / BK;
+  const double reduce_per_split = (double)M * N * 8.0 / 5.0e12 / 1.3e-6;
+  auto cost = [&](int wn, int sp) {
+    const int tiles = tiles_m * ((N + 32 * wn - 1) / (32 * wn));
+    const int items = tiles * sp, rounds = (items + num_cus - 1) / num_cus;
+    const double per_item = (double)((nk + sp - 1) / sp) * (wn + 2) / 10.0 + kItemOverhead;
+    const double reduce = sp > 1 ? sp * reduce_per_split : 0.0;
+    const double latency = rounds * per_item + reduce;
+    const double cu_time = items * per_item / num_cus + reduce;
+    return w * latency + (1.0 - w) * cu_time;
+  };
+  Plan best{8, 1};
+  double best_cost = cost(8, 1);
+  for (int wn = 7; wn >= min_wn; --wn) {
+    const double c = cost(wn, 1);
+    if (c < best_cost) {
+      best_cost = c;
+      best = {wn, 1};
+    }
+  }
+  const double unsplit = best_cost;
+  for (int sp = 2; sp <= 16 && sp <= max_splits && nk / sp >= 8; ++sp)
+    for (int wn = 8; wn >= min_wn; --wn) {
+      const double c = cost(wn, sp);
+      if (c < unsplit * 0.95 && c < best_cost) {  // a split must pay for itself clearly
+        best_cost = c;
+        best = {wn, sp};
+      }
+    }
   return best;
 }
 
@@ -827,7 +842,7 @@ inline int swiglu_wn(int M, int N, int num_cus) {
 template <bool A_T, bool B_T, int WN, int EPI = KR_GEMM_EPI_NONE>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
-           hipStream_t stream, int num_cus, const Fused& fu) {
+           hipStream_t stream, int num_cus, const Fused& fu, int planned_splits = 1) {
   constexpr size_t lds_bytes = NSLOTS * TILE * sizeof(bf16);
   // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
   static const hipError_t attr_status =
@@ -836,9 +851,8 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   if (attr_status != hipSuccess) return KR_ELAUNCH;
   if (fu.max_cus > 0 && fu.max_cus < num_cus) num_cus = fu.max_cus;
   const int tiles = ((M + BM - 1) / BM) * ((N + 32 * WN - 1) / (32 * WN));
-  // the latency-optimal count, capped by what the caller's workspace holds (a caller that wants
-  // fewer splits says so by passing the smaller workspace kr_gemm_workspace_bytes_shared sizes)
-  int splits = WN == 8 ? choose_splits(M, N, K, 1.f) : 1;
+  // the planned count, which the dispatcher has already capped by what the caller's workspace holds
+  int splits = planned_splits;
   const size_t one = (size_t)M * N * sizeof(float);
   if (workspace == nullptr || EPI != KR_GEMM_EPI_NONE) {
     splits = 1;  // a fused epilogue works on finished sums
@@ -880,20 +894,31 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   return kr_launch_status();
 }
 
+int device_compute_units() {
+  static const int num_cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return num_cus;
+}
+
 }  // namespace
 
 extern "C" size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K) {
   (void)layout;
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const int splits = choose_splits(M, N, K, 1.f);
+  const int splits = choose_plan(M, N, K, 1.f, 256, 16).splits;
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
 
 extern "C" size_t kr_gemm_workspace_bytes_shared(int layout, int M, int N, int K, float latency_weight) {
   (void)layout;
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  int splits = choose_splits(M, N, K, latency_weight);
-  const int cap = choose_splits(M, N, K, 1.f);
+  int splits = choose_plan(M, N, K, latency_weight, 256, 16).splits;
+  const int cap = choose_plan(M, N, K, 1.f, 256, 16).splits;
   if (splits > cap) splits = cap;
   return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
 }
@@ -938,15 +963,20 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   bf16* c = (bf16*)C;
   float* ws = (float*)workspace;
   hipStream_t st = (hipStream_t)stream;
-  static const int num_cus = [] {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      n = 256;
-    return n;
-  }();
+  const int num_cus = device_compute_units();
   const int cus = fu.max_cus > 0 && fu.max_cus < num_cus ? fu.max_cus : num_cus;
-  const int wn = fu.epi == KR_GEMM_EPI_SWIGLU ? swiglu_wn(M, N, cus) : choose_wn(M, N, cus);
+  // cuts of the contraction the caller's workspace can hold (a caller that wants fewer says so by
+  // passing the smaller workspace kr_gemm_workspace_bytes_shared sizes); a fused epilogue works on
+  // finished sums and is never cut
+  int max_splits = 1;
+  if (ws != nullptr && fu.epi == KR_GEMM_EPI_NONE) {
+    const size_t held = workspace_bytes / ((size_t)M * N * sizeof(float));
+    max_splits = held > 16 ? 16 : (int)held;
+    if (max_splits < 1) max_splits = 1;
+  }
+  const Plan plan = choose_plan(M, N, K, 1.f, cus, max_splits, fu.epi == KR_GEMM_EPI_NONE ? 4 : 5);
+  const int wn = fu.epi == KR_GEMM_EPI_SWIGLU ? swiglu_wn(M, N, cus) : plan.wn;
+  const int sp = plan.splits;
   if (fu.epi == KR_GEMM_EPI_SWIGLU_BWD) {
     if (lda < K || ldb < N) return KR_EINVAL;
 #define KR_GEMM_SWIGLU_BWD(W) \
@@ -981,10 +1011,11 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   }
 #define KR_GEMM_LAUNCH(AT, BT)                                                                           \
   switch (wn) {                                                                                          \
-    case 5: return launch<AT, BT, 5>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
-    case 6: return launch<AT, BT, 6>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
-    case 7: return launch<AT, BT, 7>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
-    default: return launch<AT, BT, 8>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu); \
+    case 4: return launch<AT, BT, 4>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu, sp); \
+    case 5: return launch<AT, BT, 5>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu, sp); \
+    case 6: return launch<AT, BT, 6>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu, sp); \
+    case 7: return launch<AT, BT, 7>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu, sp); \
+    default: return launch<AT, BT, 8>(a, lda, b, ldb, c, ldc, M, N, K, accumulate, ws, workspace_bytes, st, num_cus, fu, sp); \
   }
   switch (layout) {
     case KR_GEMM_TN:  // A [M,K], B [N,K]

@@ -162,7 +162,11 @@ SHAPES = [(256, 256, 64), (512, 768, 512), (264, 520, 200), (1024, 2752, 512), (
           # outputs of 192 tiles or more, where the library picks narrower tiles than 256 columns:
           (4096, 3584, 128),    # 224 columns (16 x 16 tiles fill one round of workgroups)
           (16384, 768, 64),     # 192 columns
-          (16384, 640, 72)]     # 160 columns, and a contraction tail
+          (16384, 640, 72),     # 160 columns, and a contraction tail
+          # outputs of fewer than 192 full tiles, where narrower tiles and cuts of the contraction compete:
+          (4096, 1536, 4096),   # forward: 128-column tiles uncut; the other two layouts take other plans
+          (4088, 1000, 2056),   # the same with ragged edges in all three dimensions
+          (1536, 4096, 1024)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -171,6 +175,23 @@ def test_gemm_three_layouts(be, m, n, k):
     assert rel(be.linear_fwd(x, w), x.float() @ w.float().t()) <= TOL
     assert rel(be.linear_dgrad(dy, w), dy.float() @ w.float()) <= TOL
     assert rel(be.linear_wgrad(dy, x), dy.float().t() @ x.float()) <= TOL
+
+
+def test_gemm_plan_does_not_change_the_sums_much(be):
+    """The library picks tile width and cuts of the contraction by a cost model that depends on the
+    workspace it is given (alone on the GPU: cuts allowed; beside other streams: fewer or none; never:
+    no workspace).  All plans compute the same sums, up to the rounding of a cut's fp32 partial tiles."""
+    for (m, n, k) in [(4096, 1536, 4096), (4096, 1024, 4096), (1536, 4096, 4096), (520, 264, 8192)]:
+        x, w, dy, xx = rnd(m, k, seed=31), rnd(n, k, scale=0.05, seed=32), rnd(k, m, scale=0.1, seed=33), rnd(k, n, seed=34)
+        for layout, a, b, ref in ((0, x, w, x.float() @ w.float().t()), (1, x, w.t().contiguous(), x.float() @ w.float().t()),
+                                  (2, dy, xx, dy.float().t() @ xx.float())):
+            outs = [be.gemm(layout, a, b, m, n, k, split_k=mode) for mode in (True, False, None)]
+            for o in outs:
+                assert rel(o, ref) <= TOL
+            assert rel(outs[0], outs[2]) <= 1e-2 and rel(outs[1], outs[2]) <= 1e-2
+            c0 = rnd(m, n, seed=35)
+            acc = be.gemm(layout, a, b, m, n, k, out=c0.clone(), accumulate=True, split_k=None)
+            assert rel(acc, ref + c0.float()) <= TOL
 
 
 def test_gemm_is_reproducible(be):
