@@ -77,6 +77,12 @@ int kr_gemm_bf16(int layout, int M, int N, int K,
  *                       fused_swiglu_backward(bf16(g), x) (bias_swiglu.py:34-44); bit-identical to
  *                       kr_gemm_bf16 + kr_swiglu_bwd.
  *   ADD and SWIGLU need layout TN, SWIGLU_BWD layout NN; all need accumulate == 0 and are never split-K.
+ *   KR_GEMM_BESIDE_OTHER_STREAMS  a flag, or-ed to any of the above: kernels of other streams are
+ *                       there to use the compute units this launch leaves idle, so an output with few
+ *                       tiles keeps its wide tiles and is cut little or not at all (least compute-unit
+ *                       time) instead of being spread over the device for the shortest latency; pass
+ *                       the workspace kr_gemm_workspace_bytes_shared sizes.  Results do not depend on it
+ *                       beyond the rounding of a cut's fp32 partial sums.
  * max_cus > 0 limits the launch to that many compute units (workgroups are persistent, one per
  * unit): the compute-unit share a schedule's resource_shape gives a partition
  * (kareus/megatron/core/partitions/partition_base.py:117-128); 0 = the whole device.             */
@@ -84,6 +90,7 @@ int kr_gemm_bf16(int layout, int M, int N, int K,
 #define KR_GEMM_EPI_ADD 1
 #define KR_GEMM_EPI_SWIGLU 2
 #define KR_GEMM_EPI_SWIGLU_BWD 4
+#define KR_GEMM_BESIDE_OTHER_STREAMS 0x100
 int kr_gemm_bf16_fused(int layout, int M, int N, int K,
                        const void* A, int64_t lda, const void* B, int64_t ldb,
                        void* C, int64_t ldc, int accumulate,

@@ -181,7 +181,8 @@ class HipBackend:
                 raise RuntimeError("swiglu_out must be [M, N/2] with a contiguous last dimension")
             epi, out2_ptr, out2_ld = 2, swiglu_out.data_ptr(), swiglu_out.stride(0)
         ws_bytes, ws_ptr = 0, None
-        if epi == 0 and split_k is not None:   # split_k=None: never split (no workspace is handed over)
+        fused = epi != 0
+        if not fused and split_k is not None:   # split_k=None: never split (no workspace is handed over)
             key = (layout, m, n, k, split_k)
             ws_bytes = self._gemm_ws_bytes.get(key)
             if ws_bytes is None:
@@ -194,6 +195,8 @@ class HipBackend:
             reserved = reserved_compute_units()
             if reserved:
                 max_cus = max(self._num_cus(a.device) - reserved, 8)
+        if split_k is False:
+            epi |= 0x100   # KR_GEMM_BESIDE_OTHER_STREAMS
         if epi == 0 and max_cus == 0:
             rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
                                        out.data_ptr(), out.stride(0), int(accumulate), ws_ptr, ws_bytes,
@@ -203,7 +206,7 @@ class HipBackend:
                                              b.stride(0), out.data_ptr(), out.stride(0), int(accumulate),
                                              epi, aux_ptr, aux_ld, out2_ptr, out2_ld, int(max_cus),
                                              ws_ptr, ws_bytes, self._stream())
-        self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k}, epilogue={epi})")
+        self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k}, epilogue={epi & 0xff})")
         return out
 
     def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True, out: Tensor = None,

@@ -819,6 +819,7 @@ struct Fused {
   bf16* out2 = nullptr;
   int64_t ld_out2 = 0;
   int max_cus = 0;          // > 0: use at most this many compute units
+  bool shared = false;      // other streams' kernels use the units this launch leaves idle
 };
 
 // Tile width for a projection with the SwiGLU epilogue: the tiles have to divide the 2F output
@@ -974,7 +975,8 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
     max_splits = held > 16 ? 16 : (int)held;
     if (max_splits < 1) max_splits = 1;
   }
-  const Plan plan = choose_plan(M, N, K, 1.f, cus, max_splits, fu.epi == KR_GEMM_EPI_NONE ? 4 : 5);
+  // beside other streams the compute-unit time of the launch counts, hardly its latency
+  const Plan plan = choose_plan(M, N, K, fu.shared ? 0.1f : 1.f, cus, max_splits, fu.epi == KR_GEMM_EPI_NONE ? 4 : 5);
   const int wn = fu.epi == KR_GEMM_EPI_SWIGLU ? swiglu_wn(M, N, cus) : plan.wn;
   const int sp = plan.splits;
   if (fu.epi == KR_GEMM_EPI_SWIGLU_BWD) {
@@ -1074,7 +1076,8 @@ extern "C" int kr_gemm_bf16_fused(int layout, int M, int N, int K, const void* A
                                   int64_t ld_out2, int max_cus, void* workspace,
                                   size_t workspace_bytes, void* stream) {
   Fused fu;
-  fu.epi = epilogue;
+  fu.epi = epilogue & ~KR_GEMM_BESIDE_OTHER_STREAMS;
+  fu.shared = (epilogue & KR_GEMM_BESIDE_OTHER_STREAMS) != 0;
   fu.aux = (const bf16*)aux;
   fu.ld_aux = ld_aux;
   fu.out2 = (bf16*)out2;
