@@ -190,7 +190,7 @@ def _gemm_operands(layout, m, n, k, device):
 
 
 def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False,
-              fused_swiglu_backward=False):
+              fused_swiglu_backward=False, alone=False):
     """Average duration of one launch, HIP events on the stream the kernel is launched on."""
     a, b = _gemm_operands(layout, m, n, k, device)
     out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
@@ -204,7 +204,7 @@ def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, resi
         if hx is not None:
             be.gemm(code, a, b, m, n, k, split_k=None, swiglu_bwd_x=hx)
         else:
-            be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=False, swiglu_out=y, residual=r)
+            be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=alone, swiglu_out=y, residual=r)
 
     for _ in range(5):
         fn()
@@ -252,11 +252,35 @@ def dominant_kernel_roofline(w, nnb, device, launches=30):
     return main, others
 
 
-def gemm_kernels(w, nnb, device, launches=30):
+def time_library_matmul(layout, m, n, k, device, launches=30):
+    """The same product through ``torch.matmul`` (the vendor's GEMM library), same operands and
+    layout, plain store: a yardstick for the kernel, not part of the step."""
+    a, b = _gemm_operands(layout, m, n, k, device)
+    out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
+    lhs = a.t() if layout == "NT" else a
+    rhs = b.t() if layout == "TN" else b
+
+    def fn():
+        torch.matmul(lhs, rhs, out=out)
+
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(launches):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / launches
+
+
+def gemm_kernels(w, nnb, device, launches=30, with_library=False):
     """Every GEMM of the layer alone on the GPU at the nanobatch shape, the way the engine launches
     it (forward of fc1 with the SwiGLU epilogue, of the out-projection and fc2 with the residual
     epilogue, fc2's input gradient with the SwiGLU-backward epilogue, weight gradients also
-    accumulating into an existing buffer): TFLOP/s against the peak."""
+    accumulating into an existing buffer; planned for the launch's own latency with one nanobatch,
+    for compute-unit time beside the other streams of several): TFLOP/s against the peak."""
     from kareus_amd.backend import get_backend
 
     be = get_backend("hip")
@@ -273,11 +297,13 @@ def gemm_kernels(w, nnb, device, launches=30):
             ("weight gradient, accumulating", "NT", n_out, k_in, t, dict(accumulate=True)),
         ]
         for what, layout, m, n, k, kw in variants:
-            sec = time_gemm(be, layout, m, n, k, device, launches, **kw)
+            sec = time_gemm(be, layout, m, n, k, device, launches, alone=nnb == 1, **kw)
             flops = 2.0 * m * n * k
             rows.append({"gemm": f"{name} {what}", "layout": layout, "shape": [m, n, k], "epilogue": kw,
                          "avg_launch_us": sec * 1e6, "TFLOPs": flops / sec / 1e12,
                          "frac_of_peak": flops / sec / MFMA_PEAK_BF16})
+            if with_library and not kw.get("accumulate"):
+                rows[-1]["library_matmul_us"] = time_library_matmul(layout, m, n, k, device, launches) * 1e6
     return rows
 
 
@@ -616,6 +642,8 @@ def main():
                     help="run only the attention forward/backward stand-alone (TFLOP/s against the MFMA peak)")
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
+    ap.add_argument("--with-library-matmul", action="store_true",
+                    help="with --gemm-kernels: also time torch.matmul on the plain GEMMs, as a yardstick")
     ap.add_argument("--gemm-kernels", action="store_true",
                     help="run only the layer's twelve GEMMs stand-alone at nanobatch shape, as the engine launches them")
     ap.add_argument("--cu-budget-sweep", action="store_true",
@@ -650,7 +678,7 @@ def main():
         print(json.dumps({"hbm_kernels": hbm_kernels(w, w["nnb"], device)}))
         return
     if args.gemm_kernels:
-        print(json.dumps({"gemm_kernels": gemm_kernels(w, w["nnb"], device)}))
+        print(json.dumps({"gemm_kernels": gemm_kernels(w, w["nnb"], device, with_library=args.with_library_matmul)}))
         return
     if args.cu_budget_sweep:
         print(json.dumps({"cu_budget_sweep_ms_per_step": cu_budget_sweep(w, device)}))
