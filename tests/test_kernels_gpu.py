@@ -250,7 +250,9 @@ def _grouped(s, b, nq, nkv, hd, seed):
                                         # enough 256-query tiles for every compute unit: the forward kernel whose halves share K / V tiles
                                         (1024, 8, 8, 2),    # 4 tiles x 64 (batch, head) pairs, eight pairs start together on an XCD
                                         (768, 11, 8, 8),    # 3 tiles per pair: plain longest-first order
-                                        (512, 33, 8, 2)])   # 2 tiles per pair, 264 pairs: the last group of 16 pairs is incomplete
+                                        (512, 33, 8, 2),    # 2 tiles per pair, 264 pairs: the last group of 16 pairs is incomplete
+                                        (2304, 4, 8, 2),    # 9 tiles per pair: an odd tile count, half 0 idles through two steps of 36
+                                        (512, 6, 24, 8)])   # three query heads per KV head in the shared-tile kernels
 def test_attention_forward_backward(be, s, b, nq, nkv):
     hd = 128
     _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=22)
