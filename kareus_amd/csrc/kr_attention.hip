@@ -866,7 +866,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ neg_lse2, const float* __restrict__ delta,
     bf16* __restrict__ dk, bf16* __restrict__ dv, float* __restrict__ part_k,
-    float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, float scale, float scale_log2,
+    float* __restrict__ part_v, int s, int nq, int nkv, int qsplit, int hpw, float scale, float scale_log2,
     QLayout ql, KLayout kl, KLayout vl, QLayout dol, KLayout dkl, KLayout dvl) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   // stage layout: Q tile | dO tile (blocked tiles) | lse[64] fp32 | delta[64] fp32
@@ -882,16 +882,23 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
   const int nkt = s / 128;
   const int lid_all = xcd_contiguous_id(blockIdx.x, gridDim.x);
   const int part = lid_all % qsplit, lid = lid_all / qsplit;
+  // A workgroup takes `hpw` consecutive query heads of one KV group, one after the other: its K / V
+  // fragments and its dK / dV accumulators serve them all, so a group leaves per / hpw partial
+  // results instead of per (none at all when hpw = per), and the workgroup's start and end are
+  // paid once for hpw heads.  The host picks hpw so that enough workgroups remain.
   const int kt = lid % nkt;  // low key tiles see the most queries: they come first
-  const int head = (lid / nkt) % nq;
-  const int bi = lid / (nkt * nq);
+  const int nhg = nq / hpw;
+  const int hgroup = (lid / nkt) % nhg;
+  const int head = hgroup * hpw;  // the first of this workgroup's heads
+  const int bi = lid / (nkt * nhg);
   const int per = nq / nkv;
   const int kvh = head / per;
   const int key0 = kt * 128;
   const int kw0 = key0 + wave * 32;
   const int krow = kw0 + (lane & 31);
   const int qt_first = key0 / 64;
-  const int niter = (s / 64 - qt_first - part + qsplit - 1) / qsplit;  // this part's query tiles of 64
+  const int niter = (s / 64 - qt_first - part + qsplit - 1) / qsplit;  // this part's query tiles of 64, per head
+  const int nit_all = niter * hpw;                                       // ... over all heads of the workgroup
   const uint32_t lds0 = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
   const uint32_t xch_lane = lds0 + XCH + wave * 4096 + lane * 16;  // + parity * 16384 + slot * 1024
 
@@ -996,9 +1003,10 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
     // stage is read, unused).
     f32x16 s0, dp0, s1, dp1;
     issue_scores(0, 0, s0, dp0);
-    for (int it = 0; it < niter; ++it) {
+    for (int it = 0, itl = 0; it < nit_all; ++it) {
       const int stage = it % NS;
-      const int q0 = (qt_first + it * qsplit + part) * 64;
+      const int q0 = (qt_first + itl * qsplit + part) * 64;
+      itl = itl + 1 == niter ? 0 : itl + 1;  // the next head starts over at the diagonal
       step(stage, 0, q0, s0, dp0, stage, 1, s1, dp1);
       __syncthreads();  // hand-over of block 0
       step(stage, 1, q0 + 32, s1, dp1, (it + 1) % NS, 0, s0, dp0);
@@ -1017,17 +1025,23 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
   // request_piece(i) issues piece i = 0..8, in this order (requests retire in order).
   uint32_t req_tile = 0, req_lane_off = 0;
   const bf16* req_row = nullptr;
+  const bf16 *req_q = qb, *req_do = dob;
+  int64_t req_stat = stat0;
   int req_qt = 0;
   auto request_begin = [&](int it) {
-    req_qt = qt_first + it * qsplit + part;
+    const int hh = it / niter, itl = it - hh * niter;  // head of the workgroup, query tile of that head
+    req_qt = qt_first + itl * qsplit + part;
     req_tile = lds0 + (it % NS) * STAGE;
+    req_q = qb + hh * ql.h_;    // consecutive heads of one KV group
+    req_do = dob + hh * dol.h_;
+    req_stat = stat0 + (int64_t)hh * s;
   };
   auto request_piece = [&](int i) {
     if (i == 0) {
       if (wave < 2) {
         int l2 = lane;
         asm volatile("" : "+v"(l2));
-        dma_b32((wave == 0 ? neg_lse2 : delta) + stat0 + req_qt * 64, (uint32_t)l2 * 4u,
+        dma_b32((wave == 0 ? neg_lse2 : delta) + req_stat + req_qt * 64, (uint32_t)l2 * 4u,
                 req_tile + 2 * BT_BYTES + wave * 256);
       }
       return;
@@ -1039,7 +1053,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
       asm volatile("" : "+v"(l2));  // the lane offset lives only across the four requests of a tile
       const int64_t ss = second ? dol.s_ : ql.s_;
       req_lane_off = (uint32_t)((l2 >> 4) * 16 * (int)ss + (l2 & 15) * 8) * 2u;
-      req_row = (second ? dob : qb) + ((int64_t)req_qt * 64 + 4 * wave) * ss;
+      req_row = (second ? req_do : req_q) + ((int64_t)req_qt * 64 + 4 * wave) * ss;
     }
     dma_b128(req_row, req_lane_off, req_tile + (second ? BT_BYTES : 0) + (wave + 4 * j) * BT_BLK);
     req_row += second ? dol.s_ : ql.s_;
@@ -1065,8 +1079,8 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
       dvacc[dt][e] = 0.f;
     }
   request_tile(0);
-  if (niter > 1) request_tile(1);
-  if (niter > 2) {
+  if (nit_all > 1) request_tile(1);
+  if (nit_all > 2) {
     request_tile(2);
     wait_all_but_newest_tile();
   } else {
@@ -1090,7 +1104,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
 #pragma unroll
     for (int f = 0; f < 16; ++f) fr[f] = frag(base, 0, f);
   }
-  for (int it = 0; it < niter; ++it) {
+  for (int it = 0; it < nit_all; ++it) {
     const int stage = it % NS;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
@@ -1098,7 +1112,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
       // iteration's first barrier: the score waves start on it right after.  Tile it+2 may still
       // be on its way.
       if (sub == 0 && it > 0) {  // (tiles 0 and 1 were awaited before the loop)
-        if (it + 2 < niter) {
+        if (it + 2 < nit_all) {
           // in flight behind tile it+1: the first five pieces of tile it+2
           if (wave < 2)
             __builtin_amdgcn_s_waitcnt(0x0f75);  // vmcnt(5)
@@ -1114,8 +1128,8 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
       // tile it+3 goes into its stage, one request behind each of the first MFMAs — pieces 0-4
       // in this block, pieces 5-8 in the first block of the next iteration, so that neither
       // block of the accumulate waves outlasts the score waves' step beside it.
-      const bool first_pieces = sub == 1 && it + 3 < niter;
-      const bool last_pieces = sub == 0 && it > 0 && it + 2 < niter;
+      const bool first_pieces = sub == 1 && it + 3 < nit_all;
+      const bool last_pieces = sub == 0 && it > 0 && it + 2 < nit_all;
       if (first_pieces) request_begin(it + 3);
       const uint32_t xa = xch_lane + sub * 16384;
       bf16x8 hand[4];  // P (queries 0-15, 16-31 of the block), dS (the same)
@@ -1147,7 +1161,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
   RowStage rs;
   rs.init(reinterpret_cast<char*>(smem) + XCH + wave * 4096, lane);
   if (PARTIAL) {
-    const int64_t prow = (((int64_t)bi * nq + head) * qsplit + part) * s + kw0;
+    const int64_t prow = (((int64_t)bi * nhg + hgroup) * qsplit + part) * s + kw0;
     store_rows_f32(rs, dkacc, scale, part_k + prow * HD, HD);
     store_rows_f32(rs, dvacc, 1.0f, part_v + prow * HD, HD);
   } else {
@@ -1160,19 +1174,19 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
 // 8 channels (two 16-byte reads per partial, one 16-byte bf16 store).
 __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
     const float* __restrict__ part_k, const float* __restrict__ part_v, bf16* __restrict__ dk,
-    bf16* __restrict__ dv, int s, int nq, int nkv, int qsplit, int64_t total, KLayout dkl, KLayout dvl) {
+    bf16* __restrict__ dv, int s, int nslots, int nkv, int qsplit, int64_t total, KLayout dkl, KLayout dvl) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (bi, kvh, si, chunk of 8)
   if (idx >= total) return;
   const int c = (int)(idx & 15);
   const int si = (int)((idx >> 4) % s);
   const int kvh = (int)((idx >> 4) / s % nkv);
   const int bi = (int)((idx >> 4) / ((int64_t)s * nkv));
-  const int per = nq / nkv;
+  const int per = nslots / nkv;  // partial results per KV head: one per workgroup that served the group
   float ak[8], av[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) ak[e] = av[e] = 0.f;
-  for (int j = 0; j < per * qsplit; ++j) {  // (query head of the group, query-tile part) pairs are consecutive
-    const int64_t off = (((((int64_t)bi * nq + kvh * per) * qsplit + j) * s) + si) * HD + c * 8;
+  for (int j = 0; j < per * qsplit; ++j) {  // (heads' workgroup, query-tile part) pairs are consecutive
+    const int64_t off = (((((int64_t)bi * nslots + kvh * per) * qsplit + j) * s) + si) * HD + c * 8;
     const f32x4 k0 = *reinterpret_cast<const f32x4*>(part_k + off);
     const f32x4 k1 = *reinterpret_cast<const f32x4*>(part_k + off + 4);
     const f32x4 v0 = *reinterpret_cast<const f32x4*>(part_v + off);
@@ -1358,7 +1372,7 @@ template __global__ void attn_bwd_dq_kernel<2, true>(KR_ATTN_DQ_ARGS);
 
 #define KR_ATTN_DKDV_ARGS                                                                          \
   const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, bf16*, \
-      float*, float*, int, int, int, int, float, float, QLayout, KLayout, KLayout, QLayout,      \
+      float*, float*, int, int, int, int, int, float, float, QLayout, KLayout, KLayout, QLayout,      \
       KLayout, KLayout
 template __global__ void attn_bwd_dkdv_kernel<false>(KR_ATTN_DKDV_ARGS);
 template __global__ void attn_bwd_dkdv_kernel<true>(KR_ATTN_DKDV_ARGS);
@@ -1629,11 +1643,16 @@ __global__ __launch_bounds__(GTHREADS) void attn_general_dq_kernel(
 
 }  // namespace
 
-// The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
-// set by the first key tiles (they see every query): two workgroups then share each key tile.
+// Build-time caps, for measuring one form of a kernel against another: the most query heads a
+// dK/dV workgroup takes, and the most workgroups the dQ kernel over shared key tiles is used for.
+#ifndef KR_DKDV_HPW_MAX
+#define KR_DKDV_HPW_MAX 4
+#endif
 #ifndef KR_DQ_SHARED_MAX
 #define KR_DQ_SHARED_MAX (1 << 30)
 #endif
+// The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
+// set by the first key tiles (they see every query): two workgroups then share each key tile.
 static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <= 2 * 256 ? 2 : 1; }
 
 extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
@@ -1697,7 +1716,19 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   float* part_k = neg_lse2 + rows;
   const int qsplit = dkdv_query_split(s, b, nq);
   float* part_v = part_k + rows * qsplit * hd;
-  const bool partial = nq != nkv || qsplit > 1;
+  // query heads of a KV group per dK/dV workgroup: as many as leave two workgroups per compute
+  // unit (KR_DKDV_HPW_MAX: a build-time cap, for measurements)
+  int hpw = 1;
+  {
+    const int per_group = nq / nkv;
+    const int64_t wgs = (int64_t)(s / 128) * nq * b * qsplit;
+    for (int h2 = per_group < KR_DKDV_HPW_MAX ? per_group : KR_DKDV_HPW_MAX; h2 > 1; --h2)
+      if (per_group % h2 == 0 && wgs / h2 >= 2 * (int64_t)kr_compute_units()) {
+        hpw = h2;
+        break;
+      }
+  }
+  const bool partial = nq / hpw != nkv || qsplit > 1;
   constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512) + 32768;  // three stages + the hand-over area
   constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
   static const hipError_t attr_status = [] {
@@ -1724,19 +1755,19 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
                      (const bf16*)dout, (const bf16*)o, lse, delta, neg_lse2, s, nq, per, rows, dol, ol);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
-  const dim3 grid_kv((s / 128) * nq * b * qsplit);
+  const dim3 grid_kv((s / 128) * (nq / hpw) * b * qsplit);
 #define KR_DKDV_LAUNCH(P)                                                                           \
   hipLaunchKernelGGL((attn_bwd_dkdv_kernel<P>), grid_kv, dim3(512), lds_dkdv, st, (const bf16*)q,   \
                      (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const float*)neg_lse2,     \
                      (const float*)delta, (bf16*)dk, (bf16*)dv, part_k, part_v, s, nq, nkv,         \
-                     partial ? qsplit : 1, scale, scale_log2, ql, kl, vl, dol, dkl, dvl)
+                     partial ? qsplit : 1, hpw, scale, scale_log2, ql, kl, vl, dol, dkl, dvl)
   if (partial) {
     KR_DKDV_LAUNCH(true);
     if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
     const int64_t total = (int64_t)b * nkv * s * 16;
     hipLaunchKernelGGL(attn_group_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                       st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s, nq,
-                       nkv, qsplit, total, dkl, dvl);
+                       st, (const float*)part_k, (const float*)part_v, (bf16*)dk, (bf16*)dv, s,
+                       nq / hpw, nkv, qsplit, total, dkl, dvl);
   } else {
     KR_DKDV_LAUNCH(false);
   }

@@ -252,7 +252,11 @@ def _grouped(s, b, nq, nkv, hd, seed):
                                         (768, 11, 8, 8),    # 3 tiles per pair: plain longest-first order
                                         (512, 33, 8, 2),    # 2 tiles per pair, 264 pairs: the last group of 16 pairs is incomplete
                                         (2304, 4, 8, 2),    # 9 tiles per pair: an odd tile count, half 0 idles through two steps of 36
-                                        (512, 6, 24, 8)])   # three query heads per KV head in the shared-tile kernels
+                                        (512, 6, 24, 8),    # three query heads per KV head in the shared-tile kernels
+                                        # enough key tiles that a dK/dV workgroup serves several query heads of its KV group:
+                                        (512, 32, 8, 4),    # both heads of a group: dK/dV stored directly, no partial results
+                                        (512, 64, 8, 2),    # all four heads of a group
+                                        (256, 128, 6, 2)])  # all three heads of a group
 def test_attention_forward_backward(be, s, b, nq, nkv):
     hd = 128
     _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=22)
