@@ -741,6 +741,8 @@ def main():
             "serial_1nb_ms": med["serial_1nb"] * 1e3,
             "speedup_vs_serial_1nb": med["serial_1nb"] / med["nanobatched"],
             "rounds_ms": {k: [round(t * 1e3, 4) for t in v] for k, v in samples.items()},
+            # the plan file steers the nanobatched ways; one nanobatch has no slots to schedule
+            "schedule_file_of_the_nanobatched_ways": os.path.relpath(schedule_path, ROOT) if schedule_path else None,
         }
         if "same_nb_one_stream" in med:
             out["overlap"]["same_nb_one_stream_ms"] = med["same_nb_one_stream"] * 1e3
