@@ -17,6 +17,7 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence, Tuple
 
+from ..backend import reserve_compute_units
 from ..partitions.backward_partition import BackwardPartition
 from ..partitions.context_manager import NanoBatchContext
 from ..partitions.forward_partition import ForwardPartition
@@ -129,8 +130,14 @@ class PartitionExecutor:
 
     # -- one timed unit -------------------------------------------------------------
     def execute(self, overlap_window, sm_configs):
+        """One run of the partition under ``overlap_window`` and ``sm_configs = (sm, block)``.  The
+        ``sm`` compute units are the ones handed to the overlapped work: the partition's own
+        device-filling kernels launch on the rest, as they do inside a step, so the measured time
+        and energy are those of the partition under that budget."""
         self.partition._schedule_config = (overlap_window, sm_configs)
-        return self.partition.execute(ctx=self.ctx, pre_ctx=self.pre_ctx)
+        sm = (sm_configs[0] if sm_configs else 0) or 0
+        with reserve_compute_units(sm):
+            return self.partition.execute(ctx=self.ctx, pre_ctx=self.pre_ctx)
 
     def output(self, channel: str):
         """Tensor the channel holds after the last ``execute``."""

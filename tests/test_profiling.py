@@ -96,6 +96,20 @@ def test_backward_partitions_match_autograd_and_are_repeatable(key):
         assert torch.equal(dx, first)
 
 
+def test_executor_runs_the_partition_under_its_compute_unit_budget(monkeypatch):
+    """The ``sm`` of a configuration is reserved while the partition runs (its device-filling
+    launches take the rest), and only then."""
+    from kareus_amd.backend import reserved_compute_units
+    t = PartitionTest("fwd_mlp", _cfg(), batch_size=2, seq_len=16)
+    seen = []
+    inner = t.executor.partition.execute
+    monkeypatch.setattr(t.executor.partition, "execute",
+                        lambda **kw: (seen.append(reserved_compute_units()), inner(**kw))[1])
+    for sm in (16, 64, 0):
+        t.test_config(("linear_0", "none"), (sm, 1024))
+    assert seen == [16, 64, 0] and reserved_compute_units() == 0
+
+
 def test_executor_argument_errors():
     t = PartitionTest("fwd_mlp", _cfg(), batch_size=2, seq_len=16)
     with pytest.raises(ValueError, match="Invalid direction"):
