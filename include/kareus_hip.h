@@ -32,6 +32,10 @@ extern "C" {
 int kr_version(void);
 /* Static text for a return code. */
 const char* kr_error_string(int code);
+/* Rated shader clock of the current device in MHz (0 if it cannot be read): the label a profiling
+ * sweep gives its rows when it leaves the clock alone.  The reference labels rows with the clock it
+ * locks through NVML (tests/bayesian/common/hardware.py:52-59, :107-114). */
+int kr_device_clock_mhz(void);
 
 /* ---- GEMM ------------------------------------------------------------------------------
  * bf16 x bf16 -> fp32 accumulate -> bf16.  Replaces tex.generic_gemm (cuBLASLt) as called

@@ -25,6 +25,7 @@ _c_void_p, _c_int, _c_i64, _c_float, _c_size_t = (
 _SIGNATURES = {
     "kr_version": (_c_int, []),
     "kr_error_string": (ctypes.c_char_p, [_c_int]),
+    "kr_device_clock_mhz": (_c_int, []),
     "kr_gemm_workspace_bytes": (_c_size_t, [_c_int, _c_int, _c_int, _c_int]),
     "kr_gemm_workspace_bytes_shared": (_c_size_t, [_c_int, _c_int, _c_int, _c_int, _c_float]),
     "kr_gemm_bf16": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,

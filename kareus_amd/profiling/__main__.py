@@ -16,7 +16,7 @@ import torch
 from ..block import LayerConfig
 from ..energy import PowerSampler
 from . import PARTITION_KEYS, PartitionTest, all_configurations, append_eval_log, measure_batch
-from .hardware import available_frequencies_mhz
+from .hardware import nominal_frequency_mhz
 
 
 def main(argv=None) -> int:
@@ -52,7 +52,7 @@ def main(argv=None) -> int:
         from .nonpartition import NonPartitionProfiler
 
         prof = NonPartitionProfiler(cfg, args.vocab_rows, args.batch, args.seq_len, device=device)
-        freq = (args.freq or [max(available_frequencies_mhz() or [0])])[0]
+        freq = (args.freq or [nominal_frequency_mhz()])[0]
         trials = prof.run(args.out_dir, freq, sampler=PowerSampler(), measurement_duration=args.duration,
                           cooldown_duration=args.cooldown)
         for name, t in trials.items():
@@ -60,7 +60,7 @@ def main(argv=None) -> int:
                   flush=True)
         return 0
     test = PartitionTest(args.partition, cfg, args.batch, args.seq_len, device=device)
-    freqs = args.freq or [max(available_frequencies_mhz() or [0])]
+    freqs = args.freq or [nominal_frequency_mhz()]
     configs = all_configurations(freqs, args.sm, test.overlap_windows)
     sampler = PowerSampler()
     for rec in measure_batch(test, configs, sampler, args.duration, args.cooldown):

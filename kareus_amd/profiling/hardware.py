@@ -110,6 +110,26 @@ def available_frequencies_mhz(device_index: int = 0) -> List[int]:
     return out
 
 
+def nominal_frequency_mhz(device_index: int = 0) -> int:
+    """The clock a sweep records when it leaves the clock alone: the device's rated shader clock
+    (the same number on every run and box), else the highest listed level, else 0.  The listed
+    levels are no stable label: the driver shows the clock in force as a level of its own, so
+    their maximum moves by a few MHz between reads."""
+    try:
+        import torch
+
+        if torch.cuda.is_available():
+            from ..backend.hip import load_library
+
+            with torch.cuda.device(device_index):
+                mhz = int(load_library().kr_device_clock_mhz())
+            if mhz > 0:
+                return mhz
+    except (ImportError, OSError, RuntimeError, AttributeError):
+        pass
+    return max(available_frequencies_mhz(device_index) or [0])
+
+
 def set_gpu_frequency(target_freq_mhz: int, device_index: int = 0, settle_s: float = 0.5) -> bool:
     """Pin the shader clock to the listed level closest to ``target_freq_mhz``.  Returns False
     (and changes nothing) when the files are missing or not writable by this user.  ``settle_s``:

@@ -33,6 +33,7 @@ def test_argument_checks_run_without_a_device():
     lib = hip.load_library()
     assert lib.kr_version() >= 100
     assert lib.kr_error_string(0) == b"ok" and b"unknown" in lib.kr_error_string(-99)
+    assert lib.kr_device_clock_mhz() >= 0                         # 0 where no device can be asked
     # invalid arguments are rejected before anything touches the GPU
     assert lib.kr_add(None, None, None, 8, None) == -1
     assert lib.kr_swiglu_fwd(16, 16, 4, 12, None) == -2          # F not a multiple of 8

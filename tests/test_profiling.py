@@ -269,6 +269,15 @@ from kareus_amd.profiling.profile_csv import (  # noqa: E402
 from kareus_amd.scheduler.parser import _parse_config_string  # noqa: E402
 
 
+@pytest.mark.gpu
+def test_nominal_clock_is_the_devices_rated_clock():
+    """The label of a sweep that pins no clock comes from the device's properties, so two reads
+    (and the four partitions' logs of one sweep) agree."""
+    from kareus_amd.profiling import nominal_frequency_mhz
+    a, b = nominal_frequency_mhz(), nominal_frequency_mhz()
+    assert a == b and 1000 <= a <= 4000
+
+
 def test_pareto_filter_uses_effective_energy():
     pts = [("a", (1.0, 100.0)), ("b", (2.0, 90.0)), ("c", (3.0, 95.0)), ("d", (1.0, 120.0)), ("e", (4.0, 150.0))]
     # no idle power: keep strictly improving energy along increasing time
