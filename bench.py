@@ -232,6 +232,51 @@ def _roofline_entry(kernel, layout, m, n, k, sec):
     }
 
 
+class GemmEventTimer:
+    """HIP events around the GEMM launches of given (layout, M, N, K) while a step runs: the events
+    are recorded on the stream the kernel is launched on (the current one), so on that stream an
+    interval is the kernel's own duration.  Two event records per watched launch, nothing else."""
+
+    def __init__(self, be, shapes):
+        self.be, self.shapes = be, set(shapes)
+        self.pairs = {s: [] for s in self.shapes}
+
+    def __enter__(self):
+        inner = self.be.gemm
+
+        def gemm(layout, a, b, m, n, k, *args, **kw):
+            key = (layout, m, n, k)
+            if key not in self.shapes:
+                return inner(layout, a, b, m, n, k, *args, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = inner(layout, a, b, m, n, k, *args, **kw)
+            e1.record()
+            self.pairs[key].append((e0, e1))
+            return r
+
+        self.be.gemm = gemm
+        return self
+
+    def __exit__(self, *exc):
+        del self.be.gemm    # back to the class's method
+        return False
+
+    def seconds(self, key):
+        """(average duration of a launch, launches); call after the device has been synchronised."""
+        pairs = self.pairs.get(key) or []
+        if not pairs:
+            return None, 0
+        return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / len(pairs), len(pairs)
+
+
+def dominant_gemm_shapes(w, nnb):
+    """(layout code, M, N, K) of fc1's weight gradient (NT), forward (TN) and input gradient (NN)
+    at the token count of one launch."""
+    t, two_f, h = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
+    return {"NT": (2, two_f, h, t), "TN": (0, t, two_f, h), "NN": (1, t, h, two_f)}
+
+
 def dominant_kernel_roofline(w, nnb, device, launches=30):
     """The GEMM instance with the largest share of the step's kernel time: the weight gradient of
     fc1, dW[2F, h] = dy[T_nb, 2F]^T . x[T_nb, h] (layout NT), plus the forward (TN, with the SwiGLU
@@ -717,7 +762,11 @@ def main():
 
     # the headline: W warm-up steps, then exactly K timed steps of the chosen configuration
     runner.run(args.warmup)
-    sec = runner.timed(args.steps)
+    from kareus_amd.backend import get_backend
+
+    watched = dominant_gemm_shapes(w, run_nnb)
+    with GemmEventTimer(get_backend("hip"), watched.values()) as in_step:
+        sec = runner.timed(args.steps)
 
     out = {
         "metric": "layer fwd+bwd tokens/sec on 1 MI355X",
@@ -761,7 +810,21 @@ def main():
 
     ways.clear()
     del nano, runner
-    out["roofline"], out["roofline_others"] = dominant_kernel_roofline(w, run_nnb, device)
+    # roofline of the dominant kernel: its launches inside the K timed steps; the same kernel
+    # launched back to back on its own (a hotter chip: nothing but the heaviest GEMM) beside it
+    alone_main, alone_others = dominant_kernel_roofline(w, run_nnb, device)
+    entries = []
+    for alone in [alone_main] + alone_others:
+        layout = alone["kernel"].split("<")[1][:2]
+        s, n_launches = in_step.seconds(watched[layout])
+        if s is None:
+            entries.append(dict(alone, measured="back to back on its own"))
+            continue
+        e = _roofline_entry(alone["kernel"], layout, *watched[layout][1:], s)
+        e["measured"] = f"HIP events around its {n_launches} launches inside the {args.steps} timed steps"
+        e["back_to_back_alone_us"] = alone["avg_launch_us"]
+        entries.append(e)
+    out["roofline"], out["roofline_others"] = entries[0], entries[1:]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
