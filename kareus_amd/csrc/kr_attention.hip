@@ -28,6 +28,13 @@ constexpr int BQ = 128;       // queries per workgroup (4 waves x 32, twice over
 constexpr int BKV = 64;       // keys per staged tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+// Online softmax of the MFMA forward kernels: a row's exponents are taken against a reference
+// point that follows the running maximum only when the maximum has grown by more than this many
+// powers of two.  In between, probabilities run up to 2^8 instead of 1 — rounding is relative in
+// fp32 and in bf16, the row sum and the output carry the same factor and the final division takes
+// it out — and the 64 accumulator multiplies of a rescale are skipped (with 32 rows per wave some
+// row's maximum moves in most tiles; by more than 2^8 it hardly ever does after the first).
+constexpr float kRescaleSlack = 8.0f;
 constexpr int kXcds = 8;
 
 __device__ __forceinline__ int xcd_contiguous_id(int pid, int nblocks) {
@@ -485,10 +492,11 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
       const float m_new = fmaxf(m_run, mx);
-      const float m_ref = m_new == -INFINITY ? 0.f : m_new;  // nothing seen yet: any finite reference
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);
-      const bool moved = m_new != m_run;
-      m_run = m_new;
+      const bool moved = (m_new - m_run) * scale_log2 > kRescaleSlack;  // from -inf: always
+      const float m_next = moved ? m_new : m_run;
+      const float m_ref = m_next == -INFINITY ? 0.f : m_next;  // nothing seen yet: any finite reference
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);  // 1 unless moved
+      m_run = m_next;
       const float neg_m = -m_ref * scale_log2;
       float psum = 0.f;
 #pragma unroll
@@ -746,10 +754,11 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_sh_kernel(
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[t][e]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, KR_WAVE));
       const float m_new = fmaxf(m_run, mx);
-      const float m_ref = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);
-      const bool moved = m_new != m_run;
-      m_run = m_new;
+      const bool moved = (m_new - m_run) * scale_log2 > kRescaleSlack;  // from -inf: always
+      const float m_next = moved ? m_new : m_run;
+      const float m_ref = m_next == -INFINITY ? 0.f : m_next;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * scale_log2);  // 1 unless moved
+      m_run = m_next;
       const float neg_m = -m_ref * scale_log2;
       float psum = 0.f;
 #pragma unroll

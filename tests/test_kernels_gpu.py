@@ -344,6 +344,37 @@ def test_attention_special_cases(be):
         be.attn_fwd(rnd(128, 1, 1, 136), rnd(128, 1, 1, 136), rnd(128, 1, 1, 136), 1.0)  # head_dim above 128
 
 
+@pytest.mark.parametrize("s,b,nq,nkv", [(512, 2, 4, 2),       # split-key forward (few 256-query tiles)
+                                         (512, 64, 8, 2)])     # forward over shared tiles
+@pytest.mark.parametrize("kind", ["wide", "rising", "falling"])
+def test_attention_when_the_row_maximum_keeps_moving(be, s, b, nq, nkv, kind):
+    """The forward kernels move the reference point of a row's exponents only when its maximum has grown
+    by more than 2^8.  Scores N(0,1) never do that after the first tile, so: scores spread over +-40
+    (jumps of every size), scores that rise along the keys (a new maximum in every tile, by a little or
+    by a lot depending on the row) and scores that fall (the first reference stays for good, later
+    probabilities underflow).  Checked against the fp32 oracle like every other shape, lse included."""
+    hd = 128
+    _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=300)
+    q, k = q.clone(), k.clone()
+    if kind == "wide":
+        k *= 12.0                                         # scores ~ N(0, 12^2): jumps of many powers of two
+    else:
+        # one shared direction u: score(i, j) = (q_i . u)(k_j . u) + noise, |k_j . u| growing with j
+        u = torch.nn.functional.normalize(rnd(hd, seed=301).float(), dim=0).bfloat16()
+        ramp = torch.linspace(0.0, 30.0, s, device=DEV).view(s, 1, 1, 1)
+        if kind == "falling":
+            ramp = -ramp
+        k += (ramp * u.float()).bfloat16()
+        q += (torch.linspace(0.2, 4.0, s, device=DEV).view(s, 1, 1, 1, 1) * u.float()).bfloat16()
+    scale = hd ** -0.5
+    o, lse = be.attn_fwd(q, k, v, scale)
+    qf, kf, vf = (t.float().cpu() for t in (q.flatten(2, 3), k, v))
+    ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
+    assert torch.equal(o[0], v[0].repeat_interleave(nq // nkv, dim=1))     # one visible key: o = v exactly
+
+
 @pytest.mark.parametrize("s,b,nq,nkv,hd", [(100, 1, 1, 1, 128),    # ragged length at the fast kernels' head dimension
                                             (256, 2, 8, 8, 64),     # benchmark configuration 1: 8 heads of 64
                                             (77, 3, 6, 2, 64),      # ragged, grouped queries
