@@ -269,6 +269,21 @@ from kareus_amd.profiling.profile_csv import (  # noqa: E402
 from kareus_amd.scheduler.parser import _parse_config_string  # noqa: E402
 
 
+def test_listed_clock_levels_and_the_label_without_a_device(tmp_path, monkeypatch):
+    """``pp_dpm_sclk`` lines ``"<n>: <MHz>Mhz [*]"`` are the levels (a line ``S: ...`` is the clock in
+    force, not a level); without a device to ask, a sweep that pins no clock is labelled with the
+    highest of them, and with 0 when there is no such file."""
+    from kareus_amd.profiling import hardware
+    dev = tmp_path / "dev"
+    dev.mkdir()
+    (dev / "pp_dpm_sclk").write_text("0: 132Mhz\n1: 2105Mhz *\n2: 2400Mhz\nS: 2105Mhz *\n")
+    monkeypatch.setattr(hardware, "sysfs_device_dir", lambda i=0: str(dev))
+    assert hardware.available_frequencies_mhz() == [132, 2105, 2400]
+    assert hardware.nominal_frequency_mhz() == 2400          # no GPU here: the listed maximum
+    (dev / "pp_dpm_sclk").unlink()
+    assert hardware.available_frequencies_mhz() == [] and hardware.nominal_frequency_mhz() == 0
+
+
 @pytest.mark.gpu
 def test_nominal_clock_is_the_devices_rated_clock():
     """The label of a sweep that pins no clock comes from the device's properties, so two reads
