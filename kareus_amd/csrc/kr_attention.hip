@@ -224,6 +224,13 @@ struct KLayout {
   __device__ __forceinline__ int64_t at(int bi, int kvh) const { return (int64_t)bi * b_ + kvh * h_; }
 };
 
+// Scalar loads return out of order, so while one is pending (a kernel argument fetched in the
+// prologue and first used behind the loop is, as far as the compiler's wait-count pass knows, for
+// the whole loop) every wait for an LDS read becomes lgkmcnt(0): the first MFMA of a group then
+// waits for the fragments of the next group too.  An explicit lgkmcnt(0) in front of a loop ends
+// that: inside, the waits count.
+__device__ __forceinline__ void settle_scalar_loads() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+
 // ---- direct global -> LDS loads (see the GEMM for why they are written as inline assembly:
 // the compiler must not know of them, or it drains them in front of every barrier).  The 64
 // lanes of one load land contiguously: lane p at lds_byte + 16 p.
@@ -435,6 +442,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_pp_kernel(
       }
       };
 
+  settle_scalar_loads();
   for (int j = 0; j < nsteps; ++j) {
     // ---- matrix period: O^T += V^T . P^T of tile j-1, then S^T = K . Q^T of tile j
     f32x16 sacc[2];
@@ -697,6 +705,7 @@ __global__ __launch_bounds__(512, 1) void attn_fwd_sh_kernel(
   };
 
   int slot = 0, slot_prev = 2, slot_req = 2;  // j % 3, (j - 1) % 3, (j + 2) % 3
+  settle_scalar_loads();
   for (int j = 0; j < ntiles; ++j) {
     // ---- matrix period: O^T += V^T . P^T of tile j-1, then S^T = K . Q^T of tile j
     f32x16 sacc[2];
@@ -1011,6 +1020,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
     // tile is complete by the first barrier of the iteration; behind the last tile a stale
     // stage is read, unused).
     f32x16 s0, dp0, s1, dp1;
+    settle_scalar_loads();
     issue_scores(0, 0, s0, dp0);
     for (int it = 0, itl = 0; it < nit_all; ++it) {
       const int stage = it % NS;
@@ -1113,6 +1123,7 @@ __global__ __launch_bounds__(512, 1) void attn_bwd_dkdv_kernel(
 #pragma unroll
     for (int f = 0; f < 16; ++f) fr[f] = frag(base, 0, f);
   }
+  settle_scalar_loads();
   for (int it = 0; it < nit_all; ++it) {
     const int stage = it % NS;
 #pragma unroll
@@ -1292,6 +1303,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
+  settle_scalar_loads();
   for (int j = 0; j < ntiles; ++j) {
     const int cur = j & 1;
     if (j + 1 < ntiles) stage_request(j + 1, cur ^ 1);
