@@ -170,12 +170,25 @@ def partition_times(stepper, iters=3):
 # runs of `bench.py --roofline-only`, each scaled by what the same counter reads for
 # `bench.py --copy-calibration`).  Keyed by (layout, M, N, K); a shape that was not profiled
 # reports null.  A constant read off a profile, not something measured in this run: the entry
-# names the profile it came from.
+# names the profile it came from, and it is only reported while the GEMM source is the one the
+# counters were read with (first 16 hex digits of its SHA-256).
+TRAFFIC_GEMM_SOURCE = "7cee73aae2f62812"
 MEASURED_TRAFFIC = {
-    ("NT", 7168, 4096, 16384): {"bytes": (786725.5 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("TN", 16384, 7168, 4096): {"bytes": (721829.1 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 16384, 4096, 7168): {"bytes": (688411.6 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NT", 7168, 4096, 16384): {"bytes": (761642.4 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 16384, 7168, 4096): {"bytes": (736977.8 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 16384, 4096, 7168): {"bytes": (688400.5 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
 }
+
+
+def _gemm_source_is_the_profiled_one() -> bool:
+    import hashlib
+
+    path = os.path.join(ROOT, "kareus_amd", "csrc", "kr_gemm.hip")
+    try:
+        with open(path, "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()[:16] == TRAFFIC_GEMM_SOURCE
+    except OSError:
+        return False
 
 
 def _gemm_operands(layout, m, n, k, device):
@@ -221,7 +234,7 @@ def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, resi
 def _roofline_entry(kernel, layout, m, n, k, sec):
     flops = 2.0 * m * n * k
     achieved = flops / sec / 1e12
-    traffic = MEASURED_TRAFFIC.get((layout, m, n, k))
+    traffic = MEASURED_TRAFFIC.get((layout, m, n, k)) if _gemm_source_is_the_profiled_one() else None
     return {
         "bound": "mfma", "kernel": kernel, "shape": [m, n, k],
         "flops_per_launch": flops, "avg_launch_us": sec * 1e6,
