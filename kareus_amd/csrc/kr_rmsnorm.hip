@@ -218,7 +218,12 @@ __global__ __launch_bounds__(kDgammaThreads) void rmsnorm_dgamma_kernel(const fl
 }
 
 // rows wider than 4096 elements are shared by two waves
-inline int bwd_split(int cols) { return cols > 4096 ? 2 : 1; }
+// Rows wider than this are shared by two waves (half the registers per wave, twice the waves per
+// SIMD to hide the latency of a row's loads behind)
+#ifndef KR_RMS_SPLIT_ABOVE
+#define KR_RMS_SPLIT_ABOVE 2048
+#endif
+inline int bwd_split(int cols) { return cols > KR_RMS_SPLIT_ABOVE ? 2 : 1; }
 
 inline int bwd_blocks(int rows, int cols) {
   const int rows_per_block = kWaves / bwd_split(cols);
