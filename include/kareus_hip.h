@@ -141,7 +141,9 @@ int kr_rmsnorm_dgamma(const float* partial, int nparts, int cols, void* dgamma, 
  * that the library holds in device memory on every GPU it runs on until the process ends; the
  * call itself allocates and frees nothing (its first call on a device looks the array's address
  * up, so make one call per device before a region in which even that is unwelcome).
- * cols above 8192 return KR_EUNSUPPORTED.  Results are bit-identical to kr_rmsnorm_bwd_add.
+ * cols above 8192 return KR_EUNSUPPORTED; dgamma == NULL returns KR_EINVAL (the partial rows stay
+ * in an array no caller can read, so the reduced gradient must have a destination).  Results are
+ * bit-identical to kr_rmsnorm_bwd_add.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams
  * or threads) race on it and must be ordered by the caller.                                     */
 int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const float* rstd, const void* gamma,

@@ -326,7 +326,9 @@ extern "C" int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const f
                                           const void* gamma, const void* dres, void* dx,
                                           void* dgamma, int rows, int cols, int64_t dy_ld,
                                           int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream) {
-  if (rows <= 0 || cols <= 0) return KR_EINVAL;
+  // the partial rows stay in the library's private array, which no caller can read: without a
+  // place for the reduced weight gradient the call could not hand it over at all
+  if (rows <= 0 || cols <= 0 || !dgamma) return KR_EINVAL;
   if (cols > kScratchCols) return KR_EUNSUPPORTED;  // beyond what the device array holds
   float* const ws = scratch_on_current_device();
   if (ws == nullptr) return KR_ELAUNCH;

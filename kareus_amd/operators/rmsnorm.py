@@ -52,16 +52,25 @@ class RMSNorm(BasicOperation):
             return be.rmsnorm_bwd(dy, x2d, rstd, self.weight.detach(), residual_grad=residual_grad, out=out2d)
         rows, cols = x2d.shape
         per = be.rmsnorm_partial_rows(rows, cols)
+        api = stream_api()
+        here = api.current_stream()
         buf = sink.get("buf")
         if buf is None or buf.shape[0] != n * per:
             buf = sink["buf"] = torch.empty((n * per, cols), dtype=torch.float32, device=x2d.device)
             sink["done"], sink["events"] = 0, []
+            # The block comes from the allocator's pool of THIS stream: whatever used it last is ordered
+            # before work queued here, not before the other nanobatch streams.  They wait for this event
+            # before they write their rows.
+            sink["allocated"] = None
+            if here is not None:
+                sink["allocated"] = (here, api.new_event())
+                sink["allocated"][1].record(here)
+        elif here is not None and sink.get("allocated") is not None and sink["allocated"][0] != here:
+            here.wait_event(sink["allocated"][1])
         k = sink["done"]
         dx, _ = be.rmsnorm_bwd(dy, x2d, rstd, self.weight.detach(), residual_grad=residual_grad, out=out2d,
                                partials_out=buf[k * per:(k + 1) * per])
         sink["done"] = k + 1
-        api = stream_api()
-        here = api.current_stream()
         if here is not None and hasattr(buf, "record_stream") and buf.is_cuda:
             buf.record_stream(here)   # the buffer is shared by the nanobatch streams
         if sink["done"] < n:
