@@ -607,6 +607,80 @@ def cu_budget_sweep(w, device, budgets=(0, 8, 16, 32, 64), rounds=4, steps=6):
     return {name: t * 1e3 for name, t in med.items()}
 
 
+class _SuppressedLaunches:
+    """Timing only: the library entry points named here return success without launching (their outputs
+    keep whatever the buffers held), so a step runs as if those kernels cost nothing."""
+
+    def __init__(self, lib, names):
+        self.lib, self.names, self.saved = lib, names, {}
+
+    def __enter__(self):
+        for n in self.names:
+            self.saved[n] = getattr(self.lib, n)
+            setattr(self.lib, n, lambda *a, **k: 0)
+        return self
+
+    def __exit__(self, *exc):
+        for n, fn in self.saved.items():
+            setattr(self.lib, n, fn)
+
+
+def overlap_bound(w, device, rounds=4, steps=8):
+    """What overlap between nanobatches could win on one GPU at best, and whether the host limits it.
+
+    (1) The nanobatched step with its HBM-bound launches (RMSNorm forward / backward, rotary embedding,
+        the norm weight-gradient reduction) suppressed: the time it would take if every one of them hid
+        completely behind the other nanobatches' MFMA-bound kernels.  Timing only — results are wrong.
+    (2) The same for the one-nanobatch step (its floor without those kernels).
+    (3) The nanobatched step with a busy wait added to the host's work per step: GPU time against host time.
+    All interleaved after a pre-heat, median ms per step."""
+    from kareus_amd.backend import get_backend
+
+    gen = torch.Generator().manual_seed(42)
+    x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
+    go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
+    nano = Stepper(make_model(w, w["nnb"], device), x, go)
+    serial = Stepper(make_model(w, 1, device, use_streams=False), x, go)
+    for st in (nano, serial):
+        st.run(2)
+    preheat(nano, 2.0)
+    lib = get_backend("hip").lib
+    hbm = ["kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rmsnorm_bwd_add", "kr_rmsnorm_dgamma", "kr_rope"]
+    samples = {k: [] for k in ("nanobatched", "one nanobatch", "nanobatched, HBM-bound launches suppressed",
+                               "one nanobatch, HBM-bound launches suppressed")}
+    for _ in range(rounds):
+        samples["nanobatched"].append(nano.timed(steps))
+        samples["one nanobatch"].append(serial.timed(steps))
+        with _SuppressedLaunches(lib, hbm):
+            samples["nanobatched, HBM-bound launches suppressed"].append(nano.timed(steps))
+            samples["one nanobatch, HBM-bound launches suppressed"].append(serial.timed(steps))
+    out = {"ms_per_step": {k: sorted(v)[len(v) // 2] * 1e3 for k, v in samples.items()}}
+
+    def spin(us):
+        end = time.perf_counter() + us * 1e-6
+        while time.perf_counter() < end:
+            pass
+
+    plain_step = nano.step
+    delays = {}
+    for extra_us in (0, 300, 600, 1000, 1500):
+        def step():
+            spin(extra_us)
+            plain_step()
+        nano.step = step
+        nano.run(4)
+        gpu = sorted(nano.timed(24) for _ in range(3))[1]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        nano.run(12)                      # the queues are empty: this is the host's own time per step
+        host = (time.perf_counter() - t0) / 12
+        torch.cuda.synchronize()
+        delays[f"+{extra_us} us of host work per step"] = {"ms_per_step": gpu * 1e3, "host_ms_per_step": host * 1e3}
+    nano.step = plain_step
+    out["host_delay"] = delays
+    return out
+
+
 def preheat(stepper, seconds=2.0):
     """Run the layer until the chip has been busy for `seconds`: clocks and temperature settle at what a
     training run sees, instead of the first timed window getting a cool chip and the last a hot one."""
@@ -683,9 +757,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
-    ap.add_argument("--nanobatches", default="auto",
-                    help="'auto' (default): the faster of the workload's nanobatch count and one nanobatch, "
-                         "measured; 'workload': the workload's count; or a number")
+    ap.add_argument("--nanobatches", default="workload",
+                    help="'workload' (default): the workload's nanobatch count, which is what `value` reports; "
+                         "'auto': the faster of that count and one nanobatch, measured; or a number")
     ap.add_argument("--schedule", default=None,
                     help="per-microbatch plan file for the nanobatched run (default: the shipped plan for c5, none otherwise)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -706,6 +780,9 @@ def main():
                     help="run only the layer's twelve GEMMs stand-alone at nanobatch shape, as the engine launches them")
     ap.add_argument("--cu-budget-sweep", action="store_true",
                     help="run only the nanobatched step under schedules reserving 0..64 compute units")
+    ap.add_argument("--overlap-bound", action="store_true",
+                    help="run only: the nanobatched step with its HBM-bound launches suppressed (the best any "
+                         "overlap could do) and with extra host work per step")
     ap.add_argument("--power-trace", action="store_true",
                     help="run only the power / shader-clock trace over kernels and layer steps")
     args = ap.parse_args()
@@ -744,6 +821,9 @@ def main():
     if args.power_trace:
         print(json.dumps({"power_trace": power_trace(w, device)}))
         return
+    if args.overlap_bound:
+        print(json.dumps({"overlap_bound": overlap_bound(w, device)}))
+        return
     gen = torch.Generator().manual_seed(42)
     x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
     go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
@@ -780,6 +860,11 @@ def main():
     watched = dominant_gemm_shapes(w, run_nnb)
     with GemmEventTimer(get_backend("hip"), watched.values()) as in_step:
         sec = runner.timed(args.steps)
+    # beside it, timed the same way: the one-nanobatch (serial) step of the same layer and data
+    serial_sec = None
+    if "serial_1nb" in ways and picked != "serial_1nb":
+        ways["serial_1nb"].run(args.warmup)
+        serial_sec = ways["serial_1nb"].timed(args.steps)
 
     out = {
         "metric": "layer fwd+bwd tokens/sec on 1 MI355X",
@@ -796,6 +881,11 @@ def main():
         "mfma_util_end_to_end": flops / sec / MFMA_PEAK_BF16,
         "tflops_end_to_end": flops / sec / 1e12,
     }
+    if serial_sec is not None:
+        out["serial_1nb"] = {"what": "the same layer and data run as one nanobatch on one stream (no overlap engine at "
+                                     "work), same warm-up and step count, timed right after the headline steps",
+                             "value": tokens / serial_sec, "unit": "tokens/s", "ms_per_step": serial_sec * 1e3,
+                             "mfma_util_end_to_end": flops / serial_sec / MFMA_PEAK_BF16}
     if "serial_1nb" in med:
         out["overlap"] = {
             "timing": "interleaved rounds after a 2 s pre-heat, median of 5 rounds per way",

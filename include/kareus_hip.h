@@ -214,6 +214,21 @@ int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
                 int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
                 int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
                 void* stream);
+/* The same call with a flags word (0 = kr_attn_fwd).  KR_ATTN_BESIDE_OTHER_STREAMS: kernels of other
+ * streams run beside this launch and use the compute units it leaves idle (the engine's nanobatch
+ * streams), so the launch is shaped for the least compute-unit time rather than for its own latency:
+ * whole rows / whole key tiles per workgroup whatever their number, no second pass and no merge.
+ * The two shapes sum in different orders: results agree to rounding, and for a given flags word they
+ * do not depend on the batch size.  No counterpart in the reference's call
+ * (kareus/flash_attn/flash_attn_interface.py:66-80 runs one kernel at a time).                   */
+#define KR_ATTN_BESIDE_OTHER_STREAMS 0x100
+int kr_attn_fwd_flags(const void* q, const void* k, const void* v, void* o, float* lse,
+                      int s, int b, int nq, int nkv, int hd, float scale,
+                      int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
+                      int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
+                      int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
+                      int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
+                      int flags, void* stream);
 size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);
 int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                 const void* o, const float* lse,
@@ -228,6 +243,21 @@ int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                 int64_t dk_stride_s, int64_t dk_stride_b, int64_t dk_stride_h,
                 int64_t dv_stride_s, int64_t dv_stride_b, int64_t dv_stride_h,
                 void* stream);
+/* kr_attn_bwd with the flags word of kr_attn_fwd_flags (same workspace size).
+ * Replaces the same call, kareus/flash_attn/flash_attn_interface.py:174-194.                       */
+int kr_attn_bwd_flags(const void* dout, const void* q, const void* k, const void* v,
+                      const void* o, const float* lse,
+                      void* dq, void* dk, void* dv, void* workspace,
+                      int s, int b, int nq, int nkv, int hd, float scale,
+                      int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
+                      int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
+                      int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
+                      int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
+                      int64_t do_stride_s, int64_t do_stride_b, int64_t do_stride_g, int64_t do_stride_h,
+                      int64_t dq_stride_s, int64_t dq_stride_b, int64_t dq_stride_g, int64_t dq_stride_h,
+                      int64_t dk_stride_s, int64_t dk_stride_b, int64_t dk_stride_h,
+                      int64_t dv_stride_s, int64_t dv_stride_b, int64_t dv_stride_h,
+                      int flags, void* stream);
 
 /* ---- Ends of the layer stack: embedding and loss ------------------------------------------
  * Token embedding of one vocabulary shard.  Replaces F.embedding / weight[masked_input] and the

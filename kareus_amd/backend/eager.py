@@ -136,7 +136,8 @@ class EagerBackend:
     # Causal GQA attention on [s, b, heads, hd] tensors; query head i reads KV head
     # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32
     # (kareus/flash_attn/flash_attn_interface.py:473-493).
-    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
+    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True,
+                 beside_other_streams: bool = False):
         if q.dim() == 5:
             q = q.flatten(2, 3)
         s, b, nq, hd = q.shape
@@ -154,7 +155,7 @@ class EagerBackend:
         o = (p @ vf).permute(2, 0, 1, 3).contiguous()
         return o.to(q.dtype), lse.contiguous()
 
-    def attn_bwd(self, do, q, k, v, o, lse, scale: float, causal: bool = True):
+    def attn_bwd(self, do, q, k, v, o, lse, scale: float, causal: bool = True, beside_other_streams: bool = False):
         if q.dim() == 5:
             q = q.flatten(2, 3)
         s, b, nq, hd = q.shape

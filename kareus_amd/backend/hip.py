@@ -51,11 +51,14 @@ _SIGNATURES = {
     "kr_cross_entropy_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p]),
     "kr_cross_entropy_bwd": (_c_int, [_c_void_p] * 5 + [_c_i64, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_void_p]),
+    "kr_attn_fwd_flags": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_int, _c_void_p]),
     "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
     "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_void_p]),
+    "kr_attn_bwd_flags": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_int, _c_void_p]),
 }
 
 KR_GEMM_TN, KR_GEMM_NN, KR_GEMM_NT = 0, 1, 2
+KR_ATTN_BESIDE_OTHER_STREAMS = 0x100
 
 
 def library_path() -> str:
@@ -498,7 +501,10 @@ class HipBackend:
             raise RuntimeError("grouped query tensor must have one group per KV head")
         return s, b, nq, nkv, hd
 
-    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True):
+    def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True,
+                 beside_other_streams: bool = False):
+        """``beside_other_streams``: kernels of other streams use the compute units this launch leaves idle,
+        so it is shaped for the least compute-unit time, not for its own latency."""
         if not causal:
             raise RuntimeError("only causal attention is implemented")
         self._dev(q, k, v)
@@ -507,14 +513,15 @@ class HipBackend:
         per = nq // nkv
         o = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
         lse = torch.empty((b, nq, s), dtype=torch.float32, device=q.device)
-        rc = self.lib.kr_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-                                  s, b, nq, nkv, hd, scale, *self._q_strides(q, per), *self._k_strides(k),
-                                  *self._k_strides(v), *self._q_strides(o, per), self._stream())
+        flags = KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0
+        rc = self.lib.kr_attn_fwd_flags(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                        s, b, nq, nkv, hd, scale, *self._q_strides(q, per), *self._k_strides(k),
+                                        *self._k_strides(v), *self._q_strides(o, per), flags, self._stream())
         self._check(rc, f"kr_attn_fwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
         return o, lse
 
     def attn_bwd(self, do: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor,
-                 scale: float, causal: bool = True):
+                 scale: float, causal: bool = True, beside_other_streams: bool = False):
         """Returns (dq, dk, dv).  If ``q`` is a grouped [s, b, ng, per, hd] view, the three
         gradients are views of one buffer laid out like the fused QKV projection output and
         carry it as ``_kr_mixed`` so the QKV-split backward can hand it on without a copy."""
@@ -537,13 +544,14 @@ class HipBackend:
             dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
         nbytes = self.lib.kr_attn_bwd_workspace_bytes(s, b, nq, nkv, hd)
         ws = self._workspace(max(nbytes, 16), q.device)
-        rc = self.lib.kr_attn_bwd(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
-                                  lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
-                                  s, b, nq, nkv, hd, scale,
-                                  *self._q_strides(q, per), *self._k_strides(k), *self._k_strides(v),
-                                  *self._q_strides(o4, per), *self._q_strides(do4, per),
-                                  *self._q_strides(dq, per), *self._k_strides(dk), *self._k_strides(dv),
-                                  self._stream())
+        flags = KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0
+        rc = self.lib.kr_attn_bwd_flags(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
+                                        lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
+                                        s, b, nq, nkv, hd, scale,
+                                        *self._q_strides(q, per), *self._k_strides(k), *self._k_strides(v),
+                                        *self._q_strides(o4, per), *self._q_strides(do4, per),
+                                        *self._q_strides(dq, per), *self._k_strides(dk), *self._k_strides(dv),
+                                        flags, self._stream())
         self._check(rc, f"kr_attn_bwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
         if mixed is not None:
             for t in (dq, dk, dv):

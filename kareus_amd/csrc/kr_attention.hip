@@ -1686,7 +1686,27 @@ extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int
   return bytes;
 }
 
-extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+// Which form of each kernel a launch takes.  Alone on the GPU a launch wants the shortest latency:
+// with few workgroups the keys of a row (forward, dQ) or the queries of a key tile (dK/dV) are split
+// over two workgroups, which fills the device and costs merges, partial sums and a second pass over
+// K / V.  Beside kernels of other streams (KR_ATTN_BESIDE_OTHER_STREAMS), which use the compute
+// units a launch leaves idle, its compute-unit time counts instead: the unsplit forms, whatever the
+// number of workgroups.
+struct AttnForms {
+  bool shared_fwd, shared_dq;
+  int qsplit;
+};
+static AttnForms attn_forms(int s, int b, int nq, int flags) {
+  const bool beside = (flags & KR_ATTN_BESIDE_OTHER_STREAMS) != 0;
+  const int tiles256 = (s / 256) * nq * b;
+  AttnForms f;
+  f.shared_fwd = s % 256 == 0 && (beside || tiles256 >= kr_compute_units());
+  f.shared_dq = s % 256 == 0 && (beside || tiles256 >= kr_compute_units()) && 2 * tiles256 <= KR_DQ_SHARED_MAX;
+  f.qsplit = beside ? 1 : dkdv_query_split(s, b, nq);
+  return f;
+}
+
+static int attn_bwd_impl(const void* dout, const void* q, const void* k, const void* v,
                            const void* o, const float* lse, void* dq, void* dk, void* dv,
                            void* workspace, int s, int b, int nq, int nkv, int hd, float scale,
                            int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss,
@@ -1694,7 +1714,8 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
                            int64_t o_ss, int64_t o_sb, int64_t o_sg, int64_t o_sh, int64_t do_ss,
                            int64_t do_sb, int64_t do_sg, int64_t do_sh, int64_t dq_ss, int64_t dq_sb,
                            int64_t dq_sg, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh,
-                           int64_t dv_ss, int64_t dv_sb, int64_t dv_sh, void* stream) {
+                           int64_t dv_ss, int64_t dv_sb, int64_t dv_sh, int flags, void* stream) {
+  if (flags & ~KR_ATTN_BESIDE_OTHER_STREAMS) return KR_EINVAL;
   if (!dout || !q || !k || !v || !o || !lse || !dq || !dk || !dv || !workspace) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
@@ -1735,7 +1756,8 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   const int64_t rows = (int64_t)b * nq * s;
   float* neg_lse2 = delta + rows;
   float* part_k = neg_lse2 + rows;
-  const int qsplit = dkdv_query_split(s, b, nq);
+  const AttnForms forms = attn_forms(s, b, nq, flags);
+  const int qsplit = forms.qsplit;
   float* part_v = part_k + rows * qsplit * hd;
   // query heads of a KV group per dK/dV workgroup: as many as leave two workgroups per compute
   // unit (KR_DKDV_HPW_MAX: a build-time cap, for measurements)
@@ -1795,8 +1817,8 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
 #undef KR_DKDV_LAUNCH
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int dq_blocks = (s / BQ) * nq * b;
-  if (s % 256 == 0 && dq_blocks / 2 >= kr_compute_units() && dq_blocks <= KR_DQ_SHARED_MAX) {
-    // a 256-query tile for every compute unit: the halves share their K / V tiles
+  if (forms.shared_dq) {
+    // 256-query tiles (one for every compute unit, or other streams beside): the halves share their K / V tiles
     hipLaunchKernelGGL((attn_bwd_dq_kernel<2, true>), dim3(dq_blocks / 2), dim3(512), lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
@@ -1815,11 +1837,41 @@ extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const
   return kr_launch_status();
 }
 
-extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
+extern "C" int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                           const void* o, const float* lse, void* dq, void* dk, void* dv,
+                           void* workspace, int s, int b, int nq, int nkv, int hd, float scale,
+                           int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss,
+                           int64_t k_sb, int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh,
+                           int64_t o_ss, int64_t o_sb, int64_t o_sg, int64_t o_sh, int64_t do_ss,
+                           int64_t do_sb, int64_t do_sg, int64_t do_sh, int64_t dq_ss, int64_t dq_sb,
+                           int64_t dq_sg, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh,
+                           int64_t dv_ss, int64_t dv_sb, int64_t dv_sh, void* stream) {
+  return attn_bwd_impl(dout, q, k, v, o, lse, dq, dk, dv, workspace, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg,
+                       q_sh, k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, do_ss, do_sb, do_sg,
+                       do_sh, dq_ss, dq_sb, dq_sg, dq_sh, dk_ss, dk_sb, dk_sh, dv_ss, dv_sb, dv_sh, 0, stream);
+}
+
+extern "C" int kr_attn_bwd_flags(const void* dout, const void* q, const void* k, const void* v,
+                                 const void* o, const float* lse, void* dq, void* dk, void* dv,
+                                 void* workspace, int s, int b, int nq, int nkv, int hd, float scale,
+                                 int64_t q_ss, int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss,
+                                 int64_t k_sb, int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh,
+                                 int64_t o_ss, int64_t o_sb, int64_t o_sg, int64_t o_sh, int64_t do_ss,
+                                 int64_t do_sb, int64_t do_sg, int64_t do_sh, int64_t dq_ss,
+                                 int64_t dq_sb, int64_t dq_sg, int64_t dq_sh, int64_t dk_ss,
+                                 int64_t dk_sb, int64_t dk_sh, int64_t dv_ss, int64_t dv_sb,
+                                 int64_t dv_sh, int flags, void* stream) {
+  return attn_bwd_impl(dout, q, k, v, o, lse, dq, dk, dv, workspace, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg,
+                       q_sh, k_ss, k_sb, k_sh, v_ss, v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, do_ss, do_sb, do_sg,
+                       do_sh, dq_ss, dq_sb, dq_sg, dq_sh, dk_ss, dk_sb, dk_sh, dv_ss, dv_sb, dv_sh, flags, stream);
+}
+
+static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse, int s,
                            int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
                            int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
                            int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
-                           int64_t o_sg, int64_t o_sh, void* stream) {
+                           int64_t o_sg, int64_t o_sh, int flags, void* stream) {
+  if (flags & ~KR_ATTN_BESIDE_OTHER_STREAMS) return KR_EINVAL;
   if (!q || !k || !v || !o || !lse) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
@@ -1841,8 +1893,8 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
                        lse, s, nq, nkv, hd, scale, ql, kl, vl, ol);
     return kr_launch_status();
   }
-  if (s % 256 == 0 && (s / 256) * nq * b >= kr_compute_units()) {
-    // enough 256-query tiles for every compute unit: the halves share their K / V tiles
+  if (attn_forms(s, b, nq, flags).shared_fwd) {
+    // 256-query tiles (one for every compute unit, or other streams beside): the halves share their K / V tiles
     constexpr size_t lds_sh = 3 * 16 * ((1024 + 16) + (1024 + 64));  // 100 KiB
     static const hipError_t attr_sh = hipFuncSetAttribute(
         (const void*)attn_fwd_sh_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_sh);
@@ -1868,3 +1920,20 @@ extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o,
   return kr_launch_status();
 }
 
+extern "C" int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse, int s,
+                           int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
+                           int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
+                           int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
+                           int64_t o_sg, int64_t o_sh, void* stream) {
+  return attn_fwd_impl(q, k, v, o, lse, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, 0, stream);
+}
+
+extern "C" int kr_attn_fwd_flags(const void* q, const void* k, const void* v, void* o, float* lse,
+                                 int s, int b, int nq, int nkv, int hd, float scale, int64_t q_ss,
+                                 int64_t q_sb, int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb,
+                                 int64_t k_sh, int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss,
+                                 int64_t o_sb, int64_t o_sg, int64_t o_sh, int flags, void* stream) {
+  return attn_fwd_impl(q, k, v, o, lse, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, flags, stream);
+}

@@ -217,7 +217,6 @@ __global__ __launch_bounds__(kDgammaThreads) void rmsnorm_dgamma_kernel(const fl
   }
 }
 
-// rows wider than 4096 elements are shared by two waves
 // Rows wider than this are shared by two waves (half the registers per wave, twice the waves per
 // SIMD to hide the latency of a row's loads behind)
 #ifndef KR_RMS_SPLIT_ABOVE

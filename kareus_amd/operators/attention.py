@@ -39,6 +39,10 @@ class TEDotProductAttentionOp(BasicOperation, PartitionableOperator):
         self.layer_number = layer_number
         self.softmax_scale = softmax_scale
         self._backend_name = backend
+        # True: the attention launches take their unsplit forms whatever the batch (KR_ATTN_BESIDE_OTHER_STREAMS),
+        # so a sequence gets the same bits in a nanobatch as in the whole microbatch.  Off by default: in the
+        # nanobatched step of the 8B shard the two choices time the same (5.64-5.66 against 5.68-5.70 ms).
+        self.beside_other_streams = False
 
     def get_input_channels(self) -> List[Channel]:
         return [Channel(0, "main"), Channel(1, "key"), Channel(2, "value")]
@@ -57,7 +61,8 @@ class TEDotProductAttentionOp(BasicOperation, PartitionableOperator):
             raise ValueError("query heads must be a multiple of KV heads")
         scale = self.softmax_scale if self.softmax_scale is not None else 1.0 / math.sqrt(hd)
         ctx = basic_op_ctxs[0]
-        out, lse = get_backend(self._backend_name).attn_fwd(q, key, value, scale, True)
+        out, lse = get_backend(self._backend_name).attn_fwd(q, key, value, scale, True,
+                                                            beside_other_streams=self.beside_other_streams)
         if ctx.requires_grad:
             ctx.save_for_backward(q, key, value, out, lse)
             ctx.scale = scale
@@ -67,6 +72,6 @@ class TEDotProductAttentionOp(BasicOperation, PartitionableOperator):
         ctx = basic_op_ctxs[0]
         q, key, value, out, lse = ctx.saved_tensors
         dq, dk, dv = get_backend(self._backend_name).attn_bwd(
-            grad_output, q, key, value, out, lse, ctx.scale, True
+            grad_output, q, key, value, out, lse, ctx.scale, True, beside_other_streams=self.beside_other_streams
         )
         return dq, [()], [(dk, dv)]

@@ -324,6 +324,40 @@ def test_attention_does_not_depend_on_the_launch_size(be):
         assert rel(dq_all[:, sl], dq1) <= 1e-2 and rel(dk_all[:, sl], dk1) <= 1e-2 and rel(dv_all[:, sl], dv1) <= 1e-2
 
 
+@pytest.mark.parametrize("s,b,nq,nkv", [(512, 1, 8, 2), (768, 2, 4, 4), (256, 1, 6, 2), (384, 1, 2, 1), (1024, 1, 24, 8)])
+def test_attention_beside_other_streams(be, s, b, nq, nkv):
+    """The forms the engine launches on its nanobatch streams (KR_ATTN_BESIDE_OTHER_STREAMS: whole rows and whole
+    key tiles per workgroup whatever their number; a length that is not a multiple of 256 keeps the 128-query
+    forms): against the fp32 oracle like the default forms, the same bits on every call, and — unlike the default
+    forms, which pick a variant by workgroup count — the same bits for a sequence whatever the batch around it."""
+    hd = 128
+    _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=222)
+    do = rnd(s, b, nq, hd, seed=223)
+    o, lse = be.attn_fwd(q, k, v, hd ** -0.5, beside_other_streams=True)
+    qf, kf, vf = (t.float().cpu().clone().requires_grad_(True) for t in (q.flatten(2, 3), k, v))
+    ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
+    assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
+    ro.backward(do.float().cpu())
+    dq, dk, dv = be.attn_bwd(do, q, k, v, o, lse, hd ** -0.5, beside_other_streams=True)
+    assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
+    again = be.attn_bwd(do, q, k, v, o, lse, hd ** -0.5, beside_other_streams=True)
+    assert all(torch.equal(x, y) for x, y in zip(again, (dq, dk, dv)))
+    # against the default forms: equal to rounding
+    o0, lse0 = be.attn_fwd(q, k, v, hd ** -0.5)
+    assert rel(o, o0) <= 1e-2 and rel(lse, lse0) <= 1e-5
+    # a batch of 40 such sequences (enough tiles for every compute unit) gives each of them the same bits
+    if s % 256 == 0 and nq == 8:
+        big = 40
+        qb, kb, vb = (t.repeat_interleave(big, dim=1) for t in (q, k, v))
+        ob, lseb = be.attn_fwd(qb, kb, vb, hd ** -0.5, beside_other_streams=True)
+        assert torch.equal(ob[:, 7:8], o) and torch.equal(lseb[7:8], lse)
+        ob2, _ = be.attn_fwd(qb, kb, vb, hd ** -0.5)            # alone on the GPU it takes the same form
+        assert torch.equal(ob2, ob)
+        dob = do.repeat_interleave(big, dim=1)
+        dqb, dkb, dvb = be.attn_bwd(dob, qb, kb, vb, ob, lseb, hd ** -0.5, beside_other_streams=True)
+        assert torch.equal(dqb[:, 7:8], dq)
+
+
 def test_attention_special_cases(be):
     hd, s = 128, 256
     # all keys equal -> output row i is the mean of v[0..i]
