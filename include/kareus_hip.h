@@ -101,6 +101,29 @@ int kr_gemm_bf16_fused(int layout, int M, int N, int K,
                        int epilogue, const void* aux, int64_t ld_aux, void* out2, int64_t ld_out2,
                        int max_cus, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Row runs.  A nanobatch of r sequences cut out of a [seq, batch, hidden] tensor along the batch axis
+ * (kareus/megatron/core/transformer/transformer_block.py:483-485) is not a matrix with one row
+ * stride: its rows come in runs of r consecutive rows (stride hidden) whose starts are batch*hidden
+ * elements apart.  The reference copies such a slice into a dense tensor in every linear layer
+ * (kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:565-569).  The *_runs entry points
+ * address it in place: row i of an operand with `run_rows` rows per run and run starts `run_ld`
+ * elements apart sits at (i / run_rows) * run_ld + (i % run_rows) * ld.  run_rows: a power of two that
+ * divides the operand's row count, 1 for a plain matrix (run_ld is then ignored); run_ld: a multiple
+ * of 8.
+ * kr_gemm_bf16_runs = kr_gemm_bf16_fused with runs for A, C and aux, run_rows at most 16, for the
+ * launches at the two ends of a layer stack: layout TN with the residual-add epilogue (aux and / or C
+ * in runs: the block's input as residual, the block's output as destination), layout NN plain or with
+ * the SwiGLU-backward epilogue and layout NT (A in runs: the block's incoming gradient; for NT the rows
+ * of A are the contraction index).  An output in runs is never accumulated into or cut along K.
+ * Anything else in runs returns KR_EUNSUPPORTED.                                                   */
+int kr_gemm_bf16_runs(int layout, int M, int N, int K,
+                      const void* A, int64_t lda, int a_run_rows, int64_t a_run_ld,
+                      const void* B, int64_t ldb,
+                      void* C, int64_t ldc, int c_run_rows, int64_t c_run_ld, int accumulate,
+                      int epilogue, const void* aux, int64_t ld_aux, int aux_run_rows, int64_t aux_run_ld,
+                      void* out2, int64_t ld_out2,
+                      int max_cus, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- RMSNorm ---------------------------------------------------------------------------
  * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd
  * (kareus/transformer_engine/pytorch/ops/basic/rmsnorm.py:210-219, 256-263).
@@ -113,6 +136,11 @@ int kr_gemm_bf16_fused(int layout, int M, int N, int K,
  *      dgamma = sum over rows of dy * xhat.  workspace: kr_rmsnorm_bwd_workspace_bytes().  */
 int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd,
                    int rows, int cols, int64_t x_ld, float eps, void* stream);
+/* kr_rmsnorm_fwd on an input whose rows come in runs (see "Row runs" above; same call of the
+ * reference, rmsnorm.py:210-219, fed a nanobatch of several sequences without the copy).        */
+int kr_rmsnorm_fwd_runs(const void* x, const void* gamma, void* y, float* rstd,
+                        int rows, int cols, int64_t x_ld, int x_run_rows, int64_t x_run_ld,
+                        float eps, void* stream);
 size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols);
 int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
                    void* dx, void* dgamma, void* workspace, int rows, int cols,
@@ -125,6 +153,15 @@ int kr_rmsnorm_bwd(const void* dy, const void* x, const float* rstd, const void*
 int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd, const void* gamma,
                        const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
                        int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
+/* kr_rmsnorm_bwd_add where the saved input x, the residual gradient dres and / or the result dx are
+ * nanobatches of several sequences used in place (rows in runs, see "Row runs" above;
+ * rmsnorm.py:256-263 and residual_fork.py:104-106 without the copies in and out).               */
+int kr_rmsnorm_bwd_add_runs(const void* dy, const void* x, const float* rstd, const void* gamma,
+                            const void* dres, void* dx, void* dgamma, void* workspace,
+                            int rows, int cols, int64_t dy_ld,
+                            int64_t x_ld, int x_run_rows, int64_t x_run_ld,
+                            int64_t dres_ld, int dres_run_rows, int64_t dres_run_ld,
+                            int64_t dx_ld, int dx_run_rows, int64_t dx_run_ld, void* stream);
 
 /* Weight gradient of one RMSNorm over several nanobatches of a microbatch, summed in fp32 and
  * rounded once (the reference lets autograd add the per-nanobatch bf16 gradients,

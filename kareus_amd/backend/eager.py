@@ -35,6 +35,20 @@ class EagerBackend:
     def can_fuse_swiglu(two_f: int) -> bool:
         return two_f % 2 == 0
 
+    # the eager ops take [rows, cols] matrices; anything a view cannot express is copied
+    supports_row_runs = False
+
+    @staticmethod
+    def rows_view(t: Tensor):
+        try:
+            return t.view(-1, t.shape[-1])
+        except RuntimeError:
+            return None
+
+    @staticmethod
+    def rows_in_place(t: Tensor) -> Tensor:
+        return t.reshape(-1, t.shape[-1])
+
     def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True, swiglu_bwd_x: Tensor = None) -> Tensor:
         g = dy @ w
         return g if swiglu_bwd_x is None else self.swiglu_bwd(g, swiglu_bwd_x)

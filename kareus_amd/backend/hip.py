@@ -33,7 +33,14 @@ _SIGNATURES = {
     "kr_gemm_bf16_fused": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
                                     _c_void_p, _c_i64, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
                                     _c_int, _c_void_p, _c_size_t, _c_void_p]),
+    "kr_gemm_bf16_runs": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p, _c_i64,
+                                   _c_void_p, _c_i64, _c_int, _c_i64, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64,
+                                   _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
+    "kr_rmsnorm_fwd_runs": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_int, _c_i64,
+                                     _c_float, _c_void_p]),
+    "kr_rmsnorm_bwd_add_runs": (_c_int, [_c_void_p] * 8 + [_c_int, _c_int, _c_i64, _c_i64, _c_int, _c_i64, _c_i64, _c_int,
+                                                           _c_i64, _c_i64, _c_int, _c_i64, _c_void_p]),
     "kr_rmsnorm_bwd_workspace_bytes": (_c_size_t, [_c_int, _c_int]),
     "kr_rmsnorm_bwd": (_c_int, [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_rmsnorm_bwd_add": (_c_int, [_c_void_p] * 8 + [_c_int, _c_int] + [_c_i64] * 4 + [_c_void_p]),
@@ -124,6 +131,57 @@ class HipBackend:
             if t.dtype != torch.bfloat16:
                 raise RuntimeError(f"the hip backend computes in bf16, got {t.dtype}")
 
+    # -- row runs ---------------------------------------------------------------------
+    # A nanobatch of r sequences of a [s, b, h] tensor is a [s, r, h] view with strides (b*h, h, 1): its
+    # rows come in runs of r (stride h) whose starts are b*h apart.  The *_runs entry points address it
+    # in place; r has to be a power of two (at most MAX_RUN_ROWS for the GEMM).
+    supports_row_runs = True
+    MAX_RUN_ROWS = 16
+
+    @staticmethod
+    def _operand(t: Tensor):
+        """``(rows, ld, run_rows, run_ld)`` of a [rows, cols] matrix or a [s, r, cols] run tensor that the
+        kernels address in place, or None when ``t`` has to be copied."""
+        if t.stride(-1) != 1:
+            return None
+        cols = t.shape[-1]
+        if t.dim() == 2:
+            ld = t.stride(0)
+            return (t.shape[0], ld, 1, 0) if (ld % 8 == 0 and ld >= cols) or t.shape[0] == 1 else None
+        if t.dim() != 3:
+            return None
+        s_, r, _ = t.shape
+        outer, ld = t.stride(0), t.stride(1)
+        if r == 1:
+            return (s_, outer, 1, 0) if outer % 8 == 0 and outer >= cols else None
+        if ld % 8 or ld < cols or outer % 8:
+            return None
+        if outer == r * ld or s_ == 1:
+            return (s_ * r, ld, 1, 0)
+        if r & (r - 1) or r > HipBackend.MAX_RUN_ROWS or outer < r * ld:
+            return None
+        return (s_ * r, ld, r, outer)
+
+    def rows_view(self, t: Tensor):
+        """``t`` ([..., cols]) as the kernels can address it in place: a [rows, cols] view when its rows have
+        one stride, ``t`` itself when it is a [s, r, cols] tensor whose rows come in runs; None when only a
+        copy would do."""
+        cols = t.shape[-1]
+        try:
+            m = t.view(-1, cols)
+            if self._operand(m) is not None:
+                return m
+        except RuntimeError:
+            pass
+        if t.dim() == 3 and self._operand(t) is not None:
+            return t
+        return None
+
+    def rows_in_place(self, t: Tensor) -> Tensor:
+        """``rows_view(t)``, or a dense [rows, cols] copy when the kernels cannot address ``t`` as it lies."""
+        v = self.rows_view(t)
+        return v if v is not None else t.reshape(-1, t.shape[-1]).contiguous()
+
     # -- GEMM -------------------------------------------------------------------------
     def _num_cus(self, device) -> int:
         n = self._cu_count.get(device.index)
@@ -159,6 +217,9 @@ class HipBackend:
         self._bf16(a, b)
         if a.stride(-1) != 1 or b.stride(-1) != 1:
             raise RuntimeError("GEMM operands must have a contiguous last dimension")
+        a_op = self._operand(a)
+        if a_op is None or b.dim() != 2:
+            raise RuntimeError("GEMM operands must be matrices with one row stride (A may have row runs)")
         if out is None:
             out = torch.empty((m, 2 * n if swiglu_bwd_x is not None else n), dtype=torch.bfloat16, device=a.device)
         epi, aux_ptr, aux_ld, out2_ptr, out2_ld = 0, None, 0, None, 0
@@ -170,12 +231,14 @@ class HipBackend:
             if tuple(swiglu_bwd_x.shape) != (m, 2 * n) or swiglu_bwd_x.stride(1) != 1 or tuple(out.shape) != (m, 2 * n):
                 raise RuntimeError("swiglu_bwd_x and out must be [M, 2N] with a contiguous last dimension")
             epi, aux_ptr, aux_ld = 4, swiglu_bwd_x.data_ptr(), swiglu_bwd_x.stride(0)
+        aux_op = None
         if residual is not None:
             self._dev(residual)
             self._bf16(residual)
-            if tuple(residual.shape) != (m, n) or residual.stride(1) != 1:
-                raise RuntimeError("GEMM residual must be [M, N] with a contiguous last dimension")
-            epi, aux_ptr, aux_ld = 1, residual.data_ptr(), residual.stride(0)
+            aux_op = self._operand(residual)
+            if aux_op is None or aux_op[0] != m or residual.shape[-1] != n:
+                raise RuntimeError("GEMM residual must be [M, N] (or [s, r, N] in row runs) with a contiguous last dimension")
+            epi, aux_ptr, aux_ld = 1, residual.data_ptr(), aux_op[1]
         if swiglu_out is not None:
             if residual is not None:
                 raise RuntimeError("one fused epilogue at a time")
@@ -201,13 +264,24 @@ class HipBackend:
                 max_cus = max(self._num_cus(a.device) - reserved, 8)
         if split_k is False:
             epi |= 0x100   # KR_GEMM_BESIDE_OTHER_STREAMS
-        if epi == 0 and max_cus == 0:
-            rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0),
-                                       out.data_ptr(), out.stride(0), int(accumulate), ws_ptr, ws_bytes,
+        c_op = self._operand(out)
+        if c_op is None or c_op[0] != m:
+            raise RuntimeError("GEMM output must be [M, ...] with one row stride (or [s, r, ...] in row runs)")
+        lda, ldc = a_op[1], c_op[1]
+        if a_op[2] > 1 or c_op[2] > 1 or (aux_op is not None and aux_op[2] > 1):
+            if c_op[2] > 1:
+                ws_ptr, ws_bytes = None, 0      # an output in row runs is stored by the GEMM itself: no cuts
+            rc = self.lib.kr_gemm_bf16_runs(layout, m, n, k, a.data_ptr(), lda, a_op[2], a_op[3], b.data_ptr(),
+                                            b.stride(0), out.data_ptr(), ldc, c_op[2], c_op[3], int(accumulate),
+                                            epi, aux_ptr, aux_ld, aux_op[2] if aux_op else 1, aux_op[3] if aux_op else 0,
+                                            out2_ptr, out2_ld, int(max_cus), ws_ptr, ws_bytes, self._stream())
+        elif epi == 0 and max_cus == 0:
+            rc = self.lib.kr_gemm_bf16(layout, m, n, k, a.data_ptr(), lda, b.data_ptr(), b.stride(0),
+                                       out.data_ptr(), ldc, int(accumulate), ws_ptr, ws_bytes,
                                        self._stream())
         else:
-            rc = self.lib.kr_gemm_bf16_fused(layout, m, n, k, a.data_ptr(), a.stride(0), b.data_ptr(),
-                                             b.stride(0), out.data_ptr(), out.stride(0), int(accumulate),
+            rc = self.lib.kr_gemm_bf16_fused(layout, m, n, k, a.data_ptr(), lda, b.data_ptr(),
+                                             b.stride(0), out.data_ptr(), ldc, int(accumulate),
                                              epi, aux_ptr, aux_ld, out2_ptr, out2_ld, int(max_cus),
                                              ws_ptr, ws_bytes, self._stream())
         self._check(rc, f"kr_gemm_bf16(layout={layout}, M={m}, N={n}, K={k}, epilogue={epi & 0xff})")
@@ -215,8 +289,12 @@ class HipBackend:
 
     def linear_fwd(self, x: Tensor, w: Tensor, split_k: bool = True, out: Tensor = None,
                    residual: Tensor = None, swiglu_out: Tensor = None, max_cus: int = 0) -> Tensor:
-        return self.gemm(KR_GEMM_TN, x, w, x.shape[0], w.shape[0], x.shape[1], out=out, split_k=split_k,
+        return self.gemm(KR_GEMM_TN, x, w, self._nrows(x), w.shape[0], x.shape[-1], out=out, split_k=split_k,
                          residual=residual, swiglu_out=swiglu_out, max_cus=max_cus)
+
+    @staticmethod
+    def _nrows(t: Tensor) -> int:
+        return t.shape[0] if t.dim() == 2 else t.shape[0] * t.shape[1]
 
     @staticmethod
     def can_fuse_swiglu(two_f: int) -> bool:
@@ -226,14 +304,14 @@ class HipBackend:
     def linear_dgrad(self, dy: Tensor, w: Tensor, split_k: bool = True, swiglu_bwd_x: Tensor = None) -> Tensor:
         """``dy . W``; with ``swiglu_bwd_x`` (the input of the SwiGLU activation that fed this layer) the
         result is the gradient of that input, [rows, 2 * in_features], computed in the GEMM's epilogue."""
-        return self.gemm(KR_GEMM_NN, dy, w, dy.shape[0], w.shape[1], dy.shape[1], split_k=split_k,
+        return self.gemm(KR_GEMM_NN, dy, w, self._nrows(dy), w.shape[1], dy.shape[-1], split_k=split_k,
                          swiglu_bwd_x=swiglu_bwd_x)
 
     can_fuse_swiglu_bwd = True
 
     def linear_wgrad(self, dy: Tensor, x: Tensor, out: Tensor = None, accumulate: bool = False,
                      split_k: bool = True) -> Tensor:
-        return self.gemm(KR_GEMM_NT, dy, x, dy.shape[1], x.shape[1], dy.shape[0], out=out,
+        return self.gemm(KR_GEMM_NT, dy, x, dy.shape[-1], x.shape[1], self._nrows(dy), out=out,
                          accumulate=accumulate, split_k=split_k)
 
     # -- RMSNorm ----------------------------------------------------------------------
@@ -246,14 +324,24 @@ class HipBackend:
         return t.contiguous()
 
     def rmsnorm_fwd(self, x: Tensor, gamma: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+        """``x``: [rows, cols], or a [s, r, cols] nanobatch slice whose rows come in runs (read in place).
+        Returns the dense [rows, cols] result and rstd [rows]."""
         self._dev(x, gamma)
         self._bf16(x, gamma)
-        x = self._rows(x)
-        rows, cols = x.shape
+        op = self._operand(x)
+        if op is None:
+            x = x.reshape(-1, x.shape[-1]).contiguous()
+            op = self._operand(x)
+        rows, ld, run_rows, run_ld = op
+        cols = x.shape[-1]
         y = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
-        rc = self.lib.kr_rmsnorm_fwd(x.data_ptr(), gamma.data_ptr(), y.data_ptr(), rstd.data_ptr(),
-                                     rows, cols, x.stride(0), eps, self._stream())
+        if run_rows > 1:
+            rc = self.lib.kr_rmsnorm_fwd_runs(x.data_ptr(), gamma.data_ptr(), y.data_ptr(), rstd.data_ptr(),
+                                              rows, cols, ld, run_rows, run_ld, eps, self._stream())
+        else:
+            rc = self.lib.kr_rmsnorm_fwd(x.data_ptr(), gamma.data_ptr(), y.data_ptr(), rstd.data_ptr(),
+                                         rows, cols, ld, eps, self._stream())
         self._check(rc, "kr_rmsnorm_fwd")
         return y, rstd
 
@@ -278,24 +366,35 @@ class HipBackend:
         left there as partial rows for ``rmsnorm_dgamma`` and None is returned in its place."""
         self._dev(dy, x, rstd, gamma)
         self._bf16(dy, x, gamma)
-        x, dy = self._rows(x), self._rows(dy)
-        rows, cols = x.shape
+        dy = self._rows(dy)
+        x_op = self._operand(x)
+        if x_op is None:
+            x = x.reshape(-1, x.shape[-1]).contiguous()
+            x_op = self._operand(x)
+        rows, cols = x_op[0], x.shape[-1]
+        if tuple(dy.shape) != (rows, cols):
+            raise RuntimeError("rmsnorm_bwd: dy must be [rows, cols] like x")
         if out is None:
             dx = torch.empty((rows, cols), dtype=x.dtype, device=x.device)
+            dx_op = (rows, cols, 1, 0)
         else:
             self._dev(out)
             self._bf16(out)
             dx = out
-            if dx.shape != x.shape or dx.stride(1) != 1 or dx.stride(0) % 8 or dx.stride(0) < cols:
-                raise RuntimeError("rmsnorm_bwd: out must be [rows, cols] with a single row stride")
-        res_ptr, res_ld = None, 0
+            dx_op = self._operand(dx)
+            if dx_op is None or dx_op[0] != rows or dx.shape[-1] != cols:
+                raise RuntimeError("rmsnorm_bwd: out must be [rows, cols] with a single row stride, or in row runs")
+        res_ptr, res_op = None, (rows, 0, 1, 0)
         if residual_grad is not None:
             self._dev(residual_grad)
             self._bf16(residual_grad)
-            if residual_grad.shape != x.shape:
+            res_op = self._operand(residual_grad)
+            if res_op is None:
+                residual_grad = residual_grad.reshape(-1, cols).contiguous()
+                res_op = self._operand(residual_grad)
+            if res_op[0] != rows or residual_grad.shape[-1] != cols:
                 raise RuntimeError("rmsnorm_bwd: residual_grad must have the shape of x")
-            residual_grad = self._rows(residual_grad)
-            res_ptr, res_ld = residual_grad.data_ptr(), residual_grad.stride(0)
+            res_ptr = residual_grad.data_ptr()
         if partials_out is not None:
             if (partials_out.dtype != torch.float32 or not partials_out.is_contiguous()
                     or tuple(partials_out.shape) != (self.rmsnorm_partial_rows(rows, cols), cols)):
@@ -305,9 +404,15 @@ class HipBackend:
             dgamma = torch.empty_like(gamma)
             dg_ptr = dgamma.data_ptr()
             ws = self._workspace(self.lib.kr_rmsnorm_bwd_workspace_bytes(rows, cols), x.device)
-        rc = self.lib.kr_rmsnorm_bwd_add(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
-                                         res_ptr, dx.data_ptr(), dg_ptr, ws.data_ptr(), rows, cols,
-                                         dy.stride(0), x.stride(0), res_ld, dx.stride(0), self._stream())
+        if x_op[2] > 1 or res_op[2] > 1 or dx_op[2] > 1:
+            rc = self.lib.kr_rmsnorm_bwd_add_runs(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+                                                  res_ptr, dx.data_ptr(), dg_ptr, ws.data_ptr(), rows, cols,
+                                                  dy.stride(0), x_op[1], x_op[2], x_op[3], res_op[1], res_op[2],
+                                                  res_op[3], dx_op[1], dx_op[2], dx_op[3], self._stream())
+        else:
+            rc = self.lib.kr_rmsnorm_bwd_add(dy.data_ptr(), x.data_ptr(), rstd.data_ptr(), gamma.data_ptr(),
+                                             res_ptr, dx.data_ptr(), dg_ptr, ws.data_ptr(), rows, cols,
+                                             dy.stride(0), x_op[1], res_op[1], dx_op[1], self._stream())
         self._check(rc, "kr_rmsnorm_bwd_add")
         return dx, dgamma
 

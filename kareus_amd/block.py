@@ -88,10 +88,14 @@ class LayerConfig:
         return (self.num_attention_heads + 2 * self.num_query_groups) * self.kv_channels
 
 
-def _dense_batch_slices(parts) -> bool:
-    """Whether a nanobatch of this width must be copied: only a nanobatch of one sequence (a
-    matrix with row stride ``b*h``) can be addressed by every kernel without a copy."""
-    return any(p.shape[1] > 1 or p.stride(2) != 1 or p.stride(0) % 8 for p in parts)
+def _dense_batch_slices(parts, backend: str = "eager") -> bool:
+    """Whether nanobatch slices of this width must be copied.  A nanobatch of one sequence is a matrix
+    with row stride ``b*h``; one of 2, 4, 8 or 16 sequences has its rows in runs, which the HIP kernels
+    at the two ends of a layer stack address in place (``rows_view``); anything else is copied once."""
+    from .backend import get_backend
+
+    view = get_backend(backend).rows_view
+    return any(view(p) is None for p in parts)
 
 
 def _whole_of(parts):
@@ -125,17 +129,17 @@ class _SplitNanobatches(torch.autograd.Function):
     (one copy instead of autograd's zero-fill + copy + add per slice)."""
 
     @staticmethod
-    def forward(ctx, hidden_states, n):
+    def forward(ctx, hidden_states, n, backend="eager"):
         nb = hidden_states.shape[1] // n
         parts = [hidden_states[:, i * nb:(i + 1) * nb] for i in range(n)]
-        if _dense_batch_slices(parts):
+        if _dense_batch_slices(parts, backend):
             parts = [p.contiguous() for p in parts]
         return tuple(parts)
 
     @staticmethod
     def backward(ctx, *grads):
         whole = _whole_of(grads)
-        return (whole if whole is not None else torch.cat(grads, dim=1)), None
+        return (whole if whole is not None else torch.cat(grads, dim=1)), None, None
 
 
 class _JoinNanobatches(torch.autograd.Function):
@@ -145,8 +149,9 @@ class _JoinNanobatches(torch.autograd.Function):
     gradient the way ``_SplitNanobatches`` slices the input."""
 
     @staticmethod
-    def forward(ctx, *outs):
+    def forward(ctx, backend, *outs):
         ctx.widths = [o.shape[1] for o in outs]
+        ctx.backend = backend
         whole = _whole_of(outs)
         return whole if whole is not None else torch.cat(outs, dim=1)
 
@@ -158,9 +163,9 @@ class _JoinNanobatches(torch.autograd.Function):
         for w in ctx.widths:
             parts.append(grad[:, lo:lo + w])
             lo += w
-        if _dense_batch_slices(parts):
+        if _dense_batch_slices(parts, ctx.backend):
             parts = [p.contiguous() for p in parts]
-        return tuple(parts)
+        return (None, *parts)
 
 
 class DecoderLayer(torch.nn.Module):
@@ -338,7 +343,7 @@ class LayerStack(torch.nn.Module):
         if rotary_pos_emb is None:
             rotary_pos_emb = self.rotary_pos_emb(s, device=hidden_states.device)
 
-        hs = _SplitNanobatches.apply(hidden_states, n) if n > 1 else (hidden_states,)
+        hs = _SplitNanobatches.apply(hidden_states, n, self.config.backend) if n > 1 else (hidden_states,)
         params = self._get_all_params()
         outs = TransformerBlockAutogradFunction.apply(
             *hs, rotary_pos_emb, None,
@@ -348,4 +353,4 @@ class LayerStack(torch.nn.Module):
             torch.is_grad_enabled(), self.config.checkpoint_activations,
             *(params * n),
         )
-        return outs[0] if n == 1 else _JoinNanobatches.apply(*outs)
+        return outs[0] if n == 1 else _JoinNanobatches.apply(self.config.backend, *outs)

@@ -103,10 +103,17 @@ __device__ __forceinline__ uint32_t lds_addr(const bf16* p) {
 // the first `half_rows` rows of the tile hold the gate rows row0 .., the next `half_rows` the up rows
 // of the same output columns, so that the waves of the tile's left half end up with gate values
 // and the waves of its right half with the matching up values.
+// Row runs.  The rows of an operand may come in runs of 2^sh consecutive rows (stride ld) whose starts
+// are `outer` elements apart: row r sits at (r >> sh) * outer + (r & (2^sh - 1)) * ld.  That is a
+// nanobatch of 2^sh sequences cut out of a [s, b, h] tensor along b, read in place.  A plain matrix
+// is sh = 0, outer = ld.
+__device__ __forceinline__ int run_off(int r, int ld, int sh, int outer) {
+  return (r >> sh) * outer + (r & ((1 << sh) - 1)) * ld;
+}
 template <bool TRANSPOSED>
 __device__ __forceinline__ uint32_t load_offset(int i, int wave, int lane, int ld, int row0,
                                                 int rows_total, int k_left, int gate_up_f = 0,
-                                                int half_rows = 0) {
+                                                int half_rows = 0, int sh = 0, int outer = 0) {
   if (!TRANSPOSED) {
     const int row = 8 * wave + (lane >> 3) + 32 * i;
     int chunk = ((lane & 7) ^ ((row >> 1) & 7)) * 8;
@@ -114,13 +121,15 @@ __device__ __forceinline__ uint32_t load_offset(int i, int wave, int lane, int l
     if (gate_up_f > 0) r = row < half_rows ? row0 + row : row0 + (row - half_rows) + gate_up_f;
     r = r < rows_total ? r : rows_total - 1;
     chunk = chunk + 8 <= k_left ? chunk : k_left - 8;
-    return (uint32_t)(r * ld + chunk);
+    return (uint32_t)((sh ? run_off(r, ld, sh, outer) : r * ld) + chunk);
   }
+  // (the contraction rows of a K-step start at a multiple of 64, hence of the run length: the
+  // position inside the K-step maps like a row of its own)
   int krow = 2 * wave + (lane >> 5) + 8 * i;
   int c = row0 + ((lane & 31) ^ transp_swz(krow)) * 8;
   c = c + 8 <= rows_total ? c : rows_total - 8;
   krow = krow < k_left ? krow : k_left - 1;
-  return (uint32_t)(krow * ld + c);
+  return (uint32_t)((sh ? run_off(krow, ld, sh, outer) : krow * ld) + c);
 }
 // contraction index (relative to the K-step) of the chunk that load i of this lane fills
 template <bool TRANSPOSED>
@@ -188,6 +197,12 @@ __device__ __forceinline__ void remap_block(int pid, int nblocks, int tiles_m, i
   tn = in_band / band_rows;
 }
 
+// Row runs of A, C and aux (see run_off): shift and distance between run starts; sh = 0 for a
+// plain matrix (the distance is then unused).
+struct RowRuns {
+  int a_sh, a_outer, c_sh, c_outer, x_sh, x_outer;
+};
+
 template <int WN>
 struct Frags {
   bf16x8 a[WT], b[WN];
@@ -200,14 +215,19 @@ struct Count { static constexpr int value = N; };
 // column; a K-major B tile then occupies the first 32 * WN rows of its slot and takes WN loads per wave.
 // EPI: the fused epilogue compiled into this instance (KR_GEMM_EPI_*).  A template parameter, not
 // a run-time switch: the plain instances carry none of the extra code or registers.
-template <bool A_T, bool B_T, int WN, int EPI>
+// RUNS: the instance honours row runs of A, C and aux (RowRuns); the plain instances do not carry the
+// extra address arithmetic or its registers.
+template <bool A_T, bool B_T, int WN, int EPI, bool RUNS = false>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
                                                         bf16* __restrict__ C, int ldc, int M,
                                                         int N, int K, int accumulate, int k_per,
                                                         int splits, float* __restrict__ partial,
                                                         const bf16* __restrict__ aux, int ld_aux,
-                                                        bf16* __restrict__ out2, int ld_out2) {
+                                                        bf16* __restrict__ out2, int ld_out2,
+                                                        RowRuns runs_arg) {
+  // (without RUNS every run length reads as a compile-time 1: the branches below fold away)
+  const RowRuns runs = RUNS ? runs_arg : RowRuns{0, 0, 0, 0, 0, 0};
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -256,7 +276,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       // split-K: contraction range [split*k_per, split*k_per + kc), fp32 partial tile out
       // (k_per is a multiple of 64)
       const int k0 = split * k_per;
-      a_off = A_T ? k0 * lda : k0;
+      a_off = A_T ? (runs.a_sh ? (k0 >> runs.a_sh) * runs.a_outer : k0 * lda) : k0;
       b_off = B_T ? k0 * ldb : k0;
       kc = (K - k0) < k_per ? (K - k0) : k_per;
       p_off = split * M * N;
@@ -264,7 +284,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     nk = (kc + BK - 1) / BK;
     k_tail = kc - (nk - 1) * BK;  // valid contraction rows of the last K-step (8..64)
   };
-  auto a_base = [&](int t) { return A + a_off + (int64_t)t * (A_T ? BK * lda : BK); };
+  const int a_step = A_T ? (runs.a_sh ? (BK >> runs.a_sh) * runs.a_outer : BK * lda) : BK;
+  auto a_base = [&](int t) { return A + a_off + (int64_t)t * a_step; };
   auto b_base = [&](int t) { return B + b_off + (int64_t)t * (B_T ? BK * ldb : BK); };
 
   // The ring of five 32 KB slots as LDS byte addresses, in ring order starting at A of the
@@ -288,7 +309,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     asm volatile("" : "+v"(l2));
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      la[i] = 2u * load_offset<A_T>(i, wave, l2, lda, m0, M, k_left);
+      la[i] = 2u * load_offset<A_T>(i, wave, l2, lda, m0, M, k_left, 0, 0, runs.a_sh, runs.a_outer);
       lb[i] = 2u * load_offset<B_T>(i, wave, l2, ldb, n0, N, k_left, gate_up_f, 16 * WN);
     }
   };
@@ -546,7 +567,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       const bool ncols_in = 8 * rch < 16 * WN && (swiglu || n_wave + 8 * rch < N);
       uint32_t nlo[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) nlo[q] = (uint32_t)((4 * q + quad) * ldc + ncol);
+      for (int q = 0; q < 4; ++q)   // (a 16-row block starts at a multiple of the run length: rows map inside it)
+        nlo[q] = (uint32_t)((runs.c_sh ? run_off(4 * q + quad, ldc, runs.c_sh, runs.c_outer) : (4 * q + quad) * ldc) + ncol);
       // fused residual: the values to add to a 16-row block are requested one block ahead
       // SwiGLU backward: gate and up values of a 16-row block, requested one block ahead
       bf16x8 xg[swiglu_bwd ? 2 : 1][swiglu_bwd ? 4 : 1], xu[swiglu_bwd ? 2 : 1][swiglu_bwd ? 4 : 1];
@@ -563,12 +585,15 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       if constexpr (swiglu_bwd) fetch_x(0);
       bf16x8 resv[epi_add ? 2 : 1][epi_add ? 4 : 1];
       auto fetch_res = [&](int mt) {
-        const bf16* const rb = aux + ((int64_t)(m_wave + mt * 16) * ld_aux + n_wave + 8 * rch);
+        const int r0 = m_wave + mt * 16;
+        const bf16* const rb =
+            aux + ((runs.x_sh ? (int64_t)(r0 >> runs.x_sh) * runs.x_outer : (int64_t)r0 * ld_aux) + n_wave + 8 * rch);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int rr = 4 * q + quad;
           const bool in = ncols_in && (rows_in || m_wave + mt * 16 + rr < M);
-          resv[mt & 1][q] = in ? ldg8(rb + (int64_t)rr * ld_aux) : zero8();
+          const int64_t ro = runs.x_sh ? (int64_t)run_off(rr, ld_aux, runs.x_sh, runs.x_outer) : (int64_t)rr * ld_aux;
+          resv[mt & 1][q] = in ? ldg8(rb + ro) : zero8();
         }
       };
       if constexpr (epi_add) fetch_res(0);
@@ -621,7 +646,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
           asm volatile("" : "+v"(vals[nt]));  // read here, not once in each branch below
           acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        const int64_t blk = (int64_t)(m_wave + mt * 16) * ldo + (narrow ? n_store : n_wave);
+        const int64_t blk = (narrow && runs.c_sh ? (int64_t)((m_wave + mt * 16) >> runs.c_sh) * runs.c_outer
+                                                 : (int64_t)(m_wave + mt * 16) * ldo) +
+                            (narrow ? n_store : n_wave);
         if (narrow) {
           const uint32_t buf = stage + (uint32_t)(mt & 1) * 4096u;
 #pragma unroll
@@ -820,6 +847,7 @@ struct Fused {
   int64_t ld_out2 = 0;
   int max_cus = 0;          // > 0: use at most this many compute units
   bool shared = false;      // other streams' kernels use the units this launch leaves idle
+  RowRuns runs = {0, 0, 0, 0, 0, 0};  // row runs of A, C, aux (all plain by default)
 };
 
 // Tile width for a projection with the SwiGLU epilogue: the tiles have to divide the 2F output
@@ -873,11 +901,31 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
     g = (g + 7) / 8 * 8;
     return g < num_cus ? g : num_cus;
   };
+  const bool with_runs = fu.runs.a_sh || fu.runs.c_sh || fu.runs.x_sh;
+  // instances that honour row runs exist for what the two ends of a layer stack launch: the residual-add
+  // forward (aux or C in runs), the input gradient (plain or with the SwiGLU backward) and the weight
+  // gradient (A in runs)
+  constexpr bool kRunsInstance = EPI == KR_GEMM_EPI_ADD || EPI == KR_GEMM_EPI_SWIGLU_BWD || (EPI == KR_GEMM_EPI_NONE && B_T);
+  if (with_runs && !kRunsInstance) return KR_EUNSUPPORTED;
+  if constexpr (kRunsInstance) {
+    static const hipError_t attr_runs =
+        hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN, EPI, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (with_runs && attr_runs != hipSuccess) return KR_ELAUNCH;
+  }
   if (splits == 1) {
     const int grid = grid_for(tiles);
+    if constexpr (kRunsInstance) {
+      if (with_runs) {
+        hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, EPI, true>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
+                           (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr,
+                           fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2, fu.runs);
+        return kr_launch_status();
+      }
+    }
     hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, EPI>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
                        (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr,
-                       fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2);
+                       fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2, fu.runs);
     return kr_launch_status();
   }
   int k_per = (K + splits - 1) / splits;
@@ -885,9 +933,19 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   splits = (K + k_per - 1) / k_per;
   const int items = tiles * splits;
   if constexpr (EPI != KR_GEMM_EPI_NONE) return KR_EINVAL;  // (not reached: a fused launch never splits)
-  hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE>), dim3(grid_for(items)), dim3(NTHREADS),
-                     lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
-                     (const bf16*)nullptr, 0, (bf16*)nullptr, 0);
+  bool launched = false;
+  if constexpr (EPI == KR_GEMM_EPI_NONE && B_T) {
+    if (with_runs) {   // (only A can be in runs here: an output in runs is never cut)
+      hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE, true>), dim3(grid_for(items)), dim3(NTHREADS),
+                         lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
+                         (const bf16*)nullptr, 0, (bf16*)nullptr, 0, fu.runs);
+      launched = true;
+    }
+  }
+  if (!launched)
+    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE>), dim3(grid_for(items)), dim3(NTHREADS),
+                       lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
+                       (const bf16*)nullptr, 0, (bf16*)nullptr, 0, fu.runs);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream,
@@ -939,6 +997,23 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
       N >= 1 << 26)
     return KR_EUNSUPPORTED;
   if (fu.max_cus < 0) return KR_EINVAL;
+  // row runs: 2, 4, 8 or 16 rows per run (a 16-row block of the epilogue and a 64-row K-step start
+  // at a run's first row), run starts a multiple of 8 elements apart, offsets within 32 bits
+  {
+    const RowRuns& rr = fu.runs;
+    const int shs[3] = {rr.a_sh, rr.c_sh, rr.x_sh}, outers[3] = {rr.a_outer, rr.c_outer, rr.x_outer};
+    const int64_t rows_of[3] = {layout == KR_GEMM_NT ? K : M, M, M};
+    for (int i = 0; i < 3; ++i) {
+      if (shs[i] == 0) continue;
+      if (shs[i] < 0 || shs[i] > 4 || outers[i] <= 0) return KR_EINVAL;
+      if (outers[i] % 8 || rows_of[i] % (1 << shs[i])) return KR_EUNSUPPORTED;
+      if ((rows_of[i] >> shs[i]) * (int64_t)outers[i] >= (int64_t)1 << 31) return KR_EUNSUPPORTED;
+    }
+    // the output's runs are honoured by the plain bf16 store only; the second operand of the SwiGLU
+    // backward (fc1's saved output) is read as a plain matrix
+    if (rr.c_sh && (accumulate || fu.epi == KR_GEMM_EPI_SWIGLU || fu.epi == KR_GEMM_EPI_SWIGLU_BWD)) return KR_EUNSUPPORTED;
+    if (rr.x_sh && fu.epi != KR_GEMM_EPI_ADD) return KR_EUNSUPPORTED;
+  }
   if (fu.epi != KR_GEMM_EPI_NONE) {
     if (accumulate) return KR_EINVAL;
     if (fu.epi == KR_GEMM_EPI_SWIGLU_BWD) {
@@ -970,7 +1045,7 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   // passing the smaller workspace kr_gemm_workspace_bytes_shared sizes); a fused epilogue works on
   // finished sums and is never cut
   int max_splits = 1;
-  if (ws != nullptr && fu.epi == KR_GEMM_EPI_NONE) {
+  if (ws != nullptr && fu.epi == KR_GEMM_EPI_NONE && fu.runs.c_sh == 0) {
     const size_t held = workspace_bytes / ((size_t)M * N * sizeof(float));
     max_splits = held > 16 ? 16 : (int)held;
     if (max_splits < 1) max_splits = 1;
@@ -1034,7 +1109,7 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
       // 256 x 256 are two rounds on 224 units; transposed, 512 tiles of 256 x 224 are two full
       // rounds of smaller tiles).  Only for a plain store: accumulation and split-K keep the
       // direct form.
-      if (!accumulate && ((int64_t)M * lda < ((int64_t)1 << 31)) && M <= (1 << 26)) {
+      if (!accumulate && fu.runs.a_sh == 0 && fu.runs.c_sh == 0 && ((int64_t)M * lda < ((int64_t)1 << 31)) && M <= (1 << 26)) {
         auto cost = [&](int rows, int cols, int w) {
           const int tiles = ((rows + BM - 1) / BM) * ((cols + 32 * w - 1) / (32 * w));
           return (long)((tiles + cus - 1) / cus) * (w + 1);
@@ -1083,6 +1158,38 @@ extern "C" int kr_gemm_bf16_fused(int layout, int M, int N, int K, const void* A
   fu.out2 = (bf16*)out2;
   fu.ld_out2 = ld_out2;
   fu.max_cus = max_cus;
+  return gemm_dispatch(layout, M, N, K, A, lda, B, ldb, C, ldc, accumulate, workspace, workspace_bytes,
+                       stream, fu);
+}
+
+// The same with row runs (see run_off): A, C and aux may each be a nanobatch of several sequences read or
+// written in place in a [s, b, h] tensor.  *_run_rows: rows per run (1 = a plain matrix), a power of two up
+// to 16; *_run_ld: distance between the starts of consecutive runs, in elements.
+extern "C" int kr_gemm_bf16_runs(int layout, int M, int N, int K, const void* A, int64_t lda,
+                                 int a_run_rows, int64_t a_run_ld, const void* B, int64_t ldb, void* C,
+                                 int64_t ldc, int c_run_rows, int64_t c_run_ld, int accumulate,
+                                 int epilogue, const void* aux, int64_t ld_aux, int aux_run_rows,
+                                 int64_t aux_run_ld, void* out2, int64_t ld_out2, int max_cus,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+  Fused fu;
+  fu.epi = epilogue & ~KR_GEMM_BESIDE_OTHER_STREAMS;
+  fu.shared = (epilogue & KR_GEMM_BESIDE_OTHER_STREAMS) != 0;
+  fu.aux = (const bf16*)aux;
+  fu.ld_aux = ld_aux;
+  fu.out2 = (bf16*)out2;
+  fu.ld_out2 = ld_out2;
+  fu.max_cus = max_cus;
+  const int run_rows[3] = {a_run_rows, c_run_rows, aux_run_rows};
+  const int64_t run_ld[3] = {a_run_ld, c_run_ld, aux_run_ld};
+  int sh[3];
+  for (int i = 0; i < 3; ++i) {
+    const int r = run_rows[i];
+    if (r < 1 || (r & (r - 1))) return KR_EINVAL;
+    if (r > 16) return KR_EUNSUPPORTED;
+    sh[i] = r == 1 ? 0 : (r == 2 ? 1 : (r == 4 ? 2 : (r == 8 ? 3 : 4)));
+    if (sh[i] && (run_ld[i] <= 0 || run_ld[i] >= (int64_t)1 << 31)) return KR_EINVAL;
+  }
+  fu.runs = {sh[0], sh[0] ? (int)a_run_ld : 0, sh[1], sh[1] ? (int)c_run_ld : 0, sh[2], sh[2] ? (int)aux_run_ld : 0};
   return gemm_dispatch(layout, M, N, K, A, lda, B, ldb, C, ldc, accumulate, workspace, workspace_bytes,
                        stream, fu);
 }

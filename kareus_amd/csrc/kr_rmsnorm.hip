@@ -17,12 +17,24 @@ constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * KR_WAVE;
 constexpr int kMaxBwdBlocks = 512;
 
+// Row runs: the rows of a tensor may come in runs of 2^sh consecutive rows (stride ld) whose starts are
+// `outer` elements apart — a nanobatch of 2^sh sequences cut out of a [s, b, h] tensor along b, used in
+// place.  A plain matrix has sh = 0 (outer unused).
+struct Runs {
+  int sh;
+  int64_t outer;
+};
+__device__ __forceinline__ int64_t row_at(int64_t row, int64_t ld, Runs r) {
+  return r.sh ? (row >> r.sh) * r.outer + (row & ((1 << r.sh) - 1)) * ld : row * ld;
+}
+
 template <int NCHUNK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __restrict__ x,
                                                                const bf16* __restrict__ gamma,
                                                                bf16* __restrict__ y,
                                                                float* __restrict__ rstd, int rows,
-                                                               int cols, int64_t x_ld, float eps) {
+                                                               int cols, int64_t x_ld, float eps,
+                                                               Runs x_runs) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nvec = cols / 8;
   const float inv_cols = 1.0f / (float)cols;
@@ -33,7 +45,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
     g[c] = v < nvec ? ldg8(gamma + v * 8) : zero8();
   }
   for (int row = blockIdx.x * kWaves + wave; row < rows; row += gridDim.x * kWaves) {
-    const bf16* xr = x + (int64_t)row * x_ld;
+    const bf16* xr = x + row_at(row, x_ld, x_runs);
     bf16x8 xv[NCHUNK];
     float ss = 0.f;
 #pragma unroll
@@ -80,7 +92,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bf16* __restrict__ dy, const bf16* __restrict__ x, const float* __restrict__ rstd,
     const bf16* __restrict__ gamma, const bf16* __restrict__ dres, bf16* __restrict__ dx,
     float* __restrict__ partial, int rows, int cols, int64_t dy_ld, int64_t x_ld, int64_t dres_ld,
-    int64_t dx_ld) {
+    int64_t dx_ld, Runs x_runs, Runs dres_runs, Runs dx_runs) {
   constexpr int kRowsPerBlock = kWaves / SPLIT;
   __shared__ float red[kWaves - 1][64 * 8];
   __shared__ float halves[2][kRowsPerBlock][2];  // [iteration parity][row of the block][half]
@@ -108,9 +120,9 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
     const bool active = SPLIT == 1 || row < rows;  // SPLIT == 1: the loop bound is the wave's own
     if (SPLIT == 1 && row >= rows) break;
     const int64_t r64 = active ? row : 0;
-    const bf16* xr = x + r64 * x_ld;
+    const bf16* xr = x + row_at(r64, x_ld, x_runs);
     const bf16* dr = dy + r64 * dy_ld;
-    const bf16* rr = ADD ? dres + r64 * dres_ld : nullptr;
+    const bf16* rr = ADD ? dres + row_at(r64, dres_ld, dres_runs) : nullptr;
     const float rs = active ? rstd[r64] : 0.f;
     bf16x8 xv[NCHUNK], dv[NCHUNK], rv[ADD && FULL ? NCHUNK : 1];
 #pragma unroll
@@ -141,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
       parity ^= 1;  // the next row uses the other buffer: one barrier per row is enough
     }
     dot *= inv_cols;
-    bf16* oxr = dx + r64 * dx_ld;
+    bf16* oxr = dx + row_at(r64, dx_ld, dx_runs);
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int v = v0 + c * 64;
@@ -257,8 +269,40 @@ inline int chunks_for(int cols) { return (cols / 8 + 63) / 64; }
     default: { constexpr int C_ = 16; CALL; } break; \
   }
 
+namespace {
+// rows per run (a power of two, 1 = plain) and distance between run starts -> Runs; false if invalid
+bool make_runs(int run_rows, int64_t run_ld, int rows, Runs* out, int* rc) {
+  *out = Runs{0, 0};
+  if (run_rows == 1) return true;
+  if (run_rows < 1 || (run_rows & (run_rows - 1)) || run_ld <= 0) { *rc = KR_EINVAL; return false; }
+  if (run_rows > 1024 || run_ld % 8 || rows % run_rows) { *rc = KR_EUNSUPPORTED; return false; }
+  int sh = 0;
+  while ((1 << sh) < run_rows) ++sh;
+  *out = Runs{sh, run_ld};
+  return true;
+}
+int rmsnorm_fwd_impl(const void* x, const void* gamma, void* y, float* rstd, int rows, int cols,
+                     int64_t x_ld, Runs x_runs, float eps, void* stream);
+}  // namespace
+
 extern "C" int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* rstd, int rows,
                               int cols, int64_t x_ld, float eps, void* stream) {
+  return rmsnorm_fwd_impl(x, gamma, y, rstd, rows, cols, x_ld, Runs{0, 0}, eps, stream);
+}
+
+// kr_rmsnorm_fwd on an input whose rows come in runs (a nanobatch of several sequences read in place)
+extern "C" int kr_rmsnorm_fwd_runs(const void* x, const void* gamma, void* y, float* rstd, int rows,
+                                   int cols, int64_t x_ld, int x_run_rows, int64_t x_run_ld, float eps,
+                                   void* stream) {
+  Runs xr;
+  int rc = KR_OK;
+  if (rows <= 0 || !make_runs(x_run_rows, x_run_ld, rows, &xr, &rc)) return rc == KR_OK ? KR_EINVAL : rc;
+  return rmsnorm_fwd_impl(x, gamma, y, rstd, rows, cols, x_ld, xr, eps, stream);
+}
+
+namespace {
+int rmsnorm_fwd_impl(const void* x, const void* gamma, void* y, float* rstd, int rows, int cols,
+                     int64_t x_ld, Runs x_runs, float eps, void* stream) {
   if (!x || !gamma || !y || !rstd || rows <= 0 || cols <= 0 || x_ld < cols) return KR_EINVAL;
   if (cols % 8 || x_ld % 8 || cols > 8192) return KR_EUNSUPPORTED;
   if (!kr_aligned16(x) || !kr_aligned16(y) || !kr_aligned16(gamma)) return KR_EINVAL;
@@ -267,9 +311,10 @@ extern "C" int kr_rmsnorm_fwd(const void* x, const void* gamma, void* y, float* 
   const int nc = chunks_for(cols);
   KR_DISPATCH_CHUNKS(nc, hipLaunchKernelGGL(rmsnorm_fwd_kernel<C_>, dim3(blocks), dim3(kThreads), 0,
                                            (hipStream_t)stream, (const bf16*)x, (const bf16*)gamma,
-                                           (bf16*)y, rstd, rows, cols, x_ld, eps));
+                                           (bf16*)y, rstd, rows, cols, x_ld, eps, x_runs));
   return kr_launch_status();
 }
+}  // namespace
 
 extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
   if (rows <= 0 || cols <= 0) return 0;
@@ -277,9 +322,13 @@ extern "C" size_t kr_rmsnorm_bwd_workspace_bytes(int rows, int cols) {
 }
 
 namespace {
+struct BwdRuns {
+  Runs x{0, 0}, dres{0, 0}, dx{0, 0};
+};
 int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const void* gamma,
                      const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
-                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream);
+                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream,
+                     const BwdRuns& runs = BwdRuns());
 }
 
 extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rstd,
@@ -288,6 +337,25 @@ extern "C" int kr_rmsnorm_bwd_add(const void* dy, const void* x, const float* rs
                                   int64_t dres_ld, int64_t dx_ld, void* stream) {
   return rmsnorm_bwd_impl(dy, x, rstd, gamma, dres, dx, dgamma, workspace, rows, cols, dy_ld, x_ld,
                           dres_ld, dx_ld, stream);
+}
+
+// kr_rmsnorm_bwd_add where the saved input, the residual gradient and / or the result are nanobatches
+// of several sequences used in place: rows in runs of *_run_rows (1 = plain), run starts *_run_ld apart
+extern "C" int kr_rmsnorm_bwd_add_runs(const void* dy, const void* x, const float* rstd,
+                                       const void* gamma, const void* dres, void* dx, void* dgamma,
+                                       void* workspace, int rows, int cols, int64_t dy_ld,
+                                       int64_t x_ld, int x_run_rows, int64_t x_run_ld,
+                                       int64_t dres_ld, int dres_run_rows, int64_t dres_run_ld,
+                                       int64_t dx_ld, int dx_run_rows, int64_t dx_run_ld,
+                                       void* stream) {
+  BwdRuns runs;
+  int rc = KR_OK;
+  if (rows <= 0) return KR_EINVAL;
+  if (!make_runs(x_run_rows, x_run_ld, rows, &runs.x, &rc)) return rc;
+  if (dres && !make_runs(dres_run_rows, dres_run_ld, rows, &runs.dres, &rc)) return rc;
+  if (!make_runs(dx_run_rows, dx_run_ld, rows, &runs.dx, &rc)) return rc;
+  return rmsnorm_bwd_impl(dy, x, rstd, gamma, dres, dx, dgamma, workspace, rows, cols, dy_ld, x_ld,
+                          dres_ld, dx_ld, stream, runs);
 }
 
 // ---- the variant that allocates nothing --------------------------------------------------------
@@ -338,7 +406,8 @@ extern "C" int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const f
 namespace {
 int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const void* gamma,
                      const void* dres, void* dx, void* dgamma, void* workspace, int rows, int cols,
-                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream) {
+                     int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld, void* stream,
+                     const BwdRuns& runs) {
   if (!dy || !x || !rstd || !gamma || !dx || !workspace || rows <= 0 || cols <= 0 ||
       dy_ld < cols || x_ld < cols || dx_ld < cols || (dres && dres_ld < cols))
     return KR_EINVAL;
@@ -356,7 +425,8 @@ int rmsnorm_bwd_impl(const void* dy, const void* x, const float* rstd, const voi
                                            (const bf16*)dy, (const bf16*)x, rstd,                   \
                                            (const bf16*)gamma, (const bf16*)dres, (bf16*)dx,        \
                                            (float*)workspace, rows, cols, dy_ld, x_ld,              \
-                                           dres ? dres_ld : (int64_t)0, dx_ld))
+                                           dres ? dres_ld : (int64_t)0, dx_ld, runs.x, runs.dres,  \
+                                           runs.dx))
   // rows of exactly 1, 2, 3, 4, 6 or 8 times 512 elements per wave take the straight-line kernel
   const bool full = cols % (512 * split) == 0 && cols / (512 * split) == nc && nc <= 8 && nc != 5 && nc != 7;
   if (split == 2) {

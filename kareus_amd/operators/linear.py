@@ -92,17 +92,6 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
 
     fuse_activation = True
 
-    @staticmethod
-    def _as_matrix(t, cols):
-        """``t`` as a [rows, cols] matrix with one row stride and no copy, or None."""
-        if t is None or t.shape[-1] != cols:
-            return None
-        try:
-            m = t.view(-1, cols)
-        except RuntimeError:
-            return None
-        return m if m.stride(1) == 1 and m.stride(0) % 8 == 0 and m.stride(0) >= cols else None
-
     def fuser_forward(self, basic_op_ctxs, input_, *, basic_op_extra_inputs, basic_op_prev_ops,
                       basic_op_next_ops, basic_op_kwargs):
         ctx = basic_op_ctxs[0]
@@ -110,7 +99,7 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         if input_.shape[-1] != k:
             raise ValueError(f"linear with in_features={k} got input of shape {tuple(input_.shape)}")
         be = get_backend(self._backend_name)
-        x2d = self._rows(input_.reshape(-1, k))
+        x2d = be.rows_in_place(input_)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d)
             ctx.input_requires_grad = True
@@ -119,7 +108,7 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
             # [fc1, SwiGLU]: x = input . W^T and y = silu(x[:, :F]) * x[:, F:] from one launch
             # (kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20 behind basic_linear.py:571-582)
             act_ctx = basic_op_ctxs[1]
-            y = x2d.new_empty((x2d.shape[0], n // 2))
+            y = x2d.new_empty((x2d.numel() // k, n // 2))
             x = be.linear_fwd(x2d, w, split_k=self.split_k, swiglu_out=y)
             if act_ctx.requires_grad:
                 act_ctx.save_for_backward(x)
@@ -129,9 +118,11 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         sink = ctx.__dict__.pop("out_sink", None)
         out_shape = (*input_.shape[:-1], n)
         if residual is not None:
-            res2d = self._as_matrix(residual, n)
-            out2d = self._as_matrix(sink, n) if sink is not None else None
-            if res2d is not None and res2d.shape[0] == x2d.shape[0] and (sink is None or out2d is not None):
+            # in place where the kernels can address them: row-strided one-sequence slices, row runs of wider ones
+            res2d = be.rows_view(residual) if residual.shape[-1] == n else None
+            out2d = be.rows_view(sink) if (sink is not None and sink.shape[-1] == n) else None
+            if (res2d is not None and res2d.numel() // n == x2d.numel() // k
+                    and (sink is None or (out2d is not None and out2d.numel() == res2d.numel()))):
                 y = be.linear_fwd(x2d, w, split_k=self.split_k, residual=res2d, out=out2d)
                 y = sink if sink is not None else y.view(out_shape)
                 y._kr_residual_added = True
@@ -163,8 +154,8 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         (x2d,) = ctx.saved_tensors
         (act_in,) = act_ctx.saved_tensors
         n, _k = self.weight.shape
-        dy = self._rows(grad_output.reshape(-1, n))
         be = get_backend(self._backend_name)
+        dy = be.rows_in_place(grad_output)
         dx = be.linear_dgrad(dy, self.weight.detach(), split_k=self.split_k, swiglu_bwd_x=act_in)
         dw = self._weight_grad(be, ctx, dy, x2d, self.split_k) if self.weight.requires_grad else None
         return dx.view(act_ctx.ori_shape), [(dw,), ()], [extra, ()]
@@ -172,20 +163,11 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
     def op_backward(self, ctx, grad_output):
         (x2d,) = ctx.saved_tensors
         n, k = self.weight.shape
-        dy = self._rows(grad_output.reshape(-1, n))
         be = get_backend(self._backend_name)
+        dy = be.rows_in_place(grad_output)
         dx = be.linear_dgrad(dy, self.weight.detach(), split_k=self.split_k)
         dw = self._weight_grad(be, ctx, dy, x2d, self.split_k) if self.weight.requires_grad else None
         return dx.view(*grad_output.shape[:-1], k), (dw,)
-
-    @staticmethod
-    def _rows(t2d):
-        """GEMM operands may be row-strided (a one-sequence nanobatch slice of a
-        [seq, batch, hidden] tensor is); the reference copies such slices
-        (basic_linear.py:565-569), here only layouts a leading dimension cannot express are."""
-        if t2d.stride(1) == 1 and t2d.stride(0) % 8 == 0 and t2d.stride(0) >= t2d.shape[1]:
-            return t2d
-        return t2d.contiguous()
 
     @staticmethod
     def _weight_grad(be, ctx, dy, x2d, split_k=True):

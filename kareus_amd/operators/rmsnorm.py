@@ -26,15 +26,18 @@ class RMSNorm(BasicOperation):
         h = self.weight.shape[0]
         if input_.shape[-1] != h:
             raise ValueError(f"RMSNorm over {h} features got input of shape {tuple(input_.shape)}")
-        x2d = input_.reshape(-1, h)   # a view when the rows have one stride, else a dense copy
-        y, rstd = get_backend(self._backend_name).rmsnorm_fwd(x2d, self.weight.detach(), self.eps)
+        # a view when the rows have one stride; a nanobatch of several sequences cut out of a [s, b, h]
+        # tensor stays as it is where the kernels read row runs in place; else a dense copy
+        be = get_backend(self._backend_name)
+        x2d = be.rows_in_place(input_)
+        y, rstd = be.rmsnorm_fwd(x2d, self.weight.detach(), self.eps)
         if ctx.requires_grad:
             ctx.save_for_backward(x2d, rstd)
         return y.view(input_.shape)
 
     def op_backward(self, ctx, grad_output):
         x2d, rstd = ctx.saved_tensors
-        dy = grad_output.reshape(x2d.shape)
+        dy = grad_output.reshape(-1, x2d.shape[-1])
         dx, dgamma = self._backward(ctx, dy, x2d, rstd, None, None)
         return dx.view(grad_output.shape), (dgamma,)
 
@@ -50,7 +53,8 @@ class RMSNorm(BasicOperation):
         n = sink.get("n", 0) if sink is not None else 0
         if n < 2 or not self.weight.requires_grad:
             return be.rmsnorm_bwd(dy, x2d, rstd, self.weight.detach(), residual_grad=residual_grad, out=out2d)
-        rows, cols = x2d.shape
+        cols = x2d.shape[-1]
+        rows = x2d.numel() // cols
         per = be.rmsnorm_partial_rows(rows, cols)
         api = stream_api()
         here = api.current_stream()
@@ -98,14 +102,12 @@ class RMSNorm(BasicOperation):
         (grad_residual,) = basic_op_grad_extra_outputs[1]
         sink = fork_ctx.__dict__.pop("out_sink", None)
         x2d, rstd = norm_ctx.saved_tensors
-        dy = grad_output.reshape(x2d.shape)
-        out2d = None
-        if sink is not None:
-            try:
-                out2d = sink.view(x2d.shape)   # a one-sequence slice is a row-strided matrix
-            except RuntimeError:
-                out2d = None
-        dx, dgamma = self._backward(norm_ctx, dy, x2d, rstd, grad_residual.reshape(x2d.shape), out2d)
+        be = get_backend(self._backend_name)
+        dy = grad_output.reshape(-1, x2d.shape[-1])
+        # a one-sequence slice is a row-strided matrix, a wider one has its rows in runs: written in place
+        # where the kernels can, else through a dense result and one copy
+        out2d = be.rows_view(sink) if sink is not None else None
+        dx, dgamma = self._backward(norm_ctx, dy, x2d, rstd, be.rows_in_place(grad_residual), out2d)
         if sink is not None:
             if out2d is None:
                 sink.copy_(dx.view(sink.shape))
