@@ -63,13 +63,18 @@ def total_flops(w) -> float:
     return w["layers"] * (3 * gemm_fwd + 3.5 * attn_fwd)
 
 
-def make_model(w, nnb, device, use_streams=True, schedule=None):
+def make_model(w, nnb, device, use_streams=True, schedule=None, all_on_one_stream=False):
+    """``all_on_one_stream``: the engine is set up as for concurrent nanobatch streams (same launch plans,
+    same event edges) but every nanobatch is given the caller's stream, so the very same launches run one
+    after the other."""
     from kareus_amd import LayerConfig, LayerStack
 
     cfg = LayerConfig(hidden_size=w["h"], num_attention_heads=w["nq"], num_query_groups=w["nkv"],
                       kv_channels=w["hd"], ffn_hidden_size=w["ffn"], num_layers=w["layers"],
                       num_nanobatches=nnb, backend="hip", use_streams=use_streams)
     cfg.kareus_scheduler = schedule
+    if all_on_one_stream and nnb > 1:
+        cfg.nanobatch_streams = [torch.cuda.current_stream()] * nnb
     return LayerStack(cfg, device=device, seed=1234)
 
 
@@ -172,11 +177,17 @@ def partition_times(stepper, iters=3):
 # reports null.  A constant read off a profile, not something measured in this run: the entry
 # names the profile it came from, and it is only reported while the GEMM source is the one the
 # counters were read with (first 16 hex digits of its SHA-256).
-TRAFFIC_GEMM_SOURCE = "7cee73aae2f62812"
+TRAFFIC_GEMM_SOURCE = "2ceda96f9e9624f7"
 MEASURED_TRAFFIC = {
-    ("NT", 7168, 4096, 16384): {"bytes": (761642.4 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("TN", 16384, 7168, 4096): {"bytes": (736977.8 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 16384, 4096, 7168): {"bytes": (688400.5 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    # (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000) x 1024, means over the launches of `bench.py --roofline-only`
+    # one nanobatch of four (4096 tokens), what the default run launches; NT in its accumulating form
+    ("NT", 7168, 4096, 4096): {"bytes": (234044.6 * 2.000 + 57792.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 4096, 7168, 4096): {"bytes": (180569.3 * 2.000 + 86016.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 4096, 4096, 7168): {"bytes": (172296.5 * 2.000 + 32768.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    # the whole microbatch as one nanobatch (16384 tokens, --nanobatches 1)
+    ("NT", 7168, 4096, 16384): {"bytes": (912593.3 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 16384, 7168, 4096): {"bytes": (721904.1 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 16384, 4096, 7168): {"bytes": (688405.2 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
 }
 
 
@@ -203,8 +214,10 @@ def _gemm_operands(layout, m, n, k, device):
 
 
 def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False,
-              fused_swiglu_backward=False, alone=False):
-    """Average duration of one launch, HIP events on the stream the kernel is launched on."""
+              fused_swiglu_backward=False, alone=False, preheat_s=0.0):
+    """Average duration of one launch, HIP events on the stream the kernel is launched on.  ``preheat_s``:
+    launch the same GEMM back to back for that long first, so that the timed launches see the clocks a
+    sustained run settles at instead of a rested chip's."""
     a, b = _gemm_operands(layout, m, n, k, device)
     out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
     y = torch.empty(m, n // 2, device=device, dtype=torch.bfloat16) if fused_swiglu else None
@@ -222,6 +235,11 @@ def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, resi
     for _ in range(5):
         fn()
     torch.cuda.synchronize()
+    t_end = time.perf_counter() + preheat_s
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(launches):
@@ -252,7 +270,7 @@ class GemmEventTimer:
 
     def __init__(self, be, shapes):
         self.be, self.shapes = be, set(shapes)
-        self.pairs = {s: [] for s in self.shapes}
+        self.pairs = {}     # (shape, accumulating) -> [(start event, end event)]
 
     def __enter__(self):
         inner = self.be.gemm
@@ -265,7 +283,7 @@ class GemmEventTimer:
             e0.record()
             r = inner(layout, a, b, m, n, k, *args, **kw)
             e1.record()
-            self.pairs[key].append((e0, e1))
+            self.pairs.setdefault((key, bool(kw.get("accumulate"))), []).append((e0, e1))
             return r
 
         self.be.gemm = gemm
@@ -275,9 +293,10 @@ class GemmEventTimer:
         del self.be.gemm    # back to the class's method
         return False
 
-    def seconds(self, key):
-        """(average duration of a launch, launches); call after the device has been synchronised."""
-        pairs = self.pairs.get(key) or []
+    def seconds(self, key, accumulating=None):
+        """(average duration of a launch, launches) of the launches of a shape — all of them, or only those
+        that do / do not accumulate into their output; call after the device has been synchronised."""
+        pairs = [p for (k, acc), v in self.pairs.items() if k == key and accumulating in (None, acc) for p in v]
         if not pairs:
             return None, 0
         return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / len(pairs), len(pairs)
@@ -290,7 +309,7 @@ def dominant_gemm_shapes(w, nnb):
     return {"NT": (2, two_f, h, t), "TN": (0, t, two_f, h), "NN": (1, t, h, two_f)}
 
 
-def dominant_kernel_roofline(w, nnb, device, launches=30):
+def dominant_kernel_roofline(w, nnb, device, launches=30, preheat_s=0.0):
     """The GEMM instance with the largest share of the step's kernel time: the weight gradient of
     fc1, dW[2F, h] = dy[T_nb, 2F]^T . x[T_nb, h] (layout NT), plus the forward (TN, with the SwiGLU
     epilogue the engine runs it with) and the input gradient (NN) of the same layer."""
@@ -299,13 +318,16 @@ def dominant_kernel_roofline(w, nnb, device, launches=30):
     be = get_backend("hip")
     t, two_f, h = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
     fuse = be.can_fuse_swiglu(two_f)
-    main = _roofline_entry("gemm_kernel<NT> (fc1 weight gradient)", "NT", two_f, h, t,
-                           time_gemm(be, "NT", two_f, h, t, device, launches))
+    # with several nanobatches three of four (N - 1 of N) weight-gradient launches add into the first one's
+    # result: that is the form measured
+    acc = nnb > 1
+    main = _roofline_entry("gemm_kernel<NT> (fc1 weight gradient%s)" % (", accumulating" if acc else ""), "NT", two_f, h, t,
+                           time_gemm(be, "NT", two_f, h, t, device, launches, accumulate=acc, preheat_s=preheat_s))
     others = [
         _roofline_entry("gemm_kernel<TN%s> (fc1 forward)" % (", SwiGLU epilogue" if fuse else ""), "TN", t, two_f, h,
-                        time_gemm(be, "TN", t, two_f, h, device, launches, fused_swiglu=fuse)),
+                        time_gemm(be, "TN", t, two_f, h, device, launches, fused_swiglu=fuse, preheat_s=preheat_s / 2)),
         _roofline_entry("gemm_kernel<NN> (fc1 input gradient)", "NN", t, h, two_f,
-                        time_gemm(be, "NN", t, h, two_f, device, launches)),
+                        time_gemm(be, "NN", t, h, two_f, device, launches, preheat_s=preheat_s / 2)),
     ]
     return main, others
 
@@ -766,6 +788,9 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the partition, energy and host-enqueue legs")
     ap.add_argument("--one-stream", action="store_true",
                     help="run every nanobatch on the caller's stream (no overlap; for profiling)")
+    ap.add_argument("--same-launches-one-stream", action="store_true",
+                    help="run only: K steps of the nanobatched step's own launches, all on the caller's stream "
+                         "(the region the roofline kernel is timed in; for the kernel trace of it)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant-kernel leg (the command profiled under profiles/)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -800,7 +825,8 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.roofline_only:
-        main_kernel, others = dominant_kernel_roofline(w, w["nnb"], device)
+        # stand-alone leg: a 2 s pre-heat in front, so that its launches run at the clocks they run at inside a step
+        main_kernel, others = dominant_kernel_roofline(w, w["nnb"], device, preheat_s=2.0)
         print(json.dumps({"roofline": main_kernel, "roofline_others": others}))
         return
     if args.copy_calibration:
@@ -820,6 +846,16 @@ def main():
         return
     if args.power_trace:
         print(json.dumps({"power_trace": power_trace(w, device)}))
+        return
+    if args.same_launches_one_stream:
+        gen = torch.Generator().manual_seed(42)
+        x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
+        go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
+        st = Stepper(make_model(w, w["nnb"], device, all_on_one_stream=True), x, go)
+        st.run(2)
+        preheat(st, 2.0)
+        st.run(args.warmup)
+        print(json.dumps({"same_launches_one_stream_ms_per_step": st.timed(args.steps) * 1e3, "steps": args.steps}))
         return
     if args.overlap_bound:
         print(json.dumps({"overlap_bound": overlap_bound(w, device)}))
@@ -843,6 +879,12 @@ def main():
         if not args.no_extras:
             ways["same_nb_one_stream"] = Stepper(make_model(w, w["nnb"], device, use_streams=False,
                                                             schedule=make_scheduler(schedule_path, w["nnb"])), x, go)
+    # for the roofline kernel only: the launches of the nanobatched step, one after the other
+    same_launches = None
+    if w["nnb"] > 1 and not args.one_stream:
+        same_launches = Stepper(make_model(w, w["nnb"], device, all_on_one_stream=True,
+                                           schedule=make_scheduler(schedule_path, w["nnb"])), x, go)
+        same_launches.run(2)
     for st in ways.values():
         st.run(2)
     preheat(nano, 2.0)
@@ -860,6 +902,15 @@ def main():
     watched = dominant_gemm_shapes(w, run_nnb)
     with GemmEventTimer(get_backend("hip"), watched.values()) as in_step:
         sec = runner.timed(args.steps)
+    # A kernel's interval on its own stream is its duration only while nothing else runs beside it.  With the
+    # nanobatches on concurrent streams it also holds the time its workgroups wait for compute units that the
+    # other streams' kernels occupy, so the roofline kernel is timed in a second region of K steps of the SAME
+    # nanobatches — the same launches, shapes and epilogues — on one stream.
+    alone_in_step = None
+    if run_nnb > 1 and same_launches is not None:
+        same_launches.run(args.warmup)
+        with GemmEventTimer(get_backend("hip"), watched.values()) as alone_in_step:
+            one_stream_sec = same_launches.timed(args.steps)
     # beside it, timed the same way: the one-nanobatch (serial) step of the same layer and data
     serial_sec = None
     if "serial_1nb" in ways and picked != "serial_1nb":
@@ -912,19 +963,31 @@ def main():
             out["overlap"]["overlap_efficiency"] = sum(parts.values()) * 1e-3 / med["nanobatched"]
 
     ways.clear()
-    del nano, runner
+    del nano, runner, same_launches
     # roofline of the dominant kernel: its launches inside the K timed steps; the same kernel
     # launched back to back on its own (a hotter chip: nothing but the heaviest GEMM) beside it
     alone_main, alone_others = dominant_kernel_roofline(w, run_nnb, device)
     entries = []
     for alone in [alone_main] + alone_others:
         layout = alone["kernel"].split("<")[1][:2]
-        s, n_launches = in_step.seconds(watched[layout])
+        acc = (run_nnb > 1) if layout == "NT" else None     # the accumulating launches of the weight gradient
+        s, n_launches = in_step.seconds(watched[layout], acc)
         if s is None:
             entries.append(dict(alone, measured="back to back on its own"))
             continue
-        e = _roofline_entry(alone["kernel"], layout, *watched[layout][1:], s)
-        e["measured"] = f"HIP events around its {n_launches} launches inside the {args.steps} timed steps"
+        if alone_in_step is not None:
+            s1, n1 = alone_in_step.seconds(watched[layout], acc)
+            e = _roofline_entry(alone["kernel"], layout, *watched[layout][1:], s1)
+            e["measured"] = (f"HIP events around its {n1} launches inside {args.steps} timed steps of the same "
+                             f"{run_nnb} nanobatches on one stream ({one_stream_sec * 1e3:.3f} ms per step): there the "
+                             "interval is the kernel's own duration")
+            e["interval_on_concurrent_streams_us"] = s * 1e6
+            e["interval_on_concurrent_streams_is"] = (
+                f"the same {n_launches} launches inside the {args.steps} headline steps: the interval on the launch "
+                "stream, which includes waiting for compute units held by the other nanobatch streams' kernels")
+        else:
+            e = _roofline_entry(alone["kernel"], layout, *watched[layout][1:], s)
+            e["measured"] = f"HIP events around its {n_launches} launches inside the {args.steps} timed steps"
         e["back_to_back_alone_us"] = alone["avg_launch_us"]
         entries.append(e)
     out["roofline"], out["roofline_others"] = entries[0], entries[1:]
