@@ -6,21 +6,29 @@
 A step = one forward+backward of the decoder-layer stack over one synthetic batch, inputs
 resident in HBM.  Prints ONE JSON line (metric: layer fwd+bwd tokens/s) that also carries
   roofline      the kernel with the largest share of the step's kernel time (the weight-gradient
-                GEMM of fc1 at nanobatch shape), timed live with HIP events on its stream, against
-                the 2.5 PFLOP/s dense bf16 MFMA peak; `roofline_others` has the other two layouts
+                GEMM of fc1 at nanobatch shape, in the accumulating form most of its launches take),
+                timed live with HIP events around its launches inside K steps of the nanobatched
+                step's own launches issued on one stream (on concurrent streams an event interval
+                also holds the wait for compute units; that interval is reported beside it),
+                against the 2.5 PFLOP/s dense bf16 MFMA peak; `roofline_others` has the other two
+                layouts of fc1
   cpu_baseline  the CPU oracle (plain PyTorch fp32 layer) timed on the host cores on a bounded
                 sample of the same layer shape
-plus end-to-end MFMA utilisation, the nanobatched run beside the serial (1 nanobatch) run with
-the speed-up between them, overlap efficiency (sum of serially timed partition times / overlapped
-wall time), joules/token and the host's enqueue time per step.
+  serial_1nb    the same layer and data run as one nanobatch on one stream, timed right after the
+                headline steps with the same warm-up and step count
+plus end-to-end MFMA utilisation, overlap efficiency (sum of serially timed partition times /
+overlapped wall time), joules/token and the host's enqueue time per step.
 
-The chip is pre-heated for two seconds before anything is timed, and the three ways of running the
-layer that are compared (nanobatches on their own streams, one nanobatch, the same nanobatches on
-one stream) are timed in interleaved rounds, so that all of them see the same power and thermal
-state.  `value` is the run the engine is configured for; with `--nanobatches auto` that is the
-faster of the workload's nanobatch count and a single nanobatch, picked from those rounds (the
-reference, too, falls back to sequential execution where nanobatching costs more than it gives:
+`value` is the workload as configured: its own nanobatch count (four for c4) on concurrent
+streams.  `--nanobatches N` runs another count; `--nanobatches auto` reports the faster of the
+workload's count and a single nanobatch, picked from interleaved rounds (the reference, too,
+falls back to sequential execution where nanobatching costs more than it gives:
 tests/artifact/README.md:190-196), and `config.nanobatches` names the count that was run.
+
+The chip is pre-heated for two seconds before anything is timed, and the ways of running the
+layer that are compared (nanobatches on their own streams, one nanobatch, the same nanobatches on
+one stream) are also timed in interleaved rounds (`overlap`), so that all of them see the same
+power and thermal state.
 """
 
 from __future__ import annotations
@@ -214,11 +222,16 @@ def _gemm_operands(layout, m, n, k, device):
 
 
 def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, residual=False, accumulate=False,
-              fused_swiglu_backward=False, alone=False, preheat_s=0.0):
+              fused_swiglu_backward=False, alone=False, preheat_s=0.0, pieces=1):
     """Average duration of one launch, HIP events on the stream the kernel is launched on.  ``preheat_s``:
     launch the same GEMM back to back for that long first, so that the timed launches see the clocks a
-    sustained run settles at instead of a rested chip's."""
+    sustained run settles at instead of a rested chip's.  ``pieces`` > 1 (layout NT): the operands are that
+    many separate allocations of k / pieces rows each, contracted in one launch (the weight gradient over
+    all nanobatches of a microbatch)."""
     a, b = _gemm_operands(layout, m, n, k, device)
+    if pieces > 1:
+        a_pieces = [t.clone() for t in a.chunk(pieces)]
+        b_pieces = [t.clone() for t in b.chunk(pieces)]
     out = torch.empty(m, n, device=device, dtype=torch.bfloat16)
     y = torch.empty(m, n // 2, device=device, dtype=torch.bfloat16) if fused_swiglu else None
     r = torch.randn(m, n, device=device).bfloat16() if residual else None
@@ -227,7 +240,9 @@ def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, resi
     code = {"TN": 0, "NN": 1, "NT": 2}[layout]
 
     def fn():
-        if hx is not None:
+        if pieces > 1:
+            be.linear_wgrad_segments(a_pieces, b_pieces, out=out, accumulate=accumulate, split_k=True)
+        elif hx is not None:
             be.gemm(code, a, b, m, n, k, split_k=None, swiglu_bwd_x=hx)
         else:
             be.gemm(code, a, b, m, n, k, out=out, accumulate=accumulate, split_k=alone, swiglu_out=y, residual=r)
@@ -286,11 +301,26 @@ class GemmEventTimer:
             self.pairs.setdefault((key, bool(kw.get("accumulate"))), []).append((e0, e1))
             return r
 
+        inner_segments = self.be.linear_wgrad_segments
+
+        def segments(dys, xs, *args, **kw):
+            key = (2, dys[0].shape[-1], xs[0].shape[-1], sum(d.shape[0] for d in dys))
+            if key not in self.shapes:
+                return inner_segments(dys, xs, *args, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = inner_segments(dys, xs, *args, **kw)
+            e1.record()
+            self.pairs.setdefault((key, bool(kw.get("accumulate"))), []).append((e0, e1))
+            return r
+
         self.be.gemm = gemm
+        self.be.linear_wgrad_segments = segments
         return self
 
     def __exit__(self, *exc):
-        del self.be.gemm    # back to the class's method
+        del self.be.gemm    # back to the class's methods
+        del self.be.linear_wgrad_segments
         return False
 
     def seconds(self, key, accumulating=None):
@@ -303,33 +333,34 @@ class GemmEventTimer:
 
 
 def dominant_gemm_shapes(w, nnb):
-    """(layout code, M, N, K) of fc1's weight gradient (NT), forward (TN) and input gradient (NN)
-    at the token count of one launch."""
+    """(layout code, M, N, K) of fc1's forward (TN) and input gradient (NN) at the token count of one
+    nanobatch and of its weight gradient (NT), which the engine computes once per step over the tokens of
+    all nanobatches."""
     t, two_f, h = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
-    return {"NT": (2, two_f, h, t), "TN": (0, t, two_f, h), "NN": (1, t, h, two_f)}
+    return {"NT": (2, two_f, h, t * nnb), "TN": (0, t, two_f, h), "NN": (1, t, h, two_f)}
 
 
 def dominant_kernel_roofline(w, nnb, device, launches=30, preheat_s=0.0):
-    """The GEMM instance with the largest share of the step's kernel time: the weight gradient of
-    fc1, dW[2F, h] = dy[T_nb, 2F]^T . x[T_nb, h] (layout NT), plus the forward (TN, with the SwiGLU
-    epilogue the engine runs it with) and the input gradient (NN) of the same layer."""
+    """The three GEMMs of fc1, which hold the largest share of the step's kernel time, each launched back
+    to back on its own: the forward (TN, with the SwiGLU epilogue the engine runs it with), the input
+    gradient (NN) and the weight gradient dW[2F, h] = dy[T, 2F]^T . x[T, h] (NT; with several nanobatches one
+    launch over the operand pieces of all of them).  Returned with the one that takes the most time per step
+    first: with several nanobatches the forward (one launch per nanobatch; the weight gradient is a single
+    launch), with one nanobatch the weight gradient."""
     from kareus_amd.backend import get_backend
 
     be = get_backend("hip")
     t, two_f, h = (w["b"] // nnb) * w["s"], 2 * w["ffn"], w["h"]
     fuse = be.can_fuse_swiglu(two_f)
-    # with several nanobatches three of four (N - 1 of N) weight-gradient launches add into the first one's
-    # result: that is the form measured
-    acc = nnb > 1
-    main = _roofline_entry("gemm_kernel<NT> (fc1 weight gradient%s)" % (", accumulating" if acc else ""), "NT", two_f, h, t,
-                           time_gemm(be, "NT", two_f, h, t, device, launches, accumulate=acc, preheat_s=preheat_s))
-    others = [
-        _roofline_entry("gemm_kernel<TN%s> (fc1 forward)" % (", SwiGLU epilogue" if fuse else ""), "TN", t, two_f, h,
-                        time_gemm(be, "TN", t, two_f, h, device, launches, fused_swiglu=fuse, preheat_s=preheat_s / 2)),
-        _roofline_entry("gemm_kernel<NN> (fc1 input gradient)", "NN", t, h, two_f,
-                        time_gemm(be, "NN", t, h, two_f, device, launches, preheat_s=preheat_s / 2)),
-    ]
-    return main, others
+    first = {"TN": preheat_s, "NT": preheat_s / 2} if nnb > 1 else {"NT": preheat_s, "TN": preheat_s / 2}
+    nt = _roofline_entry("gemm_kernel<NT> (fc1 weight gradient%s)" % (f", one launch over {nnb} nanobatches" if nnb > 1 else ""),
+                         "NT", two_f, h, t * nnb,
+                         time_gemm(be, "NT", two_f, h, t * nnb, device, launches, alone=True, preheat_s=first["NT"], pieces=nnb))
+    tn = _roofline_entry("gemm_kernel<TN%s> (fc1 forward)" % (", SwiGLU epilogue" if fuse else ""), "TN", t, two_f, h,
+                         time_gemm(be, "TN", t, two_f, h, device, launches, fused_swiglu=fuse, preheat_s=first["TN"]))
+    nn = _roofline_entry("gemm_kernel<NN> (fc1 input gradient)", "NN", t, h, two_f,
+                         time_gemm(be, "NN", t, h, two_f, device, launches, preheat_s=preheat_s / 2))
+    return (tn, [nn, nt]) if nnb > 1 else (nt, [tn, nn])
 
 
 def time_library_matmul(layout, m, n, k, device, launches=30):
@@ -376,6 +407,9 @@ def gemm_kernels(w, nnb, device, launches=30, with_library=False):
             ("weight gradient", "NT", n_out, k_in, t, {}),
             ("weight gradient, accumulating", "NT", n_out, k_in, t, dict(accumulate=True)),
         ]
+        if nnb > 1:
+            variants.append((f"weight gradient, one launch over {nnb} nanobatches", "NT", n_out, k_in, t * nnb,
+                             dict(pieces=nnb)))
         for what, layout, m, n, k, kw in variants:
             sec = time_gemm(be, layout, m, n, k, device, launches, alone=nnb == 1, **kw)
             flops = 2.0 * m * n * k
@@ -655,6 +689,8 @@ def overlap_bound(w, device, rounds=4, steps=8):
         completely behind the other nanobatches' MFMA-bound kernels.  Timing only — results are wrong.
     (2) The same for the one-nanobatch step (its floor without those kernels).
     (3) The nanobatched step with a busy wait added to the host's work per step: GPU time against host time.
+    (4) The nanobatched step with the attention kernels in the forms that fill the chip on their own (no
+        key split at one sequence), leaving fewer idle compute units to the other streams but less work.
     All interleaved after a pre-heat, median ms per step."""
     from kareus_amd.backend import get_backend
 
@@ -663,15 +699,20 @@ def overlap_bound(w, device, rounds=4, steps=8):
     go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
     nano = Stepper(make_model(w, w["nnb"], device), x, go)
     serial = Stepper(make_model(w, 1, device, use_streams=False), x, go)
-    for st in (nano, serial):
+    unsplit = Stepper(make_model(w, w["nnb"], device), x, go)
+    for layer in unsplit.model.layers:
+        layer.core_attention.beside_other_streams = True
+    for st in (nano, serial, unsplit):
         st.run(2)
     preheat(nano, 2.0)
     lib = get_backend("hip").lib
     hbm = ["kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rmsnorm_bwd_add", "kr_rmsnorm_dgamma", "kr_rope"]
     samples = {k: [] for k in ("nanobatched", "one nanobatch", "nanobatched, HBM-bound launches suppressed",
-                               "one nanobatch, HBM-bound launches suppressed")}
+                               "one nanobatch, HBM-bound launches suppressed",
+                               "nanobatched, attention kernels in their whole-chip forms")}
     for _ in range(rounds):
         samples["nanobatched"].append(nano.timed(steps))
+        samples["nanobatched, attention kernels in their whole-chip forms"].append(unsplit.timed(steps))
         samples["one nanobatch"].append(serial.timed(steps))
         with _SuppressedLaunches(lib, hbm):
             samples["nanobatched, HBM-bound launches suppressed"].append(nano.timed(steps))
@@ -970,7 +1011,7 @@ def main():
     entries = []
     for alone in [alone_main] + alone_others:
         layout = alone["kernel"].split("<")[1][:2]
-        acc = (run_nnb > 1) if layout == "NT" else None     # the accumulating launches of the weight gradient
+        acc = None
         s, n_launches = in_step.seconds(watched[layout], acc)
         if s is None:
             entries.append(dict(alone, measured="back to back on its own"))

@@ -54,9 +54,10 @@ int kr_device_clock_mhz(void);
 size_t kr_gemm_workspace_bytes(int layout, int M, int N, int K);
 /* Workspace for a GEMM that shares the GPU with kernels of other streams.  The split count of
  * kr_gemm_workspace_bytes() minimises the GEMM's own latency; with latency_weight < 1 the choice
- * leans towards the smallest total CU-time instead (0.3 is a good value beside other nanobatch
- * streams), which never asks for more splits.  kr_gemm_bf16 uses as many splits as the workspace
- * it is handed holds, at most the latency-optimal count.                                      */
+ * leans towards the smallest total CU-time instead, which never asks for more splits.  A launch
+ * flagged KR_GEMM_BESIDE_OTHER_STREAMS is planned with weight 0.1: size its workspace with that
+ * value, so that the cuts the dispatcher plans are the cuts the buffer holds.  kr_gemm_bf16 uses
+ * as many splits as the workspace it is handed holds, at most the planned count.              */
 size_t kr_gemm_workspace_bytes_shared(int layout, int M, int N, int K, float latency_weight);
 int kr_gemm_bf16(int layout, int M, int N, int K,
                  const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -123,6 +124,24 @@ int kr_gemm_bf16_runs(int layout, int M, int N, int K,
                       int epilogue, const void* aux, int64_t ld_aux, int aux_run_rows, int64_t aux_run_ld,
                       void* out2, int64_t ld_out2,
                       int max_cus, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The weight gradient of a linear layer over all nanobatches of a microbatch in one launch.  The
+ * reference computes dW = dy^T . x once per nanobatch and sums the products in main_grad
+ * (accumulate_into_grad_weight, kareus/transformer_engine/pytorch/ops/basic/basic_linear_bias.py:229-263,
+ * GEMM call basic_linear.py:898-909): n launches whose contraction is a nanobatch's tokens, each with a
+ * read-modify-write of the whole gradient.  The sum over nanobatches is the same contraction continued,
+ * so this entry point takes the n operand pairs where they lie and runs one GEMM over all their tokens:
+ *   C[M, N] (+)= sum_i A_i^T . B_i,  A_i [k_seg, M] (row stride lda), B_i [k_seg, N] (row stride ldb)
+ * for i < nseg <= KR_GEMM_MAX_SEGMENTS; the pieces may be anywhere in memory (16-byte aligned), k_seg must
+ * be a multiple of 64 (KR_EUNSUPPORTED otherwise: the caller then accumulates pair by pair).  Tiling,
+ * cuts of the contraction, workspace and `max_cus` as for layout NT of kr_gemm_bf16_fused on
+ * K = nseg * k_seg (size the workspace with that K); flags: 0 or KR_GEMM_BESIDE_OTHER_STREAMS.
+ * The fp32 sum runs over the pieces in the order given and is rounded to bf16 once.                  */
+#define KR_GEMM_MAX_SEGMENTS 8
+int kr_gemm_bf16_nt_segments(int M, int N, int k_seg, int nseg,
+                             const void* const* A, int64_t lda, const void* const* B, int64_t ldb,
+                             void* C, int64_t ldc, int accumulate, int flags,
+                             int max_cus, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- RMSNorm ---------------------------------------------------------------------------
  * Replaces transformer_engine_torch.rmsnorm_fwd / rmsnorm_bwd

@@ -66,6 +66,15 @@ class EagerBackend:
             out.copy_(dw)
         return out
 
+    @staticmethod
+    def wgrad_segments_ok(dys, xs) -> bool:
+        return len(dys) == len(xs) >= 1
+
+    def linear_wgrad_segments(self, dys, xs, out: Tensor = None, accumulate: bool = False,
+                              split_k: bool = True) -> Tensor:
+        """``sum_i dys[i]^T . xs[i]`` as one product over all rows."""
+        return self.linear_wgrad(torch.cat(list(dys)), torch.cat(list(xs)), out=out, accumulate=accumulate)
+
     # rs = rsqrt(mean(x^2) + eps) in fp32, y = (x * rs) * gamma
     # (3rdparty/TransformerEngine/transformer_engine/common/normalization/rmsnorm/
     #  rmsnorm_fwd_kernels.cuh:90-121)

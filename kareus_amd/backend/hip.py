@@ -36,6 +36,8 @@ _SIGNATURES = {
     "kr_gemm_bf16_runs": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p, _c_i64,
                                    _c_void_p, _c_i64, _c_int, _c_i64, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64,
                                    _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
+    "kr_gemm_bf16_nt_segments": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
+                                          _c_void_p, _c_i64, _c_int, _c_int, _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
     "kr_rmsnorm_fwd_runs": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_int, _c_i64,
                                      _c_float, _c_void_p]),
@@ -189,6 +191,11 @@ class HipBackend:
             n = self._cu_count[device.index] = torch.cuda.get_device_properties(device).multi_processor_count
         return n
 
+    # the weight the library's planner gives a launch's own latency (against its compute-unit time) when the
+    # launch runs beside other streams' kernels (KR_GEMM_BESIDE_OTHER_STREAMS): the workspace is sized with
+    # the same weight, so the cuts the dispatcher plans are the cuts the buffer holds
+    SHARED_LATENCY_WEIGHT = 0.1
+
     def _workspace(self, nbytes: int, device) -> Tensor:
         """A workspace of at least ``nbytes`` for the current stream.  One buffer per (stream, size
         class) is kept and reused: kernels on one stream run in order, so consecutive launches may
@@ -254,7 +261,7 @@ class HipBackend:
             ws_bytes = self._gemm_ws_bytes.get(key)
             if ws_bytes is None:
                 ws_bytes = (self.lib.kr_gemm_workspace_bytes(layout, m, n, k) if split_k else
-                            self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, 0.3))
+                            self.lib.kr_gemm_workspace_bytes_shared(layout, m, n, k, self.SHARED_LATENCY_WEIGHT))
                 self._gemm_ws_bytes[key] = ws_bytes
             if ws_bytes:
                 ws_ptr = self._workspace(ws_bytes, a.device).data_ptr()
@@ -313,6 +320,65 @@ class HipBackend:
                      split_k: bool = True) -> Tensor:
         return self.gemm(KR_GEMM_NT, dy, x, dy.shape[-1], x.shape[1], self._nrows(dy), out=out,
                          accumulate=accumulate, split_k=split_k)
+
+    MAX_WGRAD_SEGMENTS = 8   # KR_GEMM_MAX_SEGMENTS
+
+    def wgrad_segments_ok(self, dys, xs) -> bool:
+        """Whether ``linear_wgrad_segments`` takes these operand pairs: plain matrices (one row stride, the
+        same in every pair), the same shapes, a multiple of 64 rows each, at most MAX_WGRAD_SEGMENTS pairs."""
+        if not 1 <= len(dys) == len(xs) <= self.MAX_WGRAD_SEGMENTS:
+            return False
+        first = None
+        for dy, x in zip(dys, xs):
+            a, b = self._operand(dy), self._operand(x)
+            if a is None or b is None or a[2] > 1 or b[2] > 1 or a[0] != b[0] or a[0] % 64:
+                return False
+            if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or not dy.is_cuda or x.device != dy.device:
+                return False
+            key = (a[0], a[1], b[1], dy.shape[-1], x.shape[-1])
+            if first is None:
+                first = key
+            elif key != first:
+                return False
+        return True
+
+    def linear_wgrad_segments(self, dys, xs, out: Tensor = None, accumulate: bool = False,
+                              split_k: bool = True) -> Tensor:
+        """``sum_i dys[i]^T . xs[i]`` in one launch: the weight gradient over all nanobatches of a
+        microbatch, each pair read where it lies (``wgrad_segments_ok`` says whether the pairs qualify)."""
+        if not self.wgrad_segments_ok(dys, xs):
+            raise RuntimeError("linear_wgrad_segments: operand pairs must be plain matrices of one shape and row "
+                               "stride with a multiple of 64 rows each")
+        nseg = len(dys)
+        a0, b0 = self._operand(dys[0]), self._operand(xs[0])
+        k_seg, m, n = a0[0], dys[0].shape[-1], xs[0].shape[-1]
+        if out is None:
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=dys[0].device)
+        c_op = self._operand(out)
+        if c_op is None or c_op[2] > 1 or tuple(out.shape) != (m, n):
+            raise RuntimeError("linear_wgrad_segments: out must be a [M, N] matrix with one row stride")
+        ws_bytes, ws_ptr = 0, None
+        if split_k is not None:
+            key = (KR_GEMM_NT, m, n, k_seg * nseg, split_k)
+            ws_bytes = self._gemm_ws_bytes.get(key)
+            if ws_bytes is None:
+                ws_bytes = (self.lib.kr_gemm_workspace_bytes(KR_GEMM_NT, m, n, k_seg * nseg) if split_k else
+                            self.lib.kr_gemm_workspace_bytes_shared(KR_GEMM_NT, m, n, k_seg * nseg, self.SHARED_LATENCY_WEIGHT))
+                self._gemm_ws_bytes[key] = ws_bytes
+            if ws_bytes:
+                ws_ptr = self._workspace(ws_bytes, out.device).data_ptr()
+        max_cus = 0
+        reserved = reserved_compute_units()
+        if reserved:
+            max_cus = max(self._num_cus(out.device) - reserved, 8)
+        ptrs = ctypes.c_void_p * nseg
+        a_ptrs = ptrs(*[t.data_ptr() for t in dys])
+        b_ptrs = ptrs(*[t.data_ptr() for t in xs])
+        rc = self.lib.kr_gemm_bf16_nt_segments(m, n, k_seg, nseg, a_ptrs, a0[1], b_ptrs, b0[1], out.data_ptr(), c_op[1],
+                                               int(accumulate), 0x100 if split_k is False else 0, int(max_cus),
+                                               ws_ptr, ws_bytes, self._stream())
+        self._check(rc, f"kr_gemm_bf16_nt_segments(M={m}, N={n}, k_seg={k_seg}, nseg={nseg})")
+        return out
 
     # -- RMSNorm ----------------------------------------------------------------------
     @staticmethod

@@ -69,6 +69,10 @@ class LayerConfig:
     checkpoint_activations: bool = False
     # weight gradients of all nanobatches are summed inside the wgrad GEMM instead of by autograd
     fuse_wgrad_accumulation: bool = True
+    # ... and, where the backend can contract operand pieces, by ONE GEMM per layer over the tokens of all
+    # nanobatches, launched when the last nanobatch has delivered its operands (instead of one
+    # accumulating GEMM per nanobatch); the nanobatches' operands stay alive until then
+    wgrad_over_all_nanobatches: bool = True
     # nanobatch outputs (and input gradients) are written into slices of one tensor by the ops
     # that produce them, so joining the nanobatches needs no concatenation
     join_nanobatches_in_place: bool = True

@@ -203,6 +203,16 @@ struct RowRuns {
   int a_sh, a_outer, c_sh, c_outer, x_sh, x_outer;
 };
 
+// The contraction of a weight gradient over the nanobatches of a microbatch: layout NT, operands in up
+// to KR_GEMM_MAX_SEGMENTS pieces (one pair per nanobatch, each `steps` K-steps of 64 rows long, all with
+// the row strides lda / ldb), contracted one after the other into one sum.
+constexpr int MAX_SEGMENTS = KR_GEMM_MAX_SEGMENTS;
+struct Segments {
+  const bf16* a[MAX_SEGMENTS];
+  const bf16* b[MAX_SEGMENTS];
+  int n, steps;
+};
+
 template <int WN>
 struct Frags {
   bf16x8 a[WT], b[WN];
@@ -217,7 +227,9 @@ struct Count { static constexpr int value = N; };
 // a run-time switch: the plain instances carry none of the extra code or registers.
 // RUNS: the instance honours row runs of A, C and aux (RowRuns); the plain instances do not carry the
 // extra address arithmetic or its registers.
-template <bool A_T, bool B_T, int WN, int EPI, bool RUNS = false>
+// SEG (layout NT): A and B are the pieces named by `segs` (the A / B arguments are unused); K is their
+// total length.
+template <bool A_T, bool B_T, int WN, int EPI, bool RUNS = false, bool SEG = false>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__ A, int lda,
                                                         const bf16* __restrict__ B, int ldb,
                                                         bf16* __restrict__ C, int ldc, int M,
@@ -225,7 +237,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
                                                         int splits, float* __restrict__ partial,
                                                         const bf16* __restrict__ aux, int ld_aux,
                                                         bf16* __restrict__ out2, int ld_out2,
-                                                        RowRuns runs_arg) {
+                                                        RowRuns runs_arg, Segments segs) {
+  static_assert(!SEG || (A_T && B_T && !RUNS), "operand pieces: layout NT, plain rows");
   // (without RUNS every run length reads as a compile-time 1: the branches below fold away)
   const RowRuns runs = RUNS ? runs_arg : RowRuns{0, 0, 0, 0, 0, 0};
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
@@ -266,16 +279,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   // items blockIdx.x, blockIdx.x + gridDim.x, ...  The state below describes the current item.
   // (element offsets fit 32 bits: the host checks rows * ld < 2^31 and the workspace size)
   int m0, n0, nk, k_tail, kc = K, a_off = 0, b_off = 0, p_off = 0;
+  const bf16 *seg_a = A, *seg_b = B;
+  int seg_left = 0, seg_next = 0;
   auto select_item = [&](int v) {
     const int split = v / ntiles;
     int tile_m, tile_n;
     remap_block(v - split * ntiles, ntiles, tiles_m, tiles_n, tile_m, tile_n);
     m0 = tile_m * BM;
     n0 = swiglu ? tile_n * (16 * WN) : tile_n * BN_;
+    int k0 = 0;
     if (split_k) {
       // split-K: contraction range [split*k_per, split*k_per + kc), fp32 partial tile out
       // (k_per is a multiple of 64)
-      const int k0 = split * k_per;
+      k0 = split * k_per;
       a_off = A_T ? (runs.a_sh ? (k0 >> runs.a_sh) * runs.a_outer : k0 * lda) : k0;
       b_off = B_T ? k0 * ldb : k0;
       kc = (K - k0) < k_per ? (K - k0) : k_per;
@@ -283,10 +299,38 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     }
     nk = (kc + BK - 1) / BK;
     k_tail = kc - (nk - 1) * BK;  // valid contraction rows of the last K-step (8..64)
+    if constexpr (SEG) {
+      // the request cursor goes to K-step k0 / 64 of the whole contraction
+      const int g0 = k0 / BK, sg = g0 / segs.steps, within = g0 - sg * segs.steps;
+      seg_a = segs.a[sg] + (int64_t)within * (BK * lda);
+      seg_b = segs.b[sg] + (int64_t)within * (BK * ldb);
+      seg_left = segs.steps - within;
+      seg_next = sg + 1;
+    }
   };
   const int a_step = A_T ? (runs.a_sh ? (BK >> runs.a_sh) * runs.a_outer : BK * lda) : BK;
-  auto a_base = [&](int t) { return A + a_off + (int64_t)t * a_step; };
-  auto b_base = [&](int t) { return B + b_off + (int64_t)t * (B_T ? BK * ldb : BK); };
+  // SEG: K-steps are requested strictly in order (A then B of a step), so the bases are a cursor that
+  // seg_advance() moves on behind the requests of a step; `t` is not needed
+  auto a_base = [&](int t) {
+    if constexpr (SEG) return seg_a; else return A + a_off + (int64_t)t * a_step;
+  };
+  auto b_base = [&](int t) {
+    if constexpr (SEG) return seg_b; else return B + b_off + (int64_t)t * (B_T ? BK * ldb : BK);
+  };
+  auto seg_advance = [&]() {
+    if constexpr (SEG) {
+      seg_a += BK * lda;
+      seg_b += BK * ldb;
+      if (--seg_left == 0) {
+        if (seg_next < segs.n) {
+          seg_a = segs.a[seg_next];
+          seg_b = segs.b[seg_next];
+        }
+        seg_left = segs.steps;
+        ++seg_next;
+      }
+    }
+  };
 
   // The ring of five 32 KB slots as LDS byte addresses, in ring order starting at A of the
   // current K-step t: r0 = A(t), r1 = B(t), r2 = A(t+1), r3 = B(t+1), r4 = A(t+2); B(t+2) goes
@@ -331,10 +375,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     set_offsets(nk == 1 ? k_tail : BK);
     request(a_base(0), la, r0, Count<8>{});
     request(b_base(0), lb, r1, Count<NB_LOADS>{});
+    seg_advance();
     if (nk > 1) {
       if (nk == 2 && k_tail != BK) set_offsets(k_tail);
       request(a_base(1), la, r2, Count<8>{});
       request(b_base(1), lb, r3, Count<NB_LOADS>{});
+      seg_advance();
     }
   };
   // After this wave's loads of the last K-step have landed (A in slot sa, B in slot sb): zero
@@ -481,6 +527,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
       __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8)
       __syncthreads();
       half(Y, X, r2, r3, 0, Count<NB_LOADS>{}, b_base(t + 2), lb, r0);
+      seg_advance();
       rotate();
     }
     for (; t < nk; ++t) {
@@ -797,7 +844,7 @@ inline int choose_wn(int M, int N, int num_cus) {
 //   CU-time  the same work summed over the CUs it occupies, per CU of the device.
 // A GEMM that has the GPU to itself wants the smallest latency (latency_weight 1); one that
 // runs beside kernels of other streams, which can use the CUs it leaves idle, should mostly
-// keep its CU-time small (latency_weight ~0.3).  `max_splits` is what the caller's workspace holds.
+// keep its CU-time small (the dispatcher uses latency_weight 0.1).  `max_splits` is what the caller's workspace holds.
 struct Plan {
   int wn, splits;
 };
@@ -848,6 +895,7 @@ struct Fused {
   int max_cus = 0;          // > 0: use at most this many compute units
   bool shared = false;      // other streams' kernels use the units this launch leaves idle
   RowRuns runs = {0, 0, 0, 0, 0, 0};  // row runs of A, C, aux (all plain by default)
+  const Segments* segs = nullptr;     // layout NT: the operands come in these pieces (A and B are unused)
 };
 
 // Tile width for a projection with the SwiGLU epilogue: the tiles have to divide the 2F output
@@ -868,16 +916,22 @@ inline int swiglu_wn(int M, int N, int num_cus) {
   return best;
 }
 
+using GemmKernel = void (*)(const bf16*, int, const bf16*, int, bf16*, int, int, int, int, int, int, int, float*,
+                            const bf16*, int, bf16*, int, RowRuns, Segments);
+
+// raises the dynamic-LDS limit of one kernel instance, once (thread-safe static initialisation)
+template <GemmKernel FN>
+hipError_t raise_lds_limit() {
+  static const hipError_t status = hipFuncSetAttribute((const void*)FN, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       (int)(NSLOTS * TILE * sizeof(bf16)));
+  return status;
+}
+
 template <bool A_T, bool B_T, int WN, int EPI = KR_GEMM_EPI_NONE>
 int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int64_t ldc, int M,
            int N, int K, int accumulate, float* workspace, size_t workspace_bytes,
            hipStream_t stream, int num_cus, const Fused& fu, int planned_splits = 1) {
   constexpr size_t lds_bytes = NSLOTS * TILE * sizeof(bf16);
-  // raise the dynamic-LDS limit once per instantiation (thread-safe static initialisation)
-  static const hipError_t attr_status =
-      hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN, EPI>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (attr_status != hipSuccess) return KR_ELAUNCH;
   if (fu.max_cus > 0 && fu.max_cus < num_cus) num_cus = fu.max_cus;
   const int tiles = ((M + BM - 1) / BM) * ((N + 32 * WN - 1) / (32 * WN));
   // the planned count, which the dispatcher has already capped by what the caller's workspace holds
@@ -902,50 +956,44 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
     return g < num_cus ? g : num_cus;
   };
   const bool with_runs = fu.runs.a_sh || fu.runs.c_sh || fu.runs.x_sh;
+  const bool with_segs = fu.segs != nullptr;
   // instances that honour row runs exist for what the two ends of a layer stack launch: the residual-add
   // forward (aux or C in runs), the input gradient (plain or with the SwiGLU backward) and the weight
-  // gradient (A in runs)
+  // gradient (A in runs); instances that contract operand pieces for the weight gradient (both forms)
   constexpr bool kRunsInstance = EPI == KR_GEMM_EPI_ADD || EPI == KR_GEMM_EPI_SWIGLU_BWD || (EPI == KR_GEMM_EPI_NONE && B_T);
-  if (with_runs && !kRunsInstance) return KR_EUNSUPPORTED;
+  constexpr bool kSegsInstance = A_T && B_T && (EPI == KR_GEMM_EPI_NONE || EPI == KR_GEMM_EPI_TRANSPOSED_OUT);
+  if ((with_runs && !kRunsInstance) || (with_segs && (!kSegsInstance || with_runs))) return KR_EUNSUPPORTED;
+  GemmKernel fn = gemm_kernel<A_T, B_T, WN, EPI>;
+  hipError_t attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI>>();
   if constexpr (kRunsInstance) {
-    static const hipError_t attr_runs =
-        hipFuncSetAttribute((const void*)gemm_kernel<A_T, B_T, WN, EPI, true>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (with_runs && attr_runs != hipSuccess) return KR_ELAUNCH;
-  }
-  if (splits == 1) {
-    const int grid = grid_for(tiles);
-    if constexpr (kRunsInstance) {
-      if (with_runs) {
-        hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, EPI, true>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
-                           (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr,
-                           fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2, fu.runs);
-        return kr_launch_status();
-      }
+    if (with_runs) {
+      fn = gemm_kernel<A_T, B_T, WN, EPI, true>;
+      attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI, true>>();
     }
-    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, EPI>), dim3(grid), dim3(NTHREADS), lds_bytes, stream, A,
-                       (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr,
-                       fu.aux, (int)fu.ld_aux, fu.out2, (int)fu.ld_out2, fu.runs);
+  }
+  if constexpr (kSegsInstance) {
+    if (with_segs) {
+      fn = gemm_kernel<A_T, B_T, WN, EPI, false, true>;
+      attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI, false, true>>();
+    }
+  }
+  if (attr_status != hipSuccess) return KR_ELAUNCH;
+  const Segments segs = with_segs ? *fu.segs : Segments{};
+  if (splits == 1) {
+    hipLaunchKernelGGL(fn, dim3(grid_for(tiles)), dim3(NTHREADS), lds_bytes, stream, A, (int)lda, B, (int)ldb, C,
+                       (int)ldc, M, N, K, accumulate, 0, 1, (float*)nullptr, fu.aux, (int)fu.ld_aux, fu.out2,
+                       (int)fu.ld_out2, fu.runs, segs);
     return kr_launch_status();
   }
+  if constexpr (EPI != KR_GEMM_EPI_NONE) return KR_EINVAL;  // (not reached: a fused launch never splits)
   int k_per = (K + splits - 1) / splits;
   k_per = (k_per + BK - 1) / BK * BK;
   splits = (K + k_per - 1) / k_per;
   const int items = tiles * splits;
-  if constexpr (EPI != KR_GEMM_EPI_NONE) return KR_EINVAL;  // (not reached: a fused launch never splits)
-  bool launched = false;
-  if constexpr (EPI == KR_GEMM_EPI_NONE && B_T) {
-    if (with_runs) {   // (only A can be in runs here: an output in runs is never cut)
-      hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE, true>), dim3(grid_for(items)), dim3(NTHREADS),
-                         lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
-                         (const bf16*)nullptr, 0, (bf16*)nullptr, 0, fu.runs);
-      launched = true;
-    }
-  }
-  if (!launched)
-    hipLaunchKernelGGL((gemm_kernel<A_T, B_T, WN, KR_GEMM_EPI_NONE>), dim3(grid_for(items)), dim3(NTHREADS),
-                       lds_bytes, stream, A, (int)lda, B, (int)ldb, C, (int)ldc, M, N, K, 0, k_per, splits, workspace,
-                       (const bf16*)nullptr, 0, (bf16*)nullptr, 0, fu.runs);
+  // (of the operands only A can be in runs here: an output in runs is never cut)
+  hipLaunchKernelGGL(fn, dim3(grid_for(items)), dim3(NTHREADS), lds_bytes, stream, A, (int)lda, B, (int)ldb, C,
+                     (int)ldc, M, N, K, 0, k_per, splits, workspace, (const bf16*)nullptr, 0, (bf16*)nullptr, 0,
+                     fu.runs, segs);
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int64_t work = (int64_t)M * (N / 8);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream,
@@ -1118,8 +1166,20 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
         const int tiles_direct = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
         const int tiles_trans = ((N + BM - 1) / BM) * ((M + BN - 1) / BN);
         if (tiles_direct >= 192 && tiles_trans >= 192 && cost(N, M, wt) < cost(M, N, wn)) {
+          // (operand pieces change places with the operands)
+          Segments exchanged{};
+          Fused fut = fu;
+          if (fu.segs != nullptr) {
+            for (int i = 0; i < MAX_SEGMENTS; ++i) {
+              exchanged.a[i] = fu.segs->b[i];
+              exchanged.b[i] = fu.segs->a[i];
+            }
+            exchanged.n = fu.segs->n;
+            exchanged.steps = fu.segs->steps;
+            fut.segs = &exchanged;
+          }
 #define KR_GEMM_TRANS(W) \
-  return launch<true, true, W, KR_GEMM_EPI_TRANSPOSED_OUT>(b, ldb, a, lda, c, ldc, N, M, K, 0, nullptr, 0, st, num_cus, fu)
+  return launch<true, true, W, KR_GEMM_EPI_TRANSPOSED_OUT>(b, ldb, a, lda, c, ldc, N, M, K, 0, nullptr, 0, st, num_cus, fut)
           switch (wt) {
             case 5: KR_GEMM_TRANS(5);
             case 6: KR_GEMM_TRANS(6);
@@ -1192,4 +1252,32 @@ extern "C" int kr_gemm_bf16_runs(int layout, int M, int N, int K, const void* A,
   fu.runs = {sh[0], sh[0] ? (int)a_run_ld : 0, sh[1], sh[1] ? (int)c_run_ld : 0, sh[2], sh[2] ? (int)aux_run_ld : 0};
   return gemm_dispatch(layout, M, N, K, A, lda, B, ldb, C, ldc, accumulate, workspace, workspace_bytes,
                        stream, fu);
+}
+
+// A weight gradient over the nanobatches of a microbatch in one launch: C[M, N] (+)= sum_i A_i^T . B_i with
+// A_i [k_seg, M] (row stride lda) and B_i [k_seg, N] (row stride ldb), i < nseg <= KR_GEMM_MAX_SEGMENTS, the
+// pieces anywhere in memory.  The same kernels as layout NT of kr_gemm_bf16 on K = nseg * k_seg, with the
+// operand base exchanged at every piece boundary; k_seg must be a multiple of 64.
+extern "C" int kr_gemm_bf16_nt_segments(int M, int N, int k_seg, int nseg, const void* const* A, int64_t lda,
+                                        const void* const* B, int64_t ldb, void* C, int64_t ldc,
+                                        int accumulate, int flags, int max_cus, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+  if (!A || !B || nseg < 1 || nseg > MAX_SEGMENTS || k_seg <= 0) return KR_EINVAL;
+  if (flags & ~KR_GEMM_BESIDE_OTHER_STREAMS) return KR_EINVAL;
+  if (k_seg % BK) return KR_EUNSUPPORTED;
+  if ((int64_t)k_seg * nseg >= (int64_t)1 << 31) return KR_EUNSUPPORTED;
+  Segments segs{};
+  for (int i = 0; i < nseg; ++i) {
+    if (!A[i] || !B[i] || !kr_aligned16(A[i]) || !kr_aligned16(B[i])) return KR_EINVAL;
+    segs.a[i] = (const bf16*)A[i];
+    segs.b[i] = (const bf16*)B[i];
+  }
+  segs.n = nseg;
+  segs.steps = k_seg / BK;
+  Fused fu;
+  fu.shared = (flags & KR_GEMM_BESIDE_OTHER_STREAMS) != 0;
+  fu.max_cus = max_cus;
+  fu.segs = &segs;
+  return gemm_dispatch(KR_GEMM_NT, M, N, k_seg * nseg, A[0], lda, B[0], ldb, C, ldc, accumulate, workspace,
+                       workspace_bytes, stream, fu);
 }

@@ -73,6 +73,8 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
     # ranks has to come first, so the flag is only ever set for a world size of one.
     fuse_residual = False
     forward_accepts_out_sink = False
+    # how the one weight-gradient GEMM over all nanobatches is planned (see HipBackend.gemm's split_k)
+    wgrad_over_all_split_k = True
 
     def get_input_channels(self) -> List[Channel]:
         if self.fuse_residual:
@@ -171,18 +173,63 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
 
     @staticmethod
     def _weight_grad(be, ctx, dy, x2d, split_k=True):
-        """``dW = dy^T . x``.  When the engine attached a ``wgrad_sink`` — one dict shared by
-        this layer's contexts of all nanobatches of one backward pass — the first nanobatch to
-        get here allocates the gradient and every later one adds its product into the same
-        buffer inside the GEMM (the role of ``accumulate_into_main_grad``,
-        kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:898-909), after waiting for
-        the previous writer's event; later nanobatches then report ``None`` so that autograd
-        does not sum a second time."""
+        """``dW = dy^T . x``.  The engine attaches a ``wgrad_sink`` — one dict shared by this layer's
+        contexts of all nanobatches of one backward pass — so that the layer's gradient is summed over
+        the nanobatches here and autograd sees one tensor (the role of ``accumulate_into_main_grad``,
+        kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:898-909); the nanobatches that do
+        not deliver it report ``None``.
+
+        Where the backend can contract operand pieces (``linear_wgrad_segments``), the sum over the
+        nanobatches is one GEMM over all their tokens: every nanobatch leaves its ``(dy, x)`` pair and an
+        event in the sink, and the last one to get here launches the product of all pairs, in nanobatch
+        order, on the stream of the nanobatch whose turn it is (the launches of a backward pass take the
+        streams in rotation, so no nanobatch's chain of input gradients waits behind all of them).
+        Otherwise the first nanobatch allocates the gradient and every later one adds its product into
+        it inside its own GEMM, after waiting for the previous writer's event."""
         sink = getattr(ctx, "wgrad_sink", None)
         if sink is None:
             return be.linear_wgrad(dy, x2d, split_k=split_k)
         api = stream_api()
         here = api.current_stream()
+        n = sink.get("n", 0)
+        if n > 1 and sink.get("defer", True) and hasattr(be, "linear_wgrad_segments"):
+            ev = None
+            if here is not None:
+                ev = api.new_event()
+                ev.record(here)
+            pairs = sink.setdefault("pairs", [])
+            # (aliases: the engine drops the storage behind the saved tensor objects after each backward op)
+            pairs.append((getattr(ctx, "nanobatch_index", len(pairs)), dy.detach(), x2d.detach(), ev, here))
+            if len(pairs) < n:
+                return None
+            pairs.sort(key=lambda p: p[0])
+            sink["pairs"] = None
+            turn = sink.get("turn")
+            if turn is None:
+                turn = [0]
+            target = pairs[turn[0] % n][4]
+            turn[0] += 1
+            dys, xs = [p[1] for p in pairs], [p[2] for p in pairs]
+            with api.stream(target):
+                if target is not None:
+                    for _, _, _, ready, st in pairs:
+                        if ready is not None and st != target:
+                            target.wait_event(ready)
+                if be.wgrad_segments_ok(dys, xs):
+                    # the one launch is planned as a GEMM that has the device to itself (cuts of the contraction
+                    # where the output has few tiles): the products of the other nanobatches, which used to
+                    # fill the device beside each other, are inside it
+                    dw = be.linear_wgrad_segments(dys, xs, split_k=PartitionableLinear.wgrad_over_all_split_k)
+                else:
+                    dw = be.linear_wgrad(dys[0], xs[0], split_k=split_k)
+                    for d, x in zip(dys[1:], xs[1:]):
+                        be.linear_wgrad(d, x, out=dw, accumulate=True, split_k=split_k)
+                if target is not None:
+                    # the operands were allocated on their own nanobatch's stream
+                    for t in dys + xs:
+                        if t.is_cuda:
+                            t.record_stream(target)
+            return dw
         buf = sink.get("buf")
         if buf is None:
             buf = sink["buf"] = be.linear_wgrad(dy, x2d, split_k=split_k)

@@ -206,6 +206,7 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         func_ctx.attention_mask = mask
         func_ctx.checkpoint_activations = checkpoint_activations
         func_ctx.fuse_wgrad_accumulation = bool(getattr(config, "fuse_wgrad_accumulation", False))
+        func_ctx.wgrad_over_all_nanobatches = bool(getattr(config, "wgrad_over_all_nanobatches", True))
         func_ctx.join_in_place = in_place
 
         if checkpoint_activations:
@@ -263,9 +264,14 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         if func_ctx.fuse_wgrad_accumulation and n > 1:
             # one sink per layer operator, shared by that operator's contexts of all nanobatches
             sinks: Dict[int, dict] = {}
+            # ("turn": a counter all sinks share, by which launches that serve all nanobatches take the
+            # nanobatch streams in rotation)
+            turn = [0]
             for c in ctxs:
                 for op_id, op_ctx in c.op_contexts.items():
-                    op_ctx.wgrad_sink = sinks.setdefault(op_id, {"n": n})
+                    op_ctx.wgrad_sink = sinks.setdefault(
+                        op_id, {"n": n, "turn": turn, "defer": func_ctx.wgrad_over_all_nanobatches})
+                    op_ctx.nanobatch_index = c.batch_idx
 
         if func_ctx.join_in_place:
             last = _last_compute_op(func_ctx.backward_tensor_graph, "backward_accepts_out_sink")

@@ -78,6 +78,24 @@ def test_fused_weight_gradient_accumulation_equals_autograd_sum(recompute):
         assert (a - b).abs().max() <= 1e-5 * b.abs().max()
 
 
+@pytest.mark.parametrize("recompute", [False, True])
+def test_weight_gradient_over_all_nanobatches_equals_per_nanobatch_accumulation(recompute):
+    """One product per layer over the tokens of all nanobatches (launched by the last nanobatch to
+    deliver its operands, which survive the engine's op-by-op release of saved tensors) against one
+    accumulating product per nanobatch: the same gradient, and the oracle's."""
+    x, go, ref = _oracle(layers=2, s=128, b=4)
+    grads = {}
+    for whole in (True, False):
+        cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=4, params_dtype=torch.float32,
+                          backend="eager", checkpoint_activations=recompute,
+                          wgrad_over_all_nanobatches=whole)
+        model = LayerStack(cfg, seed=1234)
+        _check(model, x, go, ref)
+        grads[whole] = [p.grad.clone() for p in model.parameters()]
+    for a, b in zip(grads[True], grads[False]):
+        assert (a - b).abs().max() <= 1e-5 * b.abs().max()
+
+
 @pytest.mark.parametrize("b,nnb", [(4, 4), (8, 4), (4, 2)])
 @pytest.mark.parametrize("recompute", [False, True])
 def test_nanobatches_joined_in_place_equal_concatenation(b, nnb, recompute, monkeypatch):
