@@ -185,17 +185,18 @@ def partition_times(stepper, iters=3):
 # reports null.  A constant read off a profile, not something measured in this run: the entry
 # names the profile it came from, and it is only reported while the GEMM source is the one the
 # counters were read with (first 16 hex digits of its SHA-256).
-TRAFFIC_GEMM_SOURCE = "2ceda96f9e9624f7"
+TRAFFIC_GEMM_SOURCE = "bcd8c87e05236150"
 MEASURED_TRAFFIC = {
     # (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000) x 1024, means over the launches of `bench.py --roofline-only`
-    # one nanobatch of four (4096 tokens), what the default run launches; NT in its accumulating form
-    ("NT", 7168, 4096, 4096): {"bytes": (234044.6 * 2.000 + 57792.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("TN", 4096, 7168, 4096): {"bytes": (180569.3 * 2.000 + 86016.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 4096, 4096, 7168): {"bytes": (172296.5 * 2.000 + 32768.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    # one nanobatch of four (4096 tokens), what the default run launches; the weight gradient is one launch over
+    # the operand pieces of all four nanobatches
+    ("TN", 4096, 7168, 4096): {"bytes": (180574.2 * 2.000 + 86016.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 4096, 4096, 7168): {"bytes": (172287.0 * 2.000 + 32768.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NT", 7168, 4096, 16384, "pieces"): {"bytes": (784938.1 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
     # the whole microbatch as one nanobatch (16384 tokens, --nanobatches 1)
-    ("NT", 7168, 4096, 16384): {"bytes": (912593.3 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("TN", 16384, 7168, 4096): {"bytes": (721904.1 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 16384, 4096, 7168): {"bytes": (688405.2 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NT", 7168, 4096, 16384): {"bytes": (878834.5 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 16384, 7168, 4096): {"bytes": (723189.6 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 16384, 4096, 7168): {"bytes": (688400.1 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
 }
 
 
@@ -267,7 +268,8 @@ def time_gemm(be, layout, m, n, k, device, launches=30, fused_swiglu=False, resi
 def _roofline_entry(kernel, layout, m, n, k, sec):
     flops = 2.0 * m * n * k
     achieved = flops / sec / 1e12
-    traffic = MEASURED_TRAFFIC.get((layout, m, n, k)) if _gemm_source_is_the_profiled_one() else None
+    key = (layout, m, n, k, "pieces") if "one launch over" in kernel else (layout, m, n, k)
+    traffic = MEASURED_TRAFFIC.get(key) if _gemm_source_is_the_profiled_one() else None
     return {
         "bound": "mfma", "kernel": kernel, "shape": [m, n, k],
         "flops_per_launch": flops, "avg_launch_us": sec * 1e6,
@@ -689,8 +691,9 @@ def overlap_bound(w, device, rounds=4, steps=8):
         completely behind the other nanobatches' MFMA-bound kernels.  Timing only — results are wrong.
     (2) The same for the one-nanobatch step (its floor without those kernels).
     (3) The nanobatched step with a busy wait added to the host's work per step: GPU time against host time.
-    (4) The nanobatched step with the attention kernels in the forms that fill the chip on their own (no
-        key split at one sequence), leaving fewer idle compute units to the other streams but less work.
+    (4) The nanobatched step with the attention kernels in the forms they take when a launch has the device
+        to itself (keys split between the halves of a workgroup at one sequence) instead of the forms the engine
+        picks beside other streams (no split: fewer workgroups, less compute-unit time).
     All interleaved after a pre-heat, median ms per step."""
     from kareus_amd.backend import get_backend
 
@@ -701,7 +704,7 @@ def overlap_bound(w, device, rounds=4, steps=8):
     serial = Stepper(make_model(w, 1, device, use_streams=False), x, go)
     unsplit = Stepper(make_model(w, w["nnb"], device), x, go)
     for layer in unsplit.model.layers:
-        layer.core_attention.beside_other_streams = True
+        layer.core_attention.beside_other_streams = False
     for st in (nano, serial, unsplit):
         st.run(2)
     preheat(nano, 2.0)
@@ -709,10 +712,10 @@ def overlap_bound(w, device, rounds=4, steps=8):
     hbm = ["kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rmsnorm_bwd_add", "kr_rmsnorm_dgamma", "kr_rope"]
     samples = {k: [] for k in ("nanobatched", "one nanobatch", "nanobatched, HBM-bound launches suppressed",
                                "one nanobatch, HBM-bound launches suppressed",
-                               "nanobatched, attention kernels in their whole-chip forms")}
+                               "nanobatched, attention kernels in the forms they take alone on the device")}
     for _ in range(rounds):
         samples["nanobatched"].append(nano.timed(steps))
-        samples["nanobatched, attention kernels in their whole-chip forms"].append(unsplit.timed(steps))
+        samples["nanobatched, attention kernels in the forms they take alone on the device"].append(unsplit.timed(steps))
         samples["one nanobatch"].append(serial.timed(steps))
         with _SuppressedLaunches(lib, hbm):
             samples["nanobatched, HBM-bound launches suppressed"].append(nano.timed(steps))

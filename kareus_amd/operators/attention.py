@@ -40,8 +40,8 @@ class TEDotProductAttentionOp(BasicOperation, PartitionableOperator):
         self.softmax_scale = softmax_scale
         self._backend_name = backend
         # True: the attention launches take their unsplit forms whatever the batch (KR_ATTN_BESIDE_OTHER_STREAMS),
-        # so a sequence gets the same bits in a nanobatch as in the whole microbatch.  Off by default: in the
-        # nanobatched step of the 8B shard the two choices time the same (5.64-5.66 against 5.68-5.70 ms).
+        # so a sequence gets the same bits in a nanobatch as in the whole microbatch.  The block driver sets it
+        # when the nanobatches run on streams of their own.
         self.beside_other_streams = False
 
     def get_input_channels(self) -> List[Channel]:
