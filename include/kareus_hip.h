@@ -260,7 +260,12 @@ int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* ou
  * lse: [b, nq, s] fp32 contiguous (natural log-sum-exp of the scaled, masked scores).
  * Query head h reads KV head h/per.  Causal, query i sees keys <= i.
  * hd: a multiple of 8, at most 128; any s.  Head dimension 128 with s a multiple of 128 (the
- * training workloads) runs on the MFMA kernels; every other shape on general fp32 kernels that
+ * training workloads) runs on the MFMA kernels as it lies.  Every other shape is padded into them
+ * through the workspace (zero channels up to 128, zero rows up to the next multiple of 128: the
+ * causal mask keeps the added keys from every real query, and the added queries are given a
+ * log-sum-exp that makes them inert in the backward pass): kr_attn_bwd always, the forward when it
+ * is called as kr_attn_fwd_ws with a workspace.  Without one (kr_attn_fwd, kr_attn_fwd_flags), or
+ * with KR_ATTN_GENERAL_KERNELS in the flags word, such a shape runs on general fp32 kernels that
  * are correct and slow.  All strides multiples of 8.
  * kr_attn_bwd needs a workspace of kr_attn_bwd_workspace_bytes() bytes (16-byte aligned).   */
 int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
@@ -278,6 +283,7 @@ int kr_attn_fwd(const void* q, const void* k, const void* v, void* o, float* lse
  * do not depend on the batch size.  No counterpart in the reference's call
  * (kareus/flash_attn/flash_attn_interface.py:66-80 runs one kernel at a time).                   */
 #define KR_ATTN_BESIDE_OTHER_STREAMS 0x100
+#define KR_ATTN_GENERAL_KERNELS 0x200
 int kr_attn_fwd_flags(const void* q, const void* k, const void* v, void* o, float* lse,
                       int s, int b, int nq, int nkv, int hd, float scale,
                       int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
@@ -285,6 +291,18 @@ int kr_attn_fwd_flags(const void* q, const void* k, const void* v, void* o, floa
                       int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
                       int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
                       int flags, void* stream);
+/* kr_attn_fwd_flags with a workspace of kr_attn_fwd_workspace_bytes() bytes (0 for a shape the MFMA
+ * kernels take as it lies; workspace may then be NULL): the call the reference's
+ * flash_attn_gpu.fwd (kareus/flash_attn/flash_attn_interface.py:66-80) maps to for any head
+ * dimension and sequence length it accepts.                                                      */
+size_t kr_attn_fwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);
+int kr_attn_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse,
+                   int s, int b, int nq, int nkv, int hd, float scale,
+                   int64_t q_stride_s, int64_t q_stride_b, int64_t q_stride_g, int64_t q_stride_h,
+                   int64_t k_stride_s, int64_t k_stride_b, int64_t k_stride_h,
+                   int64_t v_stride_s, int64_t v_stride_b, int64_t v_stride_h,
+                   int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
+                   int flags, void* workspace, size_t workspace_bytes, void* stream);
 size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);
 int kr_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                 const void* o, const float* lse,

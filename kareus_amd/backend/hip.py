@@ -61,6 +61,9 @@ _SIGNATURES = {
     "kr_cross_entropy_bwd": (_c_int, [_c_void_p] * 5 + [_c_i64, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_attn_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_void_p]),
     "kr_attn_fwd_flags": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 + [_c_int, _c_void_p]),
+    "kr_attn_fwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
+    "kr_attn_fwd_ws": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_float] + [_c_i64] * 14 +
+                       [_c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_attn_bwd_workspace_bytes": (_c_size_t, [_c_int] * 5),
     "kr_attn_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_void_p]),
     "kr_attn_bwd_flags": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_float] + [_c_i64] * 28 + [_c_int, _c_void_p]),
@@ -68,6 +71,7 @@ _SIGNATURES = {
 
 KR_GEMM_TN, KR_GEMM_NN, KR_GEMM_NT = 0, 1, 2
 KR_ATTN_BESIDE_OTHER_STREAMS = 0x100
+KR_ATTN_GENERAL_KERNELS = 0x200
 
 
 def library_path() -> str:
@@ -97,6 +101,7 @@ class HipBackend:
         self._gemm_ws_bytes: dict = {}  # (layout, m, n, k, split_k) -> workspace bytes
         self._ws_cache: dict = {}       # (stream, device) -> reusable workspace buffer
         self._cu_count: dict = {}       # device index -> compute units
+        self._attn_ws_bytes: dict = {}  # (s, b, nq, nkv, hd) -> forward workspace bytes of a padded shape
 
     # -- plumbing -------------------------------------------------------------------
     # the raw handle of the current stream without building a torch.cuda.Stream object: this is
@@ -673,9 +678,11 @@ class HipBackend:
         return s, b, nq, nkv, hd
 
     def attn_fwd(self, q: Tensor, k: Tensor, v: Tensor, scale: float, causal: bool = True,
-                 beside_other_streams: bool = False):
+                 beside_other_streams: bool = False, general_kernels: bool = False):
         """``beside_other_streams``: kernels of other streams use the compute units this launch leaves idle,
-        so it is shaped for the least compute-unit time, not for its own latency."""
+        so it is shaped for the least compute-unit time, not for its own latency.
+        ``general_kernels``: a shape outside the MFMA kernels (head dimension below 128, a ragged length)
+        takes the general fp32 kernels instead of being padded into the MFMA ones."""
         if not causal:
             raise RuntimeError("only causal attention is implemented")
         self._dev(q, k, v)
@@ -684,15 +691,27 @@ class HipBackend:
         per = nq // nkv
         o = torch.empty((s, b, nq, hd), dtype=q.dtype, device=q.device)
         lse = torch.empty((b, nq, s), dtype=torch.float32, device=q.device)
-        flags = KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0
-        rc = self.lib.kr_attn_fwd_flags(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
-                                        s, b, nq, nkv, hd, scale, *self._q_strides(q, per), *self._k_strides(k),
-                                        *self._k_strides(v), *self._q_strides(o, per), flags, self._stream())
+        flags = (KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0) | (KR_ATTN_GENERAL_KERNELS if general_kernels else 0)
+        nbytes = 0 if general_kernels else self._attn_fwd_ws_bytes(s, b, nq, nkv, hd)
+        ws_ptr = self._workspace(nbytes, q.device).data_ptr() if nbytes else None
+        rc = self.lib.kr_attn_fwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                                     s, b, nq, nkv, hd, scale, *self._q_strides(q, per), *self._k_strides(k),
+                                     *self._k_strides(v), *self._q_strides(o, per), flags, ws_ptr, nbytes, self._stream())
         self._check(rc, f"kr_attn_fwd(s={s}, b={b}, nq={nq}, nkv={nkv}, hd={hd})")
         return o, lse
 
+    def _attn_fwd_ws_bytes(self, s, b, nq, nkv, hd) -> int:
+        if hd == 128 and s % 128 == 0:
+            return 0
+        key = (s, b, nq, nkv, hd)
+        n = self._attn_ws_bytes.get(key)
+        if n is None:
+            n = self._attn_ws_bytes[key] = self.lib.kr_attn_fwd_workspace_bytes(s, b, nq, nkv, hd)
+        return n
+
     def attn_bwd(self, do: Tensor, q: Tensor, k: Tensor, v: Tensor, o: Tensor, lse: Tensor,
-                 scale: float, causal: bool = True, beside_other_streams: bool = False):
+                 scale: float, causal: bool = True, beside_other_streams: bool = False,
+                 general_kernels: bool = False):
         """Returns (dq, dk, dv).  If ``q`` is a grouped [s, b, ng, per, hd] view, the three
         gradients are views of one buffer laid out like the fused QKV projection output and
         carry it as ``_kr_mixed`` so the QKV-split backward can hand it on without a copy."""
@@ -715,7 +734,7 @@ class HipBackend:
             dv = torch.empty((s, b, nkv, hd), dtype=q.dtype, device=q.device)
         nbytes = self.lib.kr_attn_bwd_workspace_bytes(s, b, nq, nkv, hd)
         ws = self._workspace(max(nbytes, 16), q.device)
-        flags = KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0
+        flags = (KR_ATTN_BESIDE_OTHER_STREAMS if beside_other_streams else 0) | (KR_ATTN_GENERAL_KERNELS if general_kernels else 0)
         rc = self.lib.kr_attn_bwd_flags(do4.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), o4.data_ptr(),
                                         lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(),
                                         s, b, nq, nkv, hd, scale,

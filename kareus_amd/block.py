@@ -293,10 +293,11 @@ class LayerStack(torch.nn.Module):
         for layer in self.layers:
             for op in (layer.linear_qkv, layer.linear_proj, layer.linear_fc1, layer.linear_fc2):
                 op.split_k = streams is None
-            # beside the other nanobatch streams the attention launches take the forms that cost the least
-            # compute-unit time (no split of the keys at small batches): 0.4-0.9 % of the nanobatched step on
-            # the 3B and 8B layers, and a sequence gets the same bits whatever the nanobatch count
-            layer.core_attention.beside_other_streams = streams is not None
+            # with several nanobatches the attention launches take the forms that cost the least compute-unit
+            # time (no split of the keys at small batches), which is what counts beside the other nanobatch
+            # streams: 0.4-0.9 % of the nanobatched step on the 3B and 8B layers.  The choice follows the
+            # nanobatch count, not the streams, so that a run on one stream gives the bits of a run on several.
+            layer.core_attention.beside_other_streams = n > 1
         self.allreduce_comm_ops = [
             NoOpAllReduce(batch_idx=i, world_size=1, comm_stream=streams[(i - 1) % n] if streams else None)
             for i in range(n)

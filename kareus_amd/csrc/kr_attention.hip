@@ -1662,6 +1662,53 @@ __global__ __launch_bounds__(GTHREADS) void attn_general_dq_kernel(
 
 }  // namespace general
 
+// ---- shapes outside the MFMA kernels, padded into them -----------------------------------------
+// Head dimensions below 128 and sequence lengths that are not whole 128-row tiles are copied into
+// dense [s_pad, b, heads, 128] buffers (zeros beyond the data), run through the MFMA kernels and
+// copied back.  Zero channels add nothing to Q.K^T and give zero output channels; with the causal
+// mask a query row below s never sees a key row at or beyond s, and the rows at or beyond s are
+// made inert in the backward pass by a log-sum-exp so large that their probabilities are zero.
+__global__ __launch_bounds__(256) void attn_pad_kernel(const bf16* __restrict__ src, bf16* __restrict__ dst,
+                                                       int s, int b, int heads, int per, int hd,
+                                                       int64_t total, QLayout sl) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 16-byte vector of dst
+  if (idx >= total) return;
+  const int c = (int)(idx & 15) * 8;
+  int64_t r = idx >> 4;
+  const int head = (int)(r % heads);
+  r /= heads;
+  const int bi = (int)(r % b);
+  const int row = (int)(r / b);
+  bf16x8 v = zero8();
+  if (row < s && c < hd) v = ldg8(src + (int64_t)row * sl.s_ + sl.at(bi, head, per) + c);
+  stg8(dst + idx * 8, v);
+}
+__global__ __launch_bounds__(256) void attn_unpad_kernel(const bf16* __restrict__ src, bf16* __restrict__ dst,
+                                                         int b, int heads, int per, int hd,
+                                                         int64_t total, QLayout dl) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one 16-byte vector of dst
+  if (idx >= total) return;
+  const int vec = hd / 8;
+  const int c = (int)(idx % vec) * 8;
+  int64_t r = idx / vec;
+  const int head = (int)(r % heads);
+  r /= heads;
+  const int bi = (int)(r % b);
+  const int64_t row = r / b;
+  const bf16x8 v = ldg8(src + (((row * b + bi) * heads + head) * HD + c));
+  stg8(dst + row * dl.s_ + dl.at(bi, head, per) + c, v);
+}
+// rows of fp32 statistics [n, len_src] -> [n, len_dst]; positions beyond len_src get `fill`
+__global__ __launch_bounds__(256) void attn_resize_rows_kernel(const float* __restrict__ src,
+                                                               float* __restrict__ dst, int len_src,
+                                                               int len_dst, int64_t total, float fill) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t row = idx / len_dst;
+  const int i = (int)(idx - row * len_dst);
+  dst[idx] = i < len_src ? src[row * len_src + i] : fill;
+}
+
 }  // namespace
 
 // Build-time caps, for measuring one form of a kernel against another: the most query heads a
@@ -1676,15 +1723,68 @@ __global__ __launch_bounds__(GTHREADS) void attn_general_dq_kernel(
 // set by the first key tiles (they see every query): two workgroups then share each key tile.
 static int dkdv_query_split(int s, int b, int nq) { return (s / 128) * nq * b <= 2 * 256 ? 2 : 1; }
 
-extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
-  if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
+static int attn_padded_len(int s) { return (s + BQ - 1) / BQ * BQ; }
+// bytes of one padded [s_pad, b, heads, 128] bf16 tensor / of the padded statistics [b, nq, s_pad]
+static size_t attn_padded_bytes(int s, int b, int heads) {
+  return (size_t)attn_padded_len(s) * b * heads * HD * sizeof(bf16);
+}
+static size_t attn_padded_stat_bytes(int s, int b, int nq) {
+  return (size_t)attn_padded_len(s) * b * nq * sizeof(float);
+}
+
+// workspace of the MFMA backward kernels for a shape they take as it is
+static size_t attn_bwd_fast_bytes(int s, int b, int nq, int nkv, int hd) {
   size_t bytes = 2 * (size_t)b * nq * s * sizeof(float);  // delta, and -lse in the log2 domain
-  if (!attn_fast_path(s, hd)) return bytes;               // the general kernels only keep delta
   const int qsplit = dkdv_query_split(s, b, nq);
   if (nq != nkv || qsplit > 1)  // fp32 dK, dV partials per (query head, query-tile part)
     bytes += 2 * (size_t)b * nq * qsplit * s * hd * sizeof(float);
   return bytes;
 }
+
+extern "C" size_t kr_attn_bwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
+  if (check_attn_common(s, b, nq, nkv, hd) != KR_OK) return 0;
+  if (attn_fast_path(s, hd)) return attn_bwd_fast_bytes(s, b, nq, nkv, hd);
+  // padded copies of dO, q, o, dq (query-sized) and k, v, dk, dv (key-sized), the padded log-sum-exp, and
+  // the MFMA kernels' own workspace at the padded shape (the general kernels, which only keep delta
+  // [b, nq, s], fit in the same space)
+  return 4 * attn_padded_bytes(s, b, nq) + 4 * attn_padded_bytes(s, b, nkv) + attn_padded_stat_bytes(s, b, nq) +
+         attn_bwd_fast_bytes(attn_padded_len(s), b, nq, nkv, HD);
+}
+
+extern "C" size_t kr_attn_fwd_workspace_bytes(int s, int b, int nq, int nkv, int hd) {
+  if (check_attn_common(s, b, nq, nkv, hd) != KR_OK || attn_fast_path(s, hd)) return 0;
+  // padded copies of q, o and k, v, and the padded log-sum-exp
+  return 2 * attn_padded_bytes(s, b, nq) + 2 * attn_padded_bytes(s, b, nkv) + attn_padded_stat_bytes(s, b, nq);
+}
+
+namespace {
+// dense [s_pad, b, heads, 128] as the kernels' stride quadruple / triple
+QLayout padded_qlayout(int b, int nq, int per) {
+  return QLayout{(int64_t)b * nq * HD, (int64_t)nq * HD, (int64_t)per * HD, (int64_t)HD};
+}
+KLayout padded_klayout(int b, int nkv) { return KLayout{(int64_t)b * nkv * HD, (int64_t)nkv * HD, (int64_t)HD}; }
+
+int launch_pad(const void* src, void* dst, int s, int b, int heads, int per, int hd, QLayout sl, hipStream_t st) {
+  const int64_t total = (int64_t)attn_padded_len(s) * b * heads * (HD / 8);
+  hipLaunchKernelGGL(attn_pad_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const bf16*)src,
+                     (bf16*)dst, s, b, heads, per, hd, total, sl);
+  return hipGetLastError() == hipSuccess ? KR_OK : KR_ELAUNCH;
+}
+int launch_unpad(const void* src, void* dst, int s, int b, int heads, int per, int hd, QLayout dl, hipStream_t st) {
+  const int64_t total = (int64_t)s * b * heads * (hd / 8);
+  hipLaunchKernelGGL(attn_unpad_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const bf16*)src,
+                     (bf16*)dst, b, heads, per, hd, total, dl);
+  return hipGetLastError() == hipSuccess ? KR_OK : KR_ELAUNCH;
+}
+int launch_resize_rows(const float* src, float* dst, int64_t n, int len_src, int len_dst, float fill, hipStream_t st) {
+  const int64_t total = n * len_dst;
+  hipLaunchKernelGGL(attn_resize_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, src, dst,
+                     len_src, len_dst, total, fill);
+  return hipGetLastError() == hipSuccess ? KR_OK : KR_ELAUNCH;
+}
+// a KV-like tensor's stride triple as the quadruple the pad kernels take (one head per group)
+QLayout as_qlayout(const KLayout& l) { return QLayout{l.s_, l.b_, l.h_, 0}; }
+}  // namespace
 
 // Which form of each kernel a launch takes.  Alone on the GPU a launch wants the shortest latency:
 // with few workgroups the keys of a row (forward, dQ) or the queries of a key tile (dK/dV) are split
@@ -1715,7 +1815,7 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
                            int64_t do_sb, int64_t do_sg, int64_t do_sh, int64_t dq_ss, int64_t dq_sb,
                            int64_t dq_sg, int64_t dq_sh, int64_t dk_ss, int64_t dk_sb, int64_t dk_sh,
                            int64_t dv_ss, int64_t dv_sb, int64_t dv_sh, int flags, void* stream) {
-  if (flags & ~KR_ATTN_BESIDE_OTHER_STREAMS) return KR_EINVAL;
+  if (flags & ~(KR_ATTN_BESIDE_OTHER_STREAMS | KR_ATTN_GENERAL_KERNELS)) return KR_EINVAL;
   if (!dout || !q || !k || !v || !o || !lse || !dq || !dk || !dv || !workspace) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
@@ -1738,6 +1838,37 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   const KLayout kl{k_ss, k_sb, k_sh}, vl{v_ss, v_sb, v_sh}, dkl{dk_ss, dk_sb, dk_sh},
       dvl{dv_ss, dv_sb, dv_sh};
   float* delta = (float*)workspace;
+  if (!attn_fast_path(s, hd) && !(flags & KR_ATTN_GENERAL_KERNELS)) {
+    // padded into the MFMA kernels: dO, q, o, k, v and the log-sum-exp go in, dq, dk, dv come back
+    const int sp = attn_padded_len(s), per = nq / nkv;
+    const size_t qb = attn_padded_bytes(s, b, nq), kb = attn_padded_bytes(s, b, nkv);
+    char* w = (char*)workspace;
+    void *do_p = w, *q_p = w + qb, *o_p = w + 2 * qb, *dq_p = w + 3 * qb;
+    w += 4 * qb;
+    void *k_p = w, *v_p = w + kb, *dk_p = w + 2 * kb, *dv_p = w + 3 * kb;
+    w += 4 * kb;
+    float* lse_p = (float*)w;
+    w += attn_padded_stat_bytes(s, b, nq);
+    int rc2 = launch_pad(dout, do_p, s, b, nq, per, hd, dol, st);
+    if (rc2 == KR_OK) rc2 = launch_pad(q, q_p, s, b, nq, per, hd, ql, st);
+    if (rc2 == KR_OK) rc2 = launch_pad(o, o_p, s, b, nq, per, hd, ol, st);
+    if (rc2 == KR_OK) rc2 = launch_pad(k, k_p, s, b, nkv, 1, hd, as_qlayout(kl), st);
+    if (rc2 == KR_OK) rc2 = launch_pad(v, v_p, s, b, nkv, 1, hd, as_qlayout(vl), st);
+    // rows beyond s: exp2(x - 1.4e30) = 0 for every finite score, so they add nothing to dK and dV
+    if (rc2 == KR_OK) rc2 = launch_resize_rows(lse, lse_p, (int64_t)b * nq, s, sp, 1e30f, st);
+    if (rc2 != KR_OK) return rc2;
+    const QLayout pq = padded_qlayout(b, nq, per);
+    const KLayout pk = padded_klayout(b, nkv);
+    rc2 = attn_bwd_impl(do_p, q_p, k_p, v_p, o_p, lse_p, dq_p, dk_p, dv_p, w, sp, b, nq, nkv, HD, scale, pq.s_, pq.b_,
+                        pq.g_, pq.h_, pk.s_, pk.b_, pk.h_, pk.s_, pk.b_, pk.h_, pq.s_, pq.b_, pq.g_, pq.h_, pq.s_,
+                        pq.b_, pq.g_, pq.h_, pq.s_, pq.b_, pq.g_, pq.h_, pk.s_, pk.b_, pk.h_, pk.s_, pk.b_, pk.h_,
+                        flags, stream);
+    if (rc2 != KR_OK) return rc2;
+    rc2 = launch_unpad(dq_p, dq, s, b, nq, per, hd, dql, st);
+    if (rc2 == KR_OK) rc2 = launch_unpad(dk_p, dk, s, b, nkv, 1, hd, as_qlayout(dkl), st);
+    if (rc2 == KR_OK) rc2 = launch_unpad(dv_p, dv, s, b, nkv, 1, hd, as_qlayout(dvl), st);
+    return rc2;
+  }
   if (!attn_fast_path(s, hd)) {
     using namespace general;
     const dim3 qgrid((s + GT - 1) / GT, nq, b), kgrid((s + GT - 1) / GT, nkv, b);
@@ -1870,9 +2001,11 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
                            int b, int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb,
                            int64_t q_sg, int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh,
                            int64_t v_ss, int64_t v_sb, int64_t v_sh, int64_t o_ss, int64_t o_sb,
-                           int64_t o_sg, int64_t o_sh, int flags, void* stream) {
-  if (flags & ~KR_ATTN_BESIDE_OTHER_STREAMS) return KR_EINVAL;
+                           int64_t o_sg, int64_t o_sh, int flags, void* stream, void* workspace = nullptr,
+                           size_t workspace_bytes = 0) {
+  if (flags & ~(KR_ATTN_BESIDE_OTHER_STREAMS | KR_ATTN_GENERAL_KERNELS)) return KR_EINVAL;
   if (!q || !k || !v || !o || !lse) return KR_EINVAL;
+  if (workspace && !kr_aligned16(workspace)) return KR_EINVAL;
   const int rc = check_attn_common(s, b, nq, nkv, hd);
   if (rc != KR_OK) return rc;
   if (!kr_aligned16(q) || !kr_aligned16(k) || !kr_aligned16(v) || !kr_aligned16(o)) return KR_EINVAL;
@@ -1883,6 +2016,30 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
     const int64_t seq[] = {q_ss, k_ss, v_ss, o_ss};
     if (!attn_strides_ok(seq, {q_sb, q_sg, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sg, o_sh}))
       return KR_EUNSUPPORTED;
+  }
+  if (!attn_fast_path(s, hd) && !(flags & KR_ATTN_GENERAL_KERNELS) && workspace != nullptr &&
+      workspace_bytes >= kr_attn_fwd_workspace_bytes(s, b, nq, nkv, hd)) {
+    // padded into the MFMA kernels
+    hipStream_t st = (hipStream_t)stream;
+    const int sp = attn_padded_len(s), per = nq / nkv;
+    const size_t qb = attn_padded_bytes(s, b, nq), kb = attn_padded_bytes(s, b, nkv);
+    char* w = (char*)workspace;
+    void *q_p = w, *o_p = w + qb, *k_p = w + 2 * qb, *v_p = w + 2 * qb + kb;
+    float* lse_p = (float*)(w + 2 * qb + 2 * kb);
+    const QLayout ql{q_ss, q_sb, q_sg, q_sh}, ol{o_ss, o_sb, o_sg, o_sh};
+    const KLayout kl{k_ss, k_sb, k_sh}, vl{v_ss, v_sb, v_sh};
+    int rc2 = launch_pad(q, q_p, s, b, nq, per, hd, ql, st);
+    if (rc2 == KR_OK) rc2 = launch_pad(k, k_p, s, b, nkv, 1, hd, as_qlayout(kl), st);
+    if (rc2 == KR_OK) rc2 = launch_pad(v, v_p, s, b, nkv, 1, hd, as_qlayout(vl), st);
+    if (rc2 != KR_OK) return rc2;
+    const QLayout pq = padded_qlayout(b, nq, per);
+    const KLayout pk = padded_klayout(b, nkv);
+    rc2 = attn_fwd_impl(q_p, k_p, v_p, o_p, lse_p, sp, b, nq, nkv, HD, scale, pq.s_, pq.b_, pq.g_, pq.h_, pk.s_, pk.b_,
+                        pk.h_, pk.s_, pk.b_, pk.h_, pq.s_, pq.b_, pq.g_, pq.h_, flags, stream);
+    if (rc2 != KR_OK) return rc2;
+    rc2 = launch_unpad(o_p, o, s, b, nq, per, hd, ol, st);
+    if (rc2 == KR_OK) rc2 = launch_resize_rows(lse_p, lse, (int64_t)b * nq, sp, s, 0.f, st);
+    return rc2;
   }
   if (!attn_fast_path(s, hd)) {
     using namespace general;
@@ -1936,4 +2093,16 @@ extern "C" int kr_attn_fwd_flags(const void* q, const void* k, const void* v, vo
                                  int64_t o_sb, int64_t o_sg, int64_t o_sh, int flags, void* stream) {
   return attn_fwd_impl(q, k, v, o, lse, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
                        v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, flags, stream);
+}
+
+// kr_attn_fwd_flags with a workspace of kr_attn_fwd_workspace_bytes(): a shape outside the MFMA kernels (head
+// dimension below 128, a sequence that is not whole 128-row tiles) is padded into them through the
+// workspace instead of taking the general kernels.  A shape they take as it is needs no workspace.
+extern "C" int kr_attn_fwd_ws(const void* q, const void* k, const void* v, void* o, float* lse, int s, int b,
+                              int nq, int nkv, int hd, float scale, int64_t q_ss, int64_t q_sb, int64_t q_sg,
+                              int64_t q_sh, int64_t k_ss, int64_t k_sb, int64_t k_sh, int64_t v_ss, int64_t v_sb,
+                              int64_t v_sh, int64_t o_ss, int64_t o_sb, int64_t o_sg, int64_t o_sh, int flags,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  return attn_fwd_impl(q, k, v, o, lse, s, b, nq, nkv, hd, scale, q_ss, q_sb, q_sg, q_sh, k_ss, k_sb, k_sh, v_ss,
+                       v_sb, v_sh, o_ss, o_sb, o_sg, o_sh, flags, stream, workspace, workspace_bytes);
 }

@@ -47,7 +47,14 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1
     assert lib.kr_gemm_bf16(0, 8, 8, 8, 16, 8, 16, 8, 18, 8, 0, None, 0, None) == -1   # misaligned C
     assert lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 136) == 0  # head dimensions above 128 are unsupported
-    assert lib.kr_attn_bwd_workspace_bytes(250, 1, 4, 2, 64) == 2 * 250 * 4 * 4   # general kernels: delta (+ spare)
+    # a shape padded into the MFMA kernels (256 rows, 128 channels): four query-sized and four key-sized bf16
+    # copies, the padded log-sum-exp, and the MFMA backward's own workspace at the padded shape
+    padded = 4 * 256 * 4 * 128 * 2 + 4 * 256 * 2 * 128 * 2 + 256 * 4 * 4
+    assert lib.kr_attn_bwd_workspace_bytes(250, 1, 4, 2, 64) == padded + lib.kr_attn_bwd_workspace_bytes(256, 1, 4, 2, 128)
+    assert lib.kr_attn_fwd_workspace_bytes(250, 1, 4, 2, 64) == 2 * 256 * 4 * 128 * 2 + 2 * 256 * 2 * 128 * 2 + 256 * 4 * 4
+    assert lib.kr_attn_fwd_workspace_bytes(256, 1, 4, 2, 128) == 0 and lib.kr_attn_fwd_workspace_bytes(256, 1, 4, 2, 136) == 0
+    assert lib.kr_attn_fwd_ws(16, 16, 16, 16, 16, 250, 1, 4, 2, 64, 0.125, *([64] * 14), 0x400, None, 0, None) == -1   # unknown flag
+    assert lib.kr_attn_fwd_ws(16, 16, 16, 16, 16, 250, 1, 4, 2, 64, 0.125, *([64] * 14), 0, 24, 1 << 30, None) == -1   # misaligned workspace
     # delta and the rescaled lse, plus fp32 dK/dV partials per query head when heads share KV heads ...
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 32, 128) == 2 * 4 * 32 * 4096 * 4
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 8, 128) == 2 * 4 * 32 * 4096 * 4 + 2 * 4 * 32 * 4096 * 128 * 4

@@ -412,26 +412,51 @@ def test_attention_when_the_row_maximum_keeps_moving(be, s, b, nq, nkv, kind):
 @pytest.mark.parametrize("s,b,nq,nkv,hd", [(100, 1, 1, 1, 128),    # ragged length at the fast kernels' head dimension
                                             (256, 2, 8, 8, 64),     # benchmark configuration 1: 8 heads of 64
                                             (77, 3, 6, 2, 64),      # ragged, grouped queries
-                                            (200, 1, 4, 1, 96), (1, 1, 1, 1, 64), (130, 2, 4, 2, 128), (33, 1, 2, 2, 8)])
-def test_attention_general_shapes(be, s, b, nq, nkv, hd):
-    """Head dimensions other than 128 and sequence lengths that are not whole 128-row tiles run through the
-    general kernels: same interface and layouts (fused QKV views, dense tensors), checked like the fast path."""
+                                            (200, 1, 4, 1, 96), (1, 1, 1, 1, 64), (130, 2, 4, 2, 128), (33, 1, 2, 2, 8),
+                                            (1000, 2, 8, 2, 128),   # a ragged length at a training width
+                                            (640, 2, 8, 8, 64)])    # whole tiles, half the head dimension
+@pytest.mark.parametrize("general", [False, True])
+def test_attention_general_shapes(be, s, b, nq, nkv, hd, general):
+    """Head dimensions other than 128 and sequence lengths that are not whole 128-row tiles: padded into the MFMA
+    kernels through the workspace (``general=False``, what the engine runs) or on the general fp32 kernels — same
+    interface and layouts (fused QKV views, dense tensors), checked like the fast path."""
     _, q, k, v = _grouped(s, b, nq, nkv, hd, seed=100)
     do = rnd(s, b, nq, hd, seed=101)
     scale = hd ** -0.5
-    o, lse = be.attn_fwd(q, k, v, scale)
+    attn_fwd = lambda *a: be.attn_fwd(*a, general_kernels=general)
+    attn_bwd = lambda *a: be.attn_bwd(*a, general_kernels=general)
+    o, lse = attn_fwd(q, k, v, scale)
     qf, kf, vf = (t.float().cpu().clone().requires_grad_(True) for t in (q.flatten(2, 3), k, v))
     ro, rlse = R.causal_gqa_attention(qf, kf, vf, return_lse=True)
     assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
     assert torch.equal(o[0], v[0].repeat_interleave(nq // nkv, dim=1))     # one visible key: o = v exactly
     ro.backward(do.float().cpu())
-    dq, dk, dv = be.attn_bwd(do, q, k, v, o, lse, scale)
+    dq, dk, dv = attn_bwd(do, q, k, v, o, lse, scale)
+    assert all(torch.isfinite(t.float()).all() for t in (o, dq, dk, dv))
     assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
-    again = be.attn_bwd(do, q, k, v, o, lse, scale)                         # fixed order of every sum: same bits
+    again = attn_bwd(do, q, k, v, o, lse, scale)                            # fixed order of every sum: same bits
     assert all(torch.equal(x, y) for x, y in zip(again, (dq, dk, dv)))
     qd = q.flatten(2, 3).contiguous()
-    od, lsed = be.attn_fwd(qd, k.contiguous(), v.contiguous(), scale)
+    od, lsed = attn_fwd(qd, k.contiguous(), v.contiguous(), scale)
     assert torch.equal(od, o) and torch.equal(lsed, lse)
+
+
+def test_attention_padded_into_the_mfma_kernels_equals_the_whole_tile_call(be):
+    """A ragged length is the whole-tile problem with rows taken away: queries below s see the same keys, so the
+    padded call must give the bits of the MFMA kernels on the next multiple of 128 restricted to the first s
+    rows (forward), and gradients that ignore the rows beyond s."""
+    s, sp, b, nq, nkv, hd = 300, 384, 2, 4, 2, 128
+    _, q, k, v = _grouped(sp, b, nq, nkv, hd, seed=110)
+    scale = hd ** -0.5
+    o_full, lse_full = be.attn_fwd(q, k, v, scale)
+    o, lse = be.attn_fwd(q[:s], k[:s], v[:s], scale)
+    assert torch.equal(o, o_full[:s]) and torch.equal(lse, lse_full[..., :s])
+    # backward: the whole-tile call with zero upstream gradient beyond s gives the same dq, dk, dv rows below s
+    do_full = rnd(sp, b, nq, hd, seed=111)
+    do_full[s:] = 0
+    dq_f, dk_f, dv_f = be.attn_bwd(do_full, q, k, v, o_full, lse_full, scale)
+    dq, dk, dv = be.attn_bwd(do_full[:s], q[:s], k[:s], v[:s], o, lse, scale)
+    assert torch.equal(dq, dq_f[:s]) and torch.equal(dk, dk_f[:s]) and torch.equal(dv, dv_f[:s])
 
 
 # ------------------------------------------------------------------ fused GEMM epilogues
