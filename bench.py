@@ -600,6 +600,45 @@ def attention_kernels(w, nnb, device, launches=20):
     return out
 
 
+def attention_padded_shapes(device):
+    """Attention shapes outside the MFMA kernels (a head dimension below 128, a sequence that is not whole
+    128-row tiles), forward and backward alone on the GPU both ways: padded into the MFMA kernels through the
+    workspace (what the engine runs) and on the general fp32 kernels.  Causal FLOPs as in attention_kernels."""
+    from kareus_amd.backend import get_backend
+
+    be = get_backend("hip")
+    out = []
+
+    def timed(fn, launches):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / launches
+
+    for s_len, b, nq, nkv, hd in [(1000, 4, 8, 2, 128), (4000, 4, 8, 2, 128), (4096, 2, 32, 8, 64), (2048, 4, 16, 16, 64)]:
+        per = nq // nkv
+        fused = torch.randn(s_len, b, nkv, per + 2, hd, device=device).bfloat16()   # the fused QKV layout
+        q, k, v = fused[:, :, :, :per], fused[:, :, :, per], fused[:, :, :, per + 1]
+        do = torch.randn(s_len, b, nq, hd, device=device).bfloat16()
+        scale, flops = hd ** -0.5, 2.0 * b * nq * s_len * s_len * hd
+        row = {"seq": s_len, "batch": b, "q_heads": nq, "kv_heads": nkv, "head_dim": hd}
+        for name, general in (("padded_into_mfma", False), ("general_kernels", True)):
+            o, lse = be.attn_fwd(q, k, v, scale, general_kernels=general)
+            n = 3 if general else 10
+            t_f = timed(lambda: be.attn_fwd(q, k, v, scale, general_kernels=general), n)
+            t_b = timed(lambda: be.attn_bwd(do, q, k, v, o, lse, scale, general_kernels=general), n)
+            row[name] = {"fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6, "fwd_TFLOPs": flops / t_f / 1e12,
+                         "bwd_TFLOPs": 2.5 * flops / t_b / 1e12}
+        out.append(row)
+    return out
+
+
 def cpu_baseline(w, budget_s=25.0):
     """The CPU oracle (fp32 PyTorch, autograd backward) on a bounded sample: same layer widths,
     one sequence of at most 1024 tokens, as many iterations as fit the time budget."""
@@ -841,6 +880,9 @@ def main():
                     help="run only a residual-add kernel of known size (calibrates FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--attention-kernels", action="store_true",
                     help="run only the attention forward/backward stand-alone (TFLOP/s against the MFMA peak)")
+    ap.add_argument("--attention-padded-shapes", action="store_true",
+                    help="run only: attention at head dimension 64 and ragged lengths, padded into the MFMA kernels "
+                         "and on the general kernels")
     ap.add_argument("--hbm-kernels", action="store_true",
                     help="run only the HBM-bound kernels stand-alone (achieved TB/s against 8 TB/s)")
     ap.add_argument("--with-library-matmul", action="store_true",
@@ -878,6 +920,9 @@ def main():
         return
     if args.attention_kernels:
         print(json.dumps({"attention_kernels": attention_kernels(w, w["nnb"], device)}))
+        return
+    if args.attention_padded_shapes:
+        print(json.dumps({"attention_padded_shapes": attention_padded_shapes(device)}))
         return
     if args.hbm_kernels:
         print(json.dumps({"hbm_kernels": hbm_kernels(w, w["nnb"], device)}))
