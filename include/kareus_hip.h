@@ -136,10 +136,13 @@ int kr_gemm_bf16_runs(int layout, int M, int N, int K,
  * be a multiple of 64 (KR_EUNSUPPORTED otherwise: the caller then accumulates pair by pair).  Tiling,
  * cuts of the contraction, workspace and `max_cus` as for layout NT of kr_gemm_bf16_fused on
  * K = nseg * k_seg (size the workspace with that K); flags: 0 or KR_GEMM_BESIDE_OTHER_STREAMS.
+ * The pieces of A may be in row runs, every piece alike (a_run_rows, a_run_ld as for kr_gemm_bf16_runs;
+ * 1 = plain matrices): the incoming gradient of a layer stack, cut into nanobatches of several sequences.
  * The fp32 sum runs over the pieces in the order given and is rounded to bf16 once.                  */
 #define KR_GEMM_MAX_SEGMENTS 8
 int kr_gemm_bf16_nt_segments(int M, int N, int k_seg, int nseg,
-                             const void* const* A, int64_t lda, const void* const* B, int64_t ldb,
+                             const void* const* A, int64_t lda, int a_run_rows, int64_t a_run_ld,
+                             const void* const* B, int64_t ldb,
                              void* C, int64_t ldc, int accumulate, int flags,
                              int max_cus, void* workspace, size_t workspace_bytes, void* stream);
 

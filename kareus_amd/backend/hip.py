@@ -36,7 +36,7 @@ _SIGNATURES = {
     "kr_gemm_bf16_runs": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p, _c_i64,
                                    _c_void_p, _c_i64, _c_int, _c_i64, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64,
                                    _c_void_p, _c_i64, _c_int, _c_void_p, _c_size_t, _c_void_p]),
-    "kr_gemm_bf16_nt_segments": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_void_p, _c_i64,
+    "kr_gemm_bf16_nt_segments": (_c_int, [_c_int, _c_int, _c_int, _c_int, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p, _c_i64,
                                           _c_void_p, _c_i64, _c_int, _c_int, _c_int, _c_void_p, _c_size_t, _c_void_p]),
     "kr_rmsnorm_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_float, _c_void_p]),
     "kr_rmsnorm_fwd_runs": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_i64, _c_int, _c_i64,
@@ -329,18 +329,19 @@ class HipBackend:
     MAX_WGRAD_SEGMENTS = 8   # KR_GEMM_MAX_SEGMENTS
 
     def wgrad_segments_ok(self, dys, xs) -> bool:
-        """Whether ``linear_wgrad_segments`` takes these operand pairs: plain matrices (one row stride, the
-        same in every pair), the same shapes, a multiple of 64 rows each, at most MAX_WGRAD_SEGMENTS pairs."""
+        """Whether ``linear_wgrad_segments`` takes these operand pairs: matrices of one shape and one row
+        stride in every pair (the ``dys`` may be nanobatch slices in row runs, all alike), a multiple of 64 rows
+        each, at most MAX_WGRAD_SEGMENTS pairs."""
         if not 1 <= len(dys) == len(xs) <= self.MAX_WGRAD_SEGMENTS:
             return False
         first = None
         for dy, x in zip(dys, xs):
             a, b = self._operand(dy), self._operand(x)
-            if a is None or b is None or a[2] > 1 or b[2] > 1 or a[0] != b[0] or a[0] % 64:
+            if a is None or b is None or b[2] > 1 or a[0] != b[0] or a[0] % 64:
                 return False
             if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or not dy.is_cuda or x.device != dy.device:
                 return False
-            key = (a[0], a[1], b[1], dy.shape[-1], x.shape[-1])
+            key = (a[0], a[1], a[2], a[3], b[1], dy.shape[-1], x.shape[-1])
             if first is None:
                 first = key
             elif key != first:
@@ -352,8 +353,8 @@ class HipBackend:
         """``sum_i dys[i]^T . xs[i]`` in one launch: the weight gradient over all nanobatches of a
         microbatch, each pair read where it lies (``wgrad_segments_ok`` says whether the pairs qualify)."""
         if not self.wgrad_segments_ok(dys, xs):
-            raise RuntimeError("linear_wgrad_segments: operand pairs must be plain matrices of one shape and row "
-                               "stride with a multiple of 64 rows each")
+            raise RuntimeError("linear_wgrad_segments: operand pairs must be matrices of one shape and row stride "
+                               "with a multiple of 64 rows each")
         nseg = len(dys)
         a0, b0 = self._operand(dys[0]), self._operand(xs[0])
         k_seg, m, n = a0[0], dys[0].shape[-1], xs[0].shape[-1]
@@ -379,7 +380,7 @@ class HipBackend:
         ptrs = ctypes.c_void_p * nseg
         a_ptrs = ptrs(*[t.data_ptr() for t in dys])
         b_ptrs = ptrs(*[t.data_ptr() for t in xs])
-        rc = self.lib.kr_gemm_bf16_nt_segments(m, n, k_seg, nseg, a_ptrs, a0[1], b_ptrs, b0[1], out.data_ptr(), c_op[1],
+        rc = self.lib.kr_gemm_bf16_nt_segments(m, n, k_seg, nseg, a_ptrs, a0[1], a0[2], a0[3], b_ptrs, b0[1], out.data_ptr(), c_op[1],
                                                int(accumulate), 0x100 if split_k is False else 0, int(max_cus),
                                                ws_ptr, ws_bytes, self._stream())
         self._check(rc, f"kr_gemm_bf16_nt_segments(M={m}, N={n}, k_seg={k_seg}, nseg={nseg})")

@@ -238,7 +238,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
                                                         const bf16* __restrict__ aux, int ld_aux,
                                                         bf16* __restrict__ out2, int ld_out2,
                                                         RowRuns runs_arg, Segments segs) {
-  static_assert(!SEG || (A_T && B_T && !RUNS), "operand pieces: layout NT, plain rows");
+  static_assert(!SEG || (A_T && B_T), "operand pieces: layout NT");
   // (without RUNS every run length reads as a compile-time 1: the branches below fold away)
   const RowRuns runs = RUNS ? runs_arg : RowRuns{0, 0, 0, 0, 0, 0};
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
@@ -281,6 +281,8 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   int m0, n0, nk, k_tail, kc = K, a_off = 0, b_off = 0, p_off = 0;
   const bf16 *seg_a = A, *seg_b = B;
   int seg_left = 0, seg_next = 0;
+  // elements from one K-step of A to the next (a transposed A in row runs: 64 rows are 64 / r runs)
+  const int a_step = A_T ? (runs.a_sh ? (BK >> runs.a_sh) * runs.a_outer : BK * lda) : BK;
   auto select_item = [&](int v) {
     const int split = v / ntiles;
     int tile_m, tile_n;
@@ -302,13 +304,12 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
     if constexpr (SEG) {
       // the request cursor goes to K-step k0 / 64 of the whole contraction
       const int g0 = k0 / BK, sg = g0 / segs.steps, within = g0 - sg * segs.steps;
-      seg_a = segs.a[sg] + (int64_t)within * (BK * lda);
+      seg_a = segs.a[sg] + (int64_t)within * a_step;
       seg_b = segs.b[sg] + (int64_t)within * (BK * ldb);
       seg_left = segs.steps - within;
       seg_next = sg + 1;
     }
   };
-  const int a_step = A_T ? (runs.a_sh ? (BK >> runs.a_sh) * runs.a_outer : BK * lda) : BK;
   // SEG: K-steps are requested strictly in order (A then B of a step), so the bases are a cursor that
   // seg_advance() moves on behind the requests of a step; `t` is not needed
   auto a_base = [&](int t) {
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
   };
   auto seg_advance = [&]() {
     if constexpr (SEG) {
-      seg_a += BK * lda;
+      seg_a += a_step;
       seg_b += BK * ldb;
       if (--seg_left == 0) {
         if (seg_next < segs.n) {
@@ -962,7 +963,10 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
   // gradient (A in runs); instances that contract operand pieces for the weight gradient (both forms)
   constexpr bool kRunsInstance = EPI == KR_GEMM_EPI_ADD || EPI == KR_GEMM_EPI_SWIGLU_BWD || (EPI == KR_GEMM_EPI_NONE && B_T);
   constexpr bool kSegsInstance = A_T && B_T && (EPI == KR_GEMM_EPI_NONE || EPI == KR_GEMM_EPI_TRANSPOSED_OUT);
-  if ((with_runs && !kRunsInstance) || (with_segs && (!kSegsInstance || with_runs))) return KR_EUNSUPPORTED;
+  // (pieces in row runs: the direct store form only, A in runs)
+  constexpr bool kSegsRunsInstance = kSegsInstance && EPI == KR_GEMM_EPI_NONE;
+  if ((with_runs && !kRunsInstance) || (with_segs && !kSegsInstance) || (with_segs && with_runs && !kSegsRunsInstance))
+    return KR_EUNSUPPORTED;
   GemmKernel fn = gemm_kernel<A_T, B_T, WN, EPI>;
   hipError_t attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI>>();
   if constexpr (kRunsInstance) {
@@ -972,9 +976,15 @@ int launch(const bf16* A, int64_t lda, const bf16* B, int64_t ldb, bf16* C, int6
     }
   }
   if constexpr (kSegsInstance) {
-    if (with_segs) {
+    if (with_segs && !with_runs) {
       fn = gemm_kernel<A_T, B_T, WN, EPI, false, true>;
       attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI, false, true>>();
+    }
+  }
+  if constexpr (kSegsRunsInstance) {
+    if (with_segs && with_runs) {
+      fn = gemm_kernel<A_T, B_T, WN, EPI, true, true>;
+      attr_status = raise_lds_limit<gemm_kernel<A_T, B_T, WN, EPI, true, true>>();
     }
   }
   if (attr_status != hipSuccess) return KR_ELAUNCH;
@@ -1050,7 +1060,9 @@ int gemm_dispatch(int layout, int M, int N, int K, const void* A, int64_t lda, c
   {
     const RowRuns& rr = fu.runs;
     const int shs[3] = {rr.a_sh, rr.c_sh, rr.x_sh}, outers[3] = {rr.a_outer, rr.c_outer, rr.x_outer};
-    const int64_t rows_of[3] = {layout == KR_GEMM_NT ? K : M, M, M};
+    // (A in pieces: offsets are taken from a piece's own base)
+    const int64_t a_rows_in_runs = fu.segs != nullptr ? (int64_t)fu.segs->steps * BK : (layout == KR_GEMM_NT ? K : M);
+    const int64_t rows_of[3] = {a_rows_in_runs, M, M};
     for (int i = 0; i < 3; ++i) {
       if (shs[i] == 0) continue;
       if (shs[i] < 0 || shs[i] > 4 || outers[i] <= 0) return KR_EINVAL;
@@ -1257,11 +1269,12 @@ extern "C" int kr_gemm_bf16_runs(int layout, int M, int N, int K, const void* A,
 // A weight gradient over the nanobatches of a microbatch in one launch: C[M, N] (+)= sum_i A_i^T . B_i with
 // A_i [k_seg, M] (row stride lda) and B_i [k_seg, N] (row stride ldb), i < nseg <= KR_GEMM_MAX_SEGMENTS, the
 // pieces anywhere in memory.  The same kernels as layout NT of kr_gemm_bf16 on K = nseg * k_seg, with the
-// operand base exchanged at every piece boundary; k_seg must be a multiple of 64.
+// operand base exchanged at every piece boundary; k_seg must be a multiple of 64.  The pieces of A may be in
+// row runs (a_run_rows, a_run_ld as in kr_gemm_bf16_runs; 1 = plain).
 extern "C" int kr_gemm_bf16_nt_segments(int M, int N, int k_seg, int nseg, const void* const* A, int64_t lda,
-                                        const void* const* B, int64_t ldb, void* C, int64_t ldc,
-                                        int accumulate, int flags, int max_cus, void* workspace,
-                                        size_t workspace_bytes, void* stream) {
+                                        int a_run_rows, int64_t a_run_ld, const void* const* B, int64_t ldb,
+                                        void* C, int64_t ldc, int accumulate, int flags, int max_cus,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
   if (!A || !B || nseg < 1 || nseg > MAX_SEGMENTS || k_seg <= 0) return KR_EINVAL;
   if (flags & ~KR_GEMM_BESIDE_OTHER_STREAMS) return KR_EINVAL;
   if (k_seg % BK) return KR_EUNSUPPORTED;
@@ -1278,6 +1291,16 @@ extern "C" int kr_gemm_bf16_nt_segments(int M, int N, int k_seg, int nseg, const
   fu.shared = (flags & KR_GEMM_BESIDE_OTHER_STREAMS) != 0;
   fu.max_cus = max_cus;
   fu.segs = &segs;
+  // the pieces of A in row runs (every piece alike): rows per run a power of two up to 16 that divides 64
+  if (a_run_rows < 1 || (a_run_rows & (a_run_rows - 1))) return KR_EINVAL;
+  if (a_run_rows > 16) return KR_EUNSUPPORTED;
+  if (a_run_rows > 1) {
+    if (a_run_ld <= 0 || a_run_ld >= (int64_t)1 << 31) return KR_EINVAL;
+    int sh = 0;
+    while ((1 << sh) < a_run_rows) ++sh;
+    fu.runs.a_sh = sh;
+    fu.runs.a_outer = (int)a_run_ld;
+  }
   return gemm_dispatch(KR_GEMM_NT, M, N, k_seg * nseg, A[0], lda, B[0], ldb, C, ldc, accumulate, workspace,
                        workspace_bytes, stream, fu);
 }

@@ -162,11 +162,7 @@ def test_layer_with_wide_nanobatches_equals_the_copying_run(monkeypatch, b, nnb)
 
     s, h = 256, 3072
     cfg = dict(hidden_size=h, num_attention_heads=3, num_query_groups=1, kv_channels=128, ffn_hidden_size=1024,
-               num_layers=2, num_nanobatches=nnb, backend="hip",
-               # one accumulating weight-gradient GEMM per nanobatch in both runs: the one GEMM over all
-               # nanobatches takes dense operand pieces only, so the two runs would sum the top layer's fc2
-               # gradient in different ways (that path has its own tests)
-               wgrad_over_all_nanobatches=False)
+               num_layers=2, num_nanobatches=nnb, backend="hip")
 
     def run():
         model = LayerStack(LayerConfig(**cfg), device=DEV, seed=1234)

@@ -31,14 +31,17 @@ def test_entry_point_rejects_bad_pieces_without_a_device():
     lib = hip.load_library()
     ptrs = (ctypes.c_void_p * 2)(4096, 8192)
 
-    def call(m=64, n=64, k_seg=64, nseg=2, a=ptrs, b=ptrs, flags=0):
-        return lib.kr_gemm_bf16_nt_segments(m, n, k_seg, nseg, a, 64, b, 64, 4096, 64, 0, flags, 0, None, 0, None)
+    def call(m=64, n=64, k_seg=64, nseg=2, a=ptrs, b=ptrs, flags=0, run_rows=1, run_ld=0):
+        return lib.kr_gemm_bf16_nt_segments(m, n, k_seg, nseg, a, 64, run_rows, run_ld, b, 64, 4096, 64, 0, flags, 0,
+                                            None, 0, None)
 
     assert call(nseg=0) == -1 and call(nseg=9) == -1 and call(k_seg=0) == -1
     assert call(a=None) == -1 and call(flags=2) == -1
     assert call(k_seg=96) == -2                                         # pieces are whole K-steps of 64 rows
     assert call(a=(ctypes.c_void_p * 2)(4096, 0)) == -1                  # a missing piece
     assert call(a=(ctypes.c_void_p * 2)(4096, 8200)) == -1               # not 16-byte aligned
+    assert call(run_rows=3, run_ld=512) == -1 and call(run_rows=32, run_ld=4096) == -2 and call(run_rows=2, run_ld=0) == -1
+    assert call(run_rows=2, run_ld=500) == -2                            # run starts a multiple of 8 elements apart
 
 
 def test_operand_pairs_on_the_host_are_turned_down():
@@ -117,6 +120,24 @@ def test_pieces_that_are_strided_views_in_any_order(be):
 
 
 @gpu
+@pytest.mark.parametrize("s,b,r,m,n", [(256, 8, 4, 768, 512), (64, 16, 8, 4096, 1024), (1024, 4, 2, 3072, 1024),
+                                       (128, 32, 16, 640, 384), (4096, 8, 4, 3072, 1024)])
+@pytest.mark.parametrize("split_k", [True, False])
+def test_pieces_in_row_runs_equal_dense_copies(be, s, b, r, m, n, split_k):
+    """The incoming gradient of a layer stack cut into nanobatches of r sequences: every piece of dy is a
+    [s, r, m] slice whose rows come in runs, read where it lies; bit-equal to the launch on dense copies."""
+    dy_all = _rnd(s, b, m, seed=3)
+    dys = [dy_all[:, lo:lo + r] for lo in range(0, b, r)][:8]
+    xs = [_rnd(s * r, n, seed=20 + i) for i in range(len(dys))]
+    assert be.rows_view(dys[0]).dim() == 3 and be.wgrad_segments_ok(dys, xs)
+    got = be.linear_wgrad_segments(dys, xs, split_k=split_k)
+    want = be.linear_wgrad_segments([d.reshape(-1, m).contiguous() for d in dys], xs, split_k=split_k)
+    assert torch.equal(got, want)
+    ref = torch.cat([d.reshape(-1, m) for d in dys]).float().t() @ torch.cat(xs).float()
+    assert (got.float() - ref).abs().max() <= TOL * ref.abs().max()
+
+
+@gpu
 def test_pairs_the_backend_turns_down(be):
     dys = [_rnd(128, 256, seed=i) for i in range(2)]
     xs = [_rnd(128, 512, seed=5 + i) for i in range(2)]
@@ -125,7 +146,9 @@ def test_pairs_the_backend_turns_down(be):
     assert not be.wgrad_segments_ok([d[:96] for d in dys], [x[:96] for x in xs])        # not whole K-steps
     assert not be.wgrad_segments_ok(dys * 5, xs * 5)                                    # more than eight pairs
     whole = _rnd(64, 8, 256, seed=9)
-    assert not be.wgrad_segments_ok([whole[:, 0:2], whole[:, 2:4]], xs)                 # rows in runs
+    assert be.wgrad_segments_ok([whole[:, 0:2], whole[:, 2:4]], xs)                     # rows in runs, both alike
+    assert not be.wgrad_segments_ok([whole[:, 0:2], dys[1]], xs)                        # ... one in runs, one dense
+    assert not be.wgrad_segments_ok([whole[:, 0:2], whole[:, 2:4]], [xs[0], whole[:, 4:6]])   # only dy may be in runs
     with pytest.raises(RuntimeError):
         be.linear_wgrad_segments([d[:96] for d in dys], [x[:96] for x in xs])
 
