@@ -73,6 +73,13 @@ class LayerConfig:
     # nanobatches, launched when the last nanobatch has delivered its operands (instead of one
     # accumulating GEMM per nanobatch); the nanobatches' operands stay alive until then
     wgrad_over_all_nanobatches: bool = True
+    # ... and those launches are issued at the end of the backward pass, behind every nanobatch's input
+    # gradients, instead of where the last nanobatch delivers its operands.  A launch in the middle puts one
+    # nanobatch's stream out of step with the others; with four nanobatches of one sequence, whose attention
+    # and out-projection kernels fill the device only beside each other, keeping them in step is worth 4 % of
+    # the step (8B shard), with two wide nanobatches the launches fill gaps where they are (3B shard: 2 % the
+    # other way).  None: at the end from four nanobatches on.
+    wgrad_launches_at_end: Optional[bool] = None
     # nanobatch outputs (and input gradients) are written into slices of one tensor by the ops
     # that produce them, so joining the nanobatches needs no concatenation
     join_nanobatches_in_place: bool = True

@@ -183,7 +183,9 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
         nanobatches is one GEMM over all their tokens: every nanobatch leaves its ``(dy, x)`` pair and an
         event in the sink, and the last one to get here launches the product of all pairs, in nanobatch
         order, on the stream of the nanobatch whose turn it is (the launches of a backward pass take the
-        streams in rotation, so no nanobatch's chain of input gradients waits behind all of them).
+        streams in rotation, so no nanobatch's chain of input gradients waits behind all of them) — or,
+        when the sink carries a ``pending`` list, leaves the launch there for the engine to issue at the end of
+        the backward pass, behind every nanobatch's input gradients.
         Otherwise the first nanobatch allocates the gradient and every later one adds its product into
         it inside its own GEMM, after waiting for the previous writer's event."""
         sink = getattr(ctx, "wgrad_sink", None)
@@ -204,31 +206,43 @@ class PartitionableLinear(BasicOperation, PartitionableOperator):
                 return None
             pairs.sort(key=lambda p: p[0])
             sink["pairs"] = None
+            pending = sink.get("pending")
             turn = sink.get("turn")
             if turn is None:
                 turn = [0]
-            target = pairs[turn[0] % n][4]
+            # launched at once, the launches of a backward pass take the nanobatch streams in rotation; put off
+            # to the end of the pass they all go to the first nanobatch's stream, one after the other
+            target = pairs[0 if pending is not None else turn[0] % n][4]
             turn[0] += 1
             dys, xs = [p[1] for p in pairs], [p[2] for p in pairs]
             with api.stream(target):
-                if target is not None:
-                    for _, _, _, ready, st in pairs:
-                        if ready is not None and st != target:
-                            target.wait_event(ready)
-                if be.wgrad_segments_ok(dys, xs):
-                    # the one launch is planned as a GEMM that has the device to itself (cuts of the contraction
-                    # where the output has few tiles): the products of the other nanobatches, which used to
-                    # fill the device beside each other, are inside it
-                    dw = be.linear_wgrad_segments(dys, xs, split_k=PartitionableLinear.wgrad_over_all_split_k)
-                else:
-                    dw = be.linear_wgrad(dys[0], xs[0], split_k=split_k)
-                    for d, x in zip(dys[1:], xs[1:]):
-                        be.linear_wgrad(d, x, out=dw, accumulate=True, split_k=split_k)
-                if target is not None:
-                    # the operands were allocated on their own nanobatch's stream
-                    for t in dys + xs:
-                        if t.is_cuda:
-                            t.record_stream(target)
+                dw = dys[0].new_empty((dys[0].shape[-1], xs[0].shape[-1]))
+
+            def launch():
+                with api.stream(target):
+                    if target is not None:
+                        for _, _, _, ready, st in pairs:
+                            if ready is not None and st != target:
+                                target.wait_event(ready)
+                    if be.wgrad_segments_ok(dys, xs):
+                        # planned as a GEMM that has the device to itself (cuts of the contraction where the
+                        # output has few tiles): the products of the other nanobatches, which used to fill the
+                        # device beside each other, are inside it
+                        be.linear_wgrad_segments(dys, xs, out=dw, split_k=PartitionableLinear.wgrad_over_all_split_k)
+                    else:
+                        be.linear_wgrad(dys[0], xs[0], out=dw, split_k=split_k)
+                        for d, x in zip(dys[1:], xs[1:]):
+                            be.linear_wgrad(d, x, out=dw, accumulate=True, split_k=split_k)
+                    if target is not None:
+                        # the operands were allocated on their own nanobatch's stream
+                        for t in dys + xs:
+                            if t.is_cuda:
+                                t.record_stream(target)
+
+            if pending is not None:
+                pending.append(launch)
+            else:
+                launch()
             return dw
         buf = sink.get("buf")
         if buf is None:

@@ -207,6 +207,7 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
         func_ctx.checkpoint_activations = checkpoint_activations
         func_ctx.fuse_wgrad_accumulation = bool(getattr(config, "fuse_wgrad_accumulation", False))
         func_ctx.wgrad_over_all_nanobatches = bool(getattr(config, "wgrad_over_all_nanobatches", True))
+        func_ctx.wgrad_launches_at_end = getattr(config, "wgrad_launches_at_end", None)
         func_ctx.join_in_place = in_place
 
         if checkpoint_activations:
@@ -261,16 +262,23 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             c.tensor_store = TensorStore()
             c.tensor_store.set(seed.bwd_grad_tid, g)
 
+        pending = None
         if func_ctx.fuse_wgrad_accumulation and n > 1:
             # one sink per layer operator, shared by that operator's contexts of all nanobatches
             sinks: Dict[int, dict] = {}
             # ("turn": a counter all sinks share, by which launches that serve all nanobatches take the
             # nanobatch streams in rotation)
             turn = [0]
+            at_end = func_ctx.wgrad_launches_at_end
+            if at_end is None:
+                at_end = n >= 4
+            # ("pending": where such launches are left to be issued behind the last partition of the pass)
+            pending = [] if (at_end and func_ctx.wgrad_over_all_nanobatches) else None
             for c in ctxs:
                 for op_id, op_ctx in c.op_contexts.items():
                     op_ctx.wgrad_sink = sinks.setdefault(
-                        op_id, {"n": n, "turn": turn, "defer": func_ctx.wgrad_over_all_nanobatches})
+                        op_id, {"n": n, "turn": turn, "defer": func_ctx.wgrad_over_all_nanobatches,
+                                "pending": pending})
                     op_ctx.nanobatch_index = c.batch_idx
 
         if func_ctx.join_in_place:
@@ -289,6 +297,8 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             i = part.nano_batch_idx
             got = part.execute(ctx=ctxs[i], pre_ctx=ctxs[(i - 1) % n], protected_tensor_ids=protected)
             per_nb[i].update(got)
+        for launch in pending or ():
+            launch()
         _join(streams)
 
         grad_tid = func_ctx.backward_tensor_graph.get_output_channel(seed.bwd_output_channel)

@@ -85,15 +85,16 @@ def test_weight_gradient_over_all_nanobatches_equals_per_nanobatch_accumulation(
     accumulating product per nanobatch: the same gradient, and the oracle's."""
     x, go, ref = _oracle(layers=2, s=128, b=4)
     grads = {}
-    for whole in (True, False):
+    for whole, at_end in ((True, True), (True, False), (False, None)):
         cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=4, params_dtype=torch.float32,
                           backend="eager", checkpoint_activations=recompute,
-                          wgrad_over_all_nanobatches=whole)
+                          wgrad_over_all_nanobatches=whole, wgrad_launches_at_end=at_end)
         model = LayerStack(cfg, seed=1234)
         _check(model, x, go, ref)
-        grads[whole] = [p.grad.clone() for p in model.parameters()]
-    for a, b in zip(grads[True], grads[False]):
-        assert (a - b).abs().max() <= 1e-5 * b.abs().max()
+        grads[whole, at_end] = [p.grad.clone() for p in model.parameters()]
+    for a, b, c in zip(grads[True, True], grads[True, False], grads[False, None]):
+        assert torch.equal(a, b)                         # when the launch is issued does not change what it computes
+        assert (a - c).abs().max() <= 1e-5 * c.abs().max()
 
 
 @pytest.mark.parametrize("b,nnb", [(4, 4), (8, 4), (4, 2)])

@@ -153,12 +153,12 @@ def test_pairs_the_backend_turns_down(be):
         be.linear_wgrad_segments([d[:96] for d in dys], [x[:96] for x in xs])
 
 
-def _layer_grads(whole, nnb, b, s=256):
+def _layer_grads(whole, nnb, b, s=256, at_end=None):
     from kareus_amd import LayerConfig, LayerStack
 
     cfg = LayerConfig(hidden_size=1024, num_attention_heads=8, num_query_groups=2, kv_channels=128,
                       ffn_hidden_size=1792, num_layers=2, num_nanobatches=nnb, backend="hip",
-                      wgrad_over_all_nanobatches=whole)
+                      wgrad_over_all_nanobatches=whole, wgrad_launches_at_end=at_end)
     model = LayerStack(cfg, device=DEV, seed=1234)
     g = torch.Generator().manual_seed(7)
     x = torch.randn(s, b, 1024, generator=g).to(DEV, torch.bfloat16).requires_grad_(True)
@@ -183,8 +183,11 @@ def test_layer_step_with_one_weight_gradient_per_layer(nnb, b):
     """Two layers, nanobatches on their own streams: outputs and input gradients do not depend on how the
     weight gradients are summed (bit-equal); the weight gradients agree with the per-nanobatch
     accumulation within bf16 rounding and are the same on every pass."""
-    y_w, dx_w, g_w = _layer_grads(True, nnb, b)
+    y_w, dx_w, g_w = _layer_grads(True, nnb, b, at_end=False)
     y_p, dx_p, g_p = _layer_grads(False, nnb, b)
     assert torch.equal(y_w, y_p) and torch.equal(dx_w, dx_p)
     for a, c in zip(g_w, g_p):
         assert (a.float() - c.float()).abs().max() <= TOL * c.float().abs().max()
+    # issued at the end of the backward pass instead of where the last nanobatch delivers: the same launches
+    y_e, dx_e, g_e = _layer_grads(True, nnb, b, at_end=True)
+    assert torch.equal(y_e, y_w) and torch.equal(dx_e, dx_w) and all(torch.equal(a, c) for a, c in zip(g_e, g_w))
