@@ -179,6 +179,60 @@ def partition_times(stepper, iters=3):
     return {k: v / iters for k, v in timer.totals().items()}
 
 
+def partition_timeline(w, device, steps=24, wgrad_launches_at_end=None):
+    """When each partition of each nanobatch starts and ends on the device inside one step in steady state:
+    an event pair around every partition on its own stream (no profiler: the host runs at its own speed),
+    times in microseconds from the start of the step's first partition.  ``step_us`` is the average over the
+    run, ``partitions_end_us`` the end of the last partition: what follows are the weight gradients put off
+    to the end of the backward pass."""
+    from kareus_amd.partitions.partition_base import PartitionBase
+
+    gen = torch.Generator().manual_seed(42)
+    x = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16).requires_grad_(True)
+    go = torch.randn(w["s"], w["b"], w["h"], generator=gen).to(device, torch.bfloat16)
+    model = make_model(w, w["nnb"], device)
+    model.config.wgrad_launches_at_end = wgrad_launches_at_end
+    st = Stepper(model, x, go)
+    st.run(5)
+    preheat(st, 2.0)
+
+    class Marks:
+        def __init__(self):
+            self.rows, self.step, self.begun = [], -1, None
+
+        def begin(self, part):
+            self.begun = torch.cuda.Event(enable_timing=True)
+            self.begun.record()
+
+        def end(self, part):
+            done = torch.cuda.Event(enable_timing=True)
+            done.record()
+            kind = "fwd" if "Forward" in type(part).__name__ else "bwd"
+            self.rows.append((self.step, kind, part.partition_key or "trail", part.nano_batch_idx, self.begun, done))
+
+    marks = Marks()
+    PartitionBase.timer = marks
+    try:
+        first = torch.cuda.Event(enable_timing=True)
+        first.record()
+        for i in range(steps):
+            marks.step = i
+            st.step()
+        last = torch.cuda.Event(enable_timing=True)
+        last.record()
+        torch.cuda.synchronize()
+    finally:
+        PartitionBase.timer = None
+    shown = steps - 3
+    rows = [(first.elapsed_time(b) * 1e3, first.elapsed_time(e) * 1e3, kind, key, nb)
+            for (i, kind, key, nb, b, e) in marks.rows if i == shown]
+    t0 = min(r[0] for r in rows)
+    return {"workload_nanobatches": w["nnb"], "step_us": first.elapsed_time(last) * 1e3 / steps,
+            "partitions_end_us": max(r[1] for r in rows) - t0,
+            "partitions": [{"nanobatch": nb, "pass": kind, "partition": key, "start_us": round(a - t0, 1),
+                            "end_us": round(b - t0, 1)} for a, b, kind, key, nb in sorted(rows)]}
+
+
 # HBM-side bytes per launch from hardware counters (FETCH_SIZE and WRITE_SIZE of two profiler
 # runs of `bench.py --roofline-only`, each scaled by what the same counter reads for
 # `bench.py --copy-calibration`).  Keyed by (layout, M, N, K); a shape that was not profiled
@@ -730,6 +784,9 @@ def overlap_bound(w, device, rounds=4, steps=8):
         completely behind the other nanobatches' MFMA-bound kernels.  Timing only — results are wrong.
     (2) The same for the one-nanobatch step (its floor without those kernels).
     (3) The nanobatched step with a busy wait added to the host's work per step: GPU time against host time.
+    (5) The nanobatched step with the weight gradients as one launch per layer where the last nanobatch
+        delivers its operands (instead of at the end of the backward pass), and as one accumulating launch per
+        nanobatch (the reference's way).
     (4) The nanobatched step with the attention kernels in the forms they take when a launch has the device
         to itself (keys split between the halves of a workgroup at one sequence) instead of the forms the engine
         picks beside other streams (no split: fewer workgroups, less compute-unit time).
@@ -744,16 +801,24 @@ def overlap_bound(w, device, rounds=4, steps=8):
     unsplit = Stepper(make_model(w, w["nnb"], device), x, go)
     for layer in unsplit.model.layers:
         layer.core_attention.beside_other_streams = False
-    for st in (nano, serial, unsplit):
+    in_place = Stepper(make_model(w, w["nnb"], device), x, go)     # weight-gradient launches where the last nanobatch delivers
+    in_place.model.config.wgrad_launches_at_end = False
+    per_nb = Stepper(make_model(w, w["nnb"], device), x, go)       # one accumulating weight gradient per nanobatch
+    per_nb.model.config.wgrad_over_all_nanobatches = False
+    for st in (nano, serial, unsplit, in_place, per_nb):
         st.run(2)
     preheat(nano, 2.0)
     lib = get_backend("hip").lib
     hbm = ["kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rmsnorm_bwd_add", "kr_rmsnorm_dgamma", "kr_rope"]
     samples = {k: [] for k in ("nanobatched", "one nanobatch", "nanobatched, HBM-bound launches suppressed",
                                "one nanobatch, HBM-bound launches suppressed",
-                               "nanobatched, attention kernels in the forms they take alone on the device")}
+                               "nanobatched, attention kernels in the forms they take alone on the device",
+                               "nanobatched, weight gradients launched where the last nanobatch delivers its operands",
+                               "nanobatched, one accumulating weight gradient per nanobatch")}
     for _ in range(rounds):
         samples["nanobatched"].append(nano.timed(steps))
+        samples["nanobatched, weight gradients launched where the last nanobatch delivers its operands"].append(in_place.timed(steps))
+        samples["nanobatched, one accumulating weight gradient per nanobatch"].append(per_nb.timed(steps))
         samples["nanobatched, attention kernels in the forms they take alone on the device"].append(unsplit.timed(steps))
         samples["one nanobatch"].append(serial.timed(steps))
         with _SuppressedLaunches(lib, hbm):
@@ -894,6 +959,10 @@ def main():
     ap.add_argument("--overlap-bound", action="store_true",
                     help="run only: the nanobatched step with its HBM-bound launches suppressed (the best any "
                          "overlap could do) and with extra host work per step")
+    ap.add_argument("--partition-timeline", action="store_true",
+                    help="run only: start and end of every partition of every nanobatch inside one step (events, "
+                         "no profiler), with the weight-gradient launches where the engine puts them and where the "
+                         "last nanobatch delivers its operands")
     ap.add_argument("--power-trace", action="store_true",
                     help="run only the power / shader-clock trace over kernels and layer steps")
     args = ap.parse_args()
@@ -920,6 +989,11 @@ def main():
         return
     if args.attention_kernels:
         print(json.dumps({"attention_kernels": attention_kernels(w, w["nnb"], device)}))
+        return
+    if args.partition_timeline:
+        print(json.dumps({"partition_timeline": {
+            "as the engine runs it": partition_timeline(w, device),
+            "weight gradients launched where the last nanobatch delivers": partition_timeline(w, device, wgrad_launches_at_end=False)}}))
         return
     if args.attention_padded_shapes:
         print(json.dumps({"attention_padded_shapes": attention_padded_shapes(device)}))
