@@ -295,7 +295,8 @@ int kr_attn_fwd_flags(const void* q, const void* k, const void* v, void* o, floa
                       int64_t o_stride_s, int64_t o_stride_b, int64_t o_stride_g, int64_t o_stride_h,
                       int flags, void* stream);
 /* kr_attn_fwd_flags with a workspace of kr_attn_fwd_workspace_bytes() bytes (0 for a shape the MFMA
- * kernels take as it lies; workspace may then be NULL): the call the reference's
+ * kernels take as it lies; workspace may then be NULL; a workspace that is too small for a shape that
+ * needs one is KR_EINVAL, none at all selects the general kernels): the call the reference's
  * flash_attn_gpu.fwd (kareus/flash_attn/flash_attn_interface.py:66-80) maps to for any head
  * dimension and sequence length it accepts.                                                      */
 size_t kr_attn_fwd_workspace_bytes(int s, int b, int nq, int nkv, int hd);

@@ -2017,8 +2017,11 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, void* o, f
     if (!attn_strides_ok(seq, {q_sb, q_sg, q_sh, k_sb, k_sh, v_sb, v_sh, o_sb, o_sg, o_sh}))
       return KR_EUNSUPPORTED;
   }
+  // (a workspace that is there but too small is a caller's mistake, not a request for the general kernels)
   if (!attn_fast_path(s, hd) && !(flags & KR_ATTN_GENERAL_KERNELS) && workspace != nullptr &&
-      workspace_bytes >= kr_attn_fwd_workspace_bytes(s, b, nq, nkv, hd)) {
+      workspace_bytes < kr_attn_fwd_workspace_bytes(s, b, nq, nkv, hd))
+    return KR_EINVAL;
+  if (!attn_fast_path(s, hd) && !(flags & KR_ATTN_GENERAL_KERNELS) && workspace != nullptr) {
     // padded into the MFMA kernels
     hipStream_t st = (hipStream_t)stream;
     const int sp = attn_padded_len(s), per = nq / nkv;

@@ -55,6 +55,7 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_attn_fwd_workspace_bytes(256, 1, 4, 2, 128) == 0 and lib.kr_attn_fwd_workspace_bytes(256, 1, 4, 2, 136) == 0
     assert lib.kr_attn_fwd_ws(16, 16, 16, 16, 16, 250, 1, 4, 2, 64, 0.125, *([64] * 14), 0x400, None, 0, None) == -1   # unknown flag
     assert lib.kr_attn_fwd_ws(16, 16, 16, 16, 16, 250, 1, 4, 2, 64, 0.125, *([64] * 14), 0, 24, 1 << 30, None) == -1   # misaligned workspace
+    assert lib.kr_attn_fwd_ws(16, 16, 16, 16, 16, 250, 1, 4, 2, 64, 0.125, *([64] * 14), 0, 32, 1024, None) == -1      # workspace too small
     # delta and the rescaled lse, plus fp32 dK/dV partials per query head when heads share KV heads ...
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 32, 128) == 2 * 4 * 32 * 4096 * 4
     assert lib.kr_attn_bwd_workspace_bytes(4096, 4, 32, 8, 128) == 2 * 4 * 32 * 4096 * 4 + 2 * 4 * 32 * 4096 * 128 * 4
