@@ -153,12 +153,13 @@ def test_pairs_the_backend_turns_down(be):
         be.linear_wgrad_segments([d[:96] for d in dys], [x[:96] for x in xs])
 
 
-def _layer_grads(whole, nnb, b, s=256, at_end=None):
+def _layer_grads(whole, nnb, b, s=256, at_end=None, recompute=False):
     from kareus_amd import LayerConfig, LayerStack
 
     cfg = LayerConfig(hidden_size=1024, num_attention_heads=8, num_query_groups=2, kv_channels=128,
                       ffn_hidden_size=1792, num_layers=2, num_nanobatches=nnb, backend="hip",
-                      wgrad_over_all_nanobatches=whole, wgrad_launches_at_end=at_end)
+                      wgrad_over_all_nanobatches=whole, wgrad_launches_at_end=at_end,
+                      checkpoint_activations=recompute)
     model = LayerStack(cfg, device=DEV, seed=1234)
     g = torch.Generator().manual_seed(7)
     x = torch.randn(s, b, 1024, generator=g).to(DEV, torch.bfloat16).requires_grad_(True)
@@ -191,3 +192,13 @@ def test_layer_step_with_one_weight_gradient_per_layer(nnb, b):
     # issued at the end of the backward pass instead of where the last nanobatch delivers: the same launches
     y_e, dx_e, g_e = _layer_grads(True, nnb, b, at_end=True)
     assert torch.equal(y_e, y_w) and torch.equal(dx_e, dx_w) and all(torch.equal(a, c) for a, c in zip(g_e, g_w))
+
+
+@gpu
+def test_recomputed_activations_feed_the_same_weight_gradient():
+    """Activation recompute rebuilds the saved inputs inside the backward pass; the one weight-gradient launch
+    per layer, issued at the end of that pass, must read them as it reads the saved ones."""
+    kept = _layer_grads(True, 4, 4)
+    again = _layer_grads(True, 4, 4, recompute=True)
+    assert torch.equal(kept[0], again[0]) and torch.equal(kept[1], again[1])
+    assert all(torch.equal(a, c) for a, c in zip(kept[2], again[2]))
