@@ -783,6 +783,8 @@ def overlap_bound(w, device, rounds=4, steps=8):
         the norm weight-gradient reduction) suppressed: the time it would take if every one of them hid
         completely behind the other nanobatches' MFMA-bound kernels.  Timing only — results are wrong.
     (2) The same for the one-nanobatch step (its floor without those kernels).
+    (6) Both steps with only the rotary embedding's launches suppressed: the most that folding the rotation
+        into the neighbouring kernels (qkv GEMM epilogue, attention backward stores) could win.
     (3) The nanobatched step with a busy wait added to the host's work per step: GPU time against host time.
     (5) The nanobatched step with the weight gradients as one launch per layer where the last nanobatch
         delivers its operands (instead of at the end of the backward pass), and as one accumulating launch per
@@ -812,6 +814,8 @@ def overlap_bound(w, device, rounds=4, steps=8):
     hbm = ["kr_rmsnorm_fwd", "kr_rmsnorm_bwd", "kr_rmsnorm_bwd_add", "kr_rmsnorm_dgamma", "kr_rope"]
     samples = {k: [] for k in ("nanobatched", "one nanobatch", "nanobatched, HBM-bound launches suppressed",
                                "one nanobatch, HBM-bound launches suppressed",
+                               "nanobatched, rotary embedding launches suppressed",
+                               "one nanobatch, rotary embedding launches suppressed",
                                "nanobatched, attention kernels in the forms they take alone on the device",
                                "nanobatched, weight gradients launched where the last nanobatch delivers its operands",
                                "nanobatched, one accumulating weight gradient per nanobatch")}
@@ -824,6 +828,9 @@ def overlap_bound(w, device, rounds=4, steps=8):
         with _SuppressedLaunches(lib, hbm):
             samples["nanobatched, HBM-bound launches suppressed"].append(nano.timed(steps))
             samples["one nanobatch, HBM-bound launches suppressed"].append(serial.timed(steps))
+        with _SuppressedLaunches(lib, ["kr_rope"]):
+            samples["nanobatched, rotary embedding launches suppressed"].append(nano.timed(steps))
+            samples["one nanobatch, rotary embedding launches suppressed"].append(serial.timed(steps))
     out = {"ms_per_step": {k: sorted(v)[len(v) // 2] * 1e3 for k, v in samples.items()}}
 
     def spin(us):
