@@ -1232,11 +1232,9 @@ __global__ __launch_bounds__(256) void attn_group_reduce_kernel(
 // HALVES = 2: as in the forward kernel, two halves of an 8-wave workgroup own the same 128
 // queries and walk the even / odd key tiles; half 1's dQ partial is added to half 0's through
 // LDS at the end.  Chosen by the host when there are few workgroups.
-// SHARED (with two halves): the halves own different queries (rows 0..127 and 128..255 of a
-// 256-query tile) and walk the same key tiles, which all eight waves bring in together — half
-// the K / V traffic and half the workgroups of the split form, and nothing to merge.  Chosen
-// when there is such a tile for every compute unit.
-template <int HALVES, bool SHARED>
+// When there is a 256-query tile for every compute unit (or other streams run beside the launch)
+// the host takes attn_bwd_dq_w64_kernel below instead.
+template <int HALVES>
 __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
     const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
@@ -1248,23 +1246,17 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
   const int half = HALVES == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
   const int tid = threadIdx.x & 255, lane = tid & 63, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  static_assert(!SHARED || HALVES == 2, "shared tiles need two halves");
-  constexpr int ROWS = SHARED ? 2 * BQ : BQ;  // queries per workgroup
+  constexpr int ROWS = BQ;  // queries per workgroup
   const int nqt = s / ROWS;
   const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
-  int qt, pair;
-  if (SHARED) {
-    longest_first(lid, nqt, gridDim.x / nqt, qt, pair);
-  } else {
-    qt = nqt - 1 - (lid % nqt);
-    pair = lid / nqt;
-  }
+  const int qt = nqt - 1 - (lid % nqt);
+  const int pair = lid / nqt;
   const int head = pair % nq;
   const int bi = pair / nq;
   const int per = nq / nkv;
   const int kvh = head / per;
   const int q0 = qt * ROWS;
-  const int qw0 = q0 + (SHARED ? half * BQ : 0) + wave * 32;
+  const int qw0 = q0 + wave * 32;
   const int qrow = qw0 + (lane & 31);
 
   const bf16* qp = q + ql.at(bi, head, per) + (int64_t)qrow * ql.s_;
@@ -1288,16 +1280,15 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     for (int e = 0; e < 16; ++e) dqacc[dt][e] = 0.f;
 
   // key tiles per half (the tile count is even), or all tiles up to the workgroup's last row
-  const int ntiles = SHARED ? (q0 + ROWS) / BKV : (q0 + BQ) / (HALVES * BKV);
-  auto key_of = [&](int j) { return SHARED ? j * BKV : (HALVES * j + half) * BKV; };
+  const int ntiles = (q0 + BQ) / (HALVES * BKV);
+  auto key_of = [&](int j) { return (HALVES * j + half) * BKV; };
   // K and V tiles go straight from global memory into two LDS stages: this half's own, or with
   // shared tiles the workgroup's, half 0 bringing in the K tile and half 1 the V tile
-  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + (SHARED ? 0 : half * 2 * STAGE);
+  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem + half * 2 * STAGE;
   auto stage_request = [&](int j, int buf) {
     const int key0 = key_of(j);
-    if (!SHARED || half == 0) bt_request(kb + (int64_t)key0 * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
-    if (!SHARED || half == 1)
-      bt_request(vb + (int64_t)key0 * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
+    bt_request(kb + (int64_t)key0 * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
+    bt_request(vb + (int64_t)key0 * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
   };
   stage_request(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
@@ -1360,7 +1351,7 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
     __syncthreads();
   }
 
-  if (HALVES == 2 && !SHARED) {  // half 1 -> LDS -> half 0 ([value][wave][lane]; the staging areas are free)
+  if (HALVES == 2) {  // half 1 -> LDS -> half 0 ([value][wave][lane]; the staging areas are free)
     float* xch = reinterpret_cast<float*>(smem);
     const int slot = wave * 64 + lane;
     if (half == 1) {
@@ -1379,16 +1370,276 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
 
   // output transposition through LDS (behind the 64 KiB hand-over buffer when there are two halves)
   RowStage rs;
-  rs.init(reinterpret_cast<char*>(smem) + (SHARED ? half * 16384 : HALVES == 2 ? 64 * 1024 : 0) + wave * 4096, lane);
+  rs.init(reinterpret_cast<char*>(smem) + (HALVES == 2 ? 64 * 1024 : 0) + wave * 4096, lane);
   store_rows_bf16(rs, dqacc, scale, dq + dql.at(bi, head, per) + (int64_t)qw0 * dql.s_, dql.s_);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ with ONE wave per SIMD.  A wave owns 64 query rows (two blocks of 32) and all 512 registers of
+// its lanes, so that every K / V fragment it reads from LDS feeds two MFMAs — a wave cannot fetch a
+// 1 KB fragment faster than an MFMA takes, which is what holds the two-waves-per-SIMD kernels at
+// half of the matrix pipe.  With a single instruction stream per SIMD nothing else would fill the
+// pipe while the wave does its vector work, so the loop is software-pipelined by hand: behind each of
+// the 32 score MFMAs (S^T, dP^T) of the NEXT 32 keys sits the exponential, multiply-add, subtraction,
+// multiplication and rounding of one score per lane of THIS step, then come this step's 16 dQ MFMAs.
+//
+// The score MFMAs are inline assembly because their register file has to be chosen: a kernel with more
+// than 256 registers gets its MFMA results in the accumulation registers, and every score would
+// then pass through a copy before a vector instruction can read it.  Written by hand they land in
+// ordinary VGPRs (with most Q / dO fragments in the accumulation registers, which the MFMA reads
+// directly); the dQ MFMAs are ordinary builtins and keep dQ in the accumulation registers.  The
+// compiler does not see an MFMA in the assembly, so the waits it would insert between such an
+// instruction and a reader of its result are provided by construction:
+//   * a score accumulator is read by vector instructions one step after the MFMAs that wrote it,
+//     with that step's 16 dQ MFMAs in between (before the loop: explicit s_nop);
+//   * accumulators start from the instruction's zero operand, never from a vector write, and a
+//     result that is not also the addend is an early-clobber operand.
+// tests/test_attention_asm.py checks the compiled kernel for any reader that comes too early.
+// Fragments come from LDS through ordinary loads, whose waits the compiler does insert.
+// ---------------------------------------------------------------------------------------------
+struct DqScores {
+  f32x16 s[2], dp[2];  // per 32-query block: S^T and dP^T of 32 keys
+};
+
+// c = a . b / c += a . b with c in VGPRs; b in the accumulation registers or in VGPRs.  A result that
+// is not also the addend must not share registers with the operands (early clobber): the
+// instruction writes while it still reads.
+__device__ __forceinline__ void mfma_set_v(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma_acc_v(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma_set_vv(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_acc_vv(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+
+// c = a . b + c0 with c and c0 in VGPRs (c0 is kept)
+__device__ __forceinline__ void mfma_from_v(f32x16& c, bf16x8 a, bf16x8 b, const f32x16& c0) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "a"(b), "v"(c0));
+}
+__device__ __forceinline__ void mfma_from_vv(f32x16& c, bf16x8 a, bf16x8 b, const f32x16& c0) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "v"(b), "v"(c0));
+}
+
+// MFMA m (0..3) of contraction step kk: S^T of block 0, block 1, dP^T of block 0, block 1.  dP^T
+// starts from -delta of the lane's row (sixteen copies per block, set up once), which takes the
+// subtraction out of every score's vector work.
+__device__ __forceinline__ void dq_score_mfma(DqScores& x, int kk, int m, bf16x8 kf, bf16x8 vf,
+                                              const bf16x8 (&qf)[2][HD / 16], const bf16x8 (&dof)[2][HD / 16],
+                                              const f32x16 (&neg_delta)[2]) {
+  if (kk == 0) {
+    if (m == 0) mfma_set_v(x.s[0], kf, qf[0][kk]);
+    if (m == 1) mfma_set_v(x.s[1], kf, qf[1][kk]);
+    if (m == 2) mfma_from_v(x.dp[0], vf, dof[0][kk], neg_delta[0]);
+    if (m == 3) mfma_from_vv(x.dp[1], vf, dof[1][kk], neg_delta[1]);
+  } else {
+    if (m == 0) mfma_acc_v(x.s[0], kf, qf[0][kk]);
+    if (m == 1) mfma_acc_v(x.s[1], kf, qf[1][kk]);
+    if (m == 2) mfma_acc_v(x.dp[0], vf, dof[0][kk]);
+    if (m == 3) mfma_acc_vv(x.dp[1], vf, dof[1][kk]);
+  }
+}
+
+// One step (32 keys).  NEXT: issue the score MFMAs of the following 32 keys (fragments of sub-tile nt
+// at nk_rows / nv_rows) into `nxt`.  MASK: the step is on the causal diagonal; lim[qb] is the last
+// visible key of the lane's row, relative to the lane's first key of the step.
+template <bool NEXT, bool MASK>
+__device__ __forceinline__ void dq_step(DqScores& nxt, const DqScores& cur, f32x16 (&dq)[2][HD / 32],
+                                        uint32_t nk_rows, uint32_t nv_rows, int nt, uint32_t k_cols, int t,
+                                        const bf16x8 (&qf)[2][HD / 16], const bf16x8 (&dof)[2][HD / 16],
+                                        float scale_log2, const float (&neg_lse)[2],
+                                        const f32x16 (&neg_delta)[2], const int (&lim)[2]) {
+  bf16x8 dsb[2][2];
+  auto one_score = [&](int g) {  // lane: query row of block g / 16, key 8 (e / 4) + e % 4 (+ 4 h) of the step
+    const int qb = g >> 4, e = g & 15;
+    float sv = cur.s[qb][e];
+    if (MASK) sv = 8 * (e >> 2) + (e & 3) > lim[qb] ? -INFINITY : sv;
+    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sv, scale_log2, neg_lse[qb]));
+    dsb[qb][e >> 3][e & 7] = (bf16)(p * cur.dp[qb][e]);  // dP - delta comes out of the MFMAs
+  };
+  // Fragments are requested from LDS well ahead of the MFMA that takes them (two contraction steps
+  // = eight MFMAs for the score products, three fragments = six MFMAs for dQ): one wave per SIMD has
+  // nobody to cover an LDS round trip for it.
+  constexpr int NKT = 2 * (HD / 32);  // K^T fragments of the step: 2 contraction steps x 4 channel blocks
+  auto kt_frag = [&](int i) { return bt_cols(k_cols, 2 * t + i / (HD / 32), i % (HD / 32)); };
+  bf16x8 kt[3];
+  if (NEXT) {
+    bf16x8 kf[3], vf[3];
+    kf[0] = bt_rows(nk_rows, nt, 0);
+    vf[0] = bt_rows(nv_rows, nt, 0);
+    kf[1] = bt_rows(nk_rows, nt, 1);
+    vf[1] = bt_rows(nv_rows, nt, 1);
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        if (m == 0 && kk + 2 < HD / 16) kf[(kk + 2) % 3] = bt_rows(nk_rows, nt, kk + 2);
+        if (m == 2 && kk + 2 < HD / 16) vf[(kk + 2) % 3] = bt_rows(nv_rows, nt, kk + 2);
+        if (m == 1 && kk >= HD / 16 - 3) kt[kk - (HD / 16 - 3)] = kt_frag(kk - (HD / 16 - 3));
+        dq_score_mfma(nxt, kk, m, kf[kk % 3], vf[kk % 3], qf, dof, neg_delta);
+        one_score(kk * 4 + m);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) kt[i] = kt_frag(i);
+#pragma unroll
+    for (int g = 0; g < 32; ++g) one_score(g);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 3");
+  }
+#pragma unroll
+  for (int i = 0; i < NKT; ++i) {
+    const int k2 = i / (HD / 32), dt = i % (HD / 32);
+    const bf16x8 frag = kt[i % 3];
+    dq[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, dsb[0][k2], dq[0][dt], 0, 0, 0);
+    dq[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag, dsb[1][k2], dq[1][dt], 0, 0, 0);
+    if (i + 3 < NKT) kt[i % 3] = kt_frag(i + 3);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+__global__ __launch_bounds__(256, 1) void attn_bwd_dq_w64_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
+    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
+    KLayout kl, KLayout vl, QLayout dol, QLayout dql) {
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];
+  constexpr uint32_t STAGE = 2 * BT_BYTES;  // K tile | V tile
+  constexpr int ROWS = 256;                 // queries per workgroup: 64 per wave
+  constexpr int NSTAGE = 3;                 // tiles in LDS: the one in use, the next, the one after
+
+  const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nqt = s / ROWS;
+  const int lid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  int qt, pair;
+  longest_first(lid, nqt, gridDim.x / nqt, qt, pair);
+  const int head = pair % nq;
+  const int bi = pair / nq;
+  const int per = nq / nkv;
+  const int kvh = head / per;
+  const int q0 = qt * ROWS;
+  const int qw0 = q0 + wave * 64;
+
+  const bf16* kb = k + kl.at(bi, kvh);
+  const bf16* vb = v + vl.at(bi, kvh);
+  bf16x8 qf[2][HD / 16], dof[2][HD / 16];
+  float neg_lse[2];
+  f32x16 neg_delta[2];
+  int lim[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qrow = qw0 + 32 * qb + (lane & 31);
+    const bf16* qp = q + ql.at(bi, head, per) + (int64_t)qrow * ql.s_;
+    const bf16* dop = dout + dol.at(bi, head, per) + (int64_t)qrow * dol.s_;
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+      qf[qb][kk] = ldg8(qp + kk * 16 + h * 8);
+      dof[qb][kk] = ldg8(dop + kk * 16 + h * 8);
+    }
+    const int64_t stat = ((int64_t)bi * nq + head) * s + qrow;
+    neg_lse[qb] = -lse[stat] * kLog2e;
+    const float d = -delta[stat];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) neg_delta[qb][e] = d;
+  }
+
+  f32x16 dqacc[2][HD / 32];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dqacc[qb][dt][e] = 0.f;
+
+  const int ntiles = (q0 + ROWS) / BKV;                             // key tiles of the workgroup
+  const int last = __builtin_amdgcn_readfirstlane(qw0 / BKV);       // this wave's tile on the diagonal
+  const uint32_t area = (uint32_t)(uintptr_t)(KR_LDS const bf16*)smem;
+  auto stage_request = [&](int j, int buf) {  // the four waves bring in the K and the V tile together
+    bt_request(kb + (int64_t)(j * BKV) * kl.s_, kl.s_, area + buf * STAGE, wave, lane);
+    bt_request(vb + (int64_t)(j * BKV) * vl.s_, vl.s_, area + buf * STAGE + BT_BYTES, wave, lane);
+  };
+  stage_request(0, 0);
+  stage_request(1, 1);  // ntiles >= 4
+  __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): everything but the second tile's requests has landed
+  __syncthreads();
+  settle_scalar_loads();
+
+  const uint32_t rows_lane = bt_rows_lane(lane), cols_lane = bt_cols_lane(lane);
+  DqScores a, b;
+  {  // scores of the first 32 keys (tile 0 is below every wave's diagonal or on it)
+    const uint32_t k_rows = area + rows_lane, v_rows = k_rows + BT_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < HD / 16; ++kk) {
+      const bf16x8 kf = bt_rows(k_rows, 0, kk), vf = bt_rows(v_rows, 0, kk);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) dq_score_mfma(a, kk, m, kf, vf, qf, dof, neg_delta);
+    }
+    asm volatile("s_nop 15\n\ts_nop 15");
+  }
+  // Every wave passes the same ntiles barriers and makes the same requests; what differs is how many
+  // of the tiles it computes on (those up to its diagonal).  Three loops without branches inside
+  // (a branch around a step would put copies of all accumulators at the merge): tiles below the
+  // diagonal, the diagonal tile, the tiles only the waves further down still need.
+  int buf = 0;  // stage of tile j
+  auto arrive = [&](int j) {  // between the two steps of tile j
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile j + 1 has landed
+    __syncthreads();                     // ... and everyone's; nobody reads tile j - 1 any more
+  };
+  auto turn = [&](int j) {
+    arrive(j);
+    if (j + NSTAGE - 1 < ntiles) stage_request(j + NSTAGE - 1, buf == 0 ? NSTAGE - 1 : buf - 1);
+  };
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) lim[qb] = 0;
+  for (int j = 0; j < last; ++j) {
+    const int buf_next = buf == NSTAGE - 1 ? 0 : buf + 1;
+    uint32_t k_rows = area + buf * STAGE + rows_lane, v_rows = k_rows + BT_BYTES;
+    uint32_t k_cols = area + buf * STAGE + cols_lane;
+    uint32_t nk_rows = area + buf_next * STAGE + rows_lane, nv_rows = nk_rows + BT_BYTES;
+    asm volatile("" : "+v"(k_rows), "+v"(v_rows), "+v"(k_cols), "+v"(nk_rows), "+v"(nv_rows));
+    dq_step<true, false>(b, a, dqacc, k_rows, v_rows, 1, k_cols, 0, qf, dof, scale_log2, neg_lse, neg_delta, lim);
+    turn(j);
+    dq_step<true, false>(a, b, dqacc, nk_rows, nv_rows, 0, k_cols, 1, qf, dof, scale_log2, neg_lse, neg_delta, lim);
+    buf = buf_next;
+  }
+  {  // the diagonal tile (keys qw0 .. qw0 + 63): lim = last visible key of the lane's row, counted
+     // from the lane's first key of the step
+    uint32_t k_rows = area + buf * STAGE + rows_lane, v_rows = k_rows + BT_BYTES;
+    uint32_t k_cols = area + buf * STAGE + cols_lane;
+    asm volatile("" : "+v"(k_rows), "+v"(v_rows), "+v"(k_cols));
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) lim[qb] = 32 * qb + (lane & 31) - 4 * h;
+    dq_step<true, true>(b, a, dqacc, k_rows, v_rows, 1, k_cols, 0, qf, dof, scale_log2, neg_lse, neg_delta, lim);
+    turn(last);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) lim[qb] -= 32;
+    dq_step<false, true>(a, b, dqacc, 0, 0, 0, k_cols, 1, qf, dof, scale_log2, neg_lse, neg_delta, lim);
+    buf = buf == NSTAGE - 1 ? 0 : buf + 1;
+  }
+  for (int j = last + 1; j < ntiles; ++j) {
+    turn(j);
+    buf = buf == NSTAGE - 1 ? 0 : buf + 1;
+  }
+
+  RowStage rs;
+  rs.init(reinterpret_cast<char*>(smem) + NSTAGE * STAGE + wave * 4096, lane);
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+    store_rows_bf16(rs, dqacc[qb], scale, dq + dql.at(bi, head, per) + (int64_t)(qw0 + 32 * qb) * dql.s_, dql.s_);
 }
 
 #define KR_ATTN_DQ_ARGS                                                                          \
   const bf16*, const bf16*, const bf16*, const bf16*, const float*, const float*, bf16*, int, int, \
       int, float, float, QLayout, KLayout, KLayout, QLayout, QLayout
-template __global__ void attn_bwd_dq_kernel<1, false>(KR_ATTN_DQ_ARGS);
-template __global__ void attn_bwd_dq_kernel<2, false>(KR_ATTN_DQ_ARGS);
-template __global__ void attn_bwd_dq_kernel<2, true>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<1>(KR_ATTN_DQ_ARGS);
+template __global__ void attn_bwd_dq_kernel<2>(KR_ATTN_DQ_ARGS);
 #undef KR_ATTN_DQ_ARGS
 
 #define KR_ATTN_DKDV_ARGS                                                                          \
@@ -1711,13 +1962,10 @@ __global__ __launch_bounds__(256) void attn_resize_rows_kernel(const float* __re
 
 }  // namespace
 
-// Build-time caps, for measuring one form of a kernel against another: the most query heads a
-// dK/dV workgroup takes, and the most workgroups the dQ kernel over shared key tiles is used for.
+// Build-time cap, for measuring one form of a kernel against another: the most query heads a
+// dK/dV workgroup takes.
 #ifndef KR_DKDV_HPW_MAX
 #define KR_DKDV_HPW_MAX 4
-#endif
-#ifndef KR_DQ_SHARED_MAX
-#define KR_DQ_SHARED_MAX (1 << 30)
 #endif
 // The dK/dV kernel runs one workgroup per CU.  With at most two rounds of workgroups its time is
 // set by the first key tiles (they see every query): two workgroups then share each key tile.
@@ -1801,7 +2049,7 @@ static AttnForms attn_forms(int s, int b, int nq, int flags) {
   const int tiles256 = (s / 256) * nq * b;
   AttnForms f;
   f.shared_fwd = s % 256 == 0 && (beside || tiles256 >= kr_compute_units());
-  f.shared_dq = s % 256 == 0 && (beside || tiles256 >= kr_compute_units()) && 2 * tiles256 <= KR_DQ_SHARED_MAX;
+  f.shared_dq = s % 256 == 0 && (beside || tiles256 >= kr_compute_units());
   f.qsplit = beside ? 1 : dkdv_query_split(s, b, nq);
   return f;
 }
@@ -1905,6 +2153,7 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   const bool partial = nq / hpw != nkv || qsplit > 1;
   constexpr size_t lds_dkdv = 3 * (2 * BT_BYTES + 512) + 32768;  // three stages + the hand-over area
   constexpr size_t lds_dq = 2 * (2 * BT_BYTES);  // two stages of a K and a V tile
+  constexpr size_t lds_dq_w64 = 3 * (2 * BT_BYTES) + 4 * 4096;  // three stages + a 4 KB output stage per wave
   static const hipError_t attr_status = [] {
     hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
@@ -1912,14 +2161,14 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
       e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkdv);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1, false>,
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<1>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2, false>,
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * lds_dq));
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<2, true>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq);
+      e = hipFuncSetAttribute((const void*)attn_bwd_dq_w64_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq_w64);
     return e;
   }();
   if (attr_status != hipSuccess) return KR_ELAUNCH;
@@ -1949,18 +2198,18 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const int dq_blocks = (s / BQ) * nq * b;
   if (forms.shared_dq) {
-    // 256-query tiles (one for every compute unit, or other streams beside): the halves share their K / V tiles
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<2, true>), dim3(dq_blocks / 2), dim3(512), lds_dq, st,
+    // 256-query tiles (one for every compute unit, or other streams beside): one wave per SIMD, 64 rows each
+    hipLaunchKernelGGL(attn_bwd_dq_w64_kernel, dim3(dq_blocks / 2), dim3(256), lds_dq_w64, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
                        dql);
   } else if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<2, false>), dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<2>), dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
                        dql);
   } else {
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<1, false>), dim3(dq_blocks), dim3(256), lds_dq, st,
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<1>), dim3(dq_blocks), dim3(256), lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
                        dql);
