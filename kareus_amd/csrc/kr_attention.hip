@@ -1581,7 +1581,8 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_w64_kernel(
 #pragma unroll
       for (int m = 0; m < 4; ++m) dq_score_mfma(a, kk, m, kf, vf, qf, dof, neg_delta);
     }
-    asm volatile("s_nop 15\n\ts_nop 15");
+    // the scores pass through the wait: no reader can be moved in front of it
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a.s[0]), "+v"(a.s[1]), "+v"(a.dp[0]), "+v"(a.dp[1]));
   }
   // Every wave passes the same ntiles barriers and makes the same requests; what differs is how many
   // of the tiles it computes on (those up to its diagonal).  Three loops without branches inside
