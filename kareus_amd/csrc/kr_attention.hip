@@ -1380,8 +1380,9 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
 // 1 KB fragment faster than an MFMA takes, which is what holds the two-waves-per-SIMD kernels at
 // half of the matrix pipe.  With a single instruction stream per SIMD nothing else would fill the
 // pipe while the wave does its vector work, so the loop is software-pipelined by hand: behind each of
-// the 32 score MFMAs (S^T, dP^T) of the NEXT 32 keys sits the exponential, multiply-add, subtraction,
-// multiplication and rounding of one score per lane of THIS step, then come this step's 16 dQ MFMAs.
+// the 32 score MFMAs (S^T, dP^T) of the NEXT 32 keys sits the multiply-add, exponential, multiplication
+// and rounding of one score per lane of THIS step (dP^T comes out of its MFMAs with delta already
+// subtracted), then come this step's 16 dQ MFMAs.
 //
 // The score MFMAs are inline assembly because their register file has to be chosen: a kernel with more
 // than 256 registers gets its MFMA results in the accumulation registers, and every score would
@@ -1392,8 +1393,9 @@ __global__ __launch_bounds__(256 * HALVES, HALVES == 1 ? 2 : 1) void attn_bwd_dq
 // instruction and a reader of its result are provided by construction:
 //   * a score accumulator is read by vector instructions one step after the MFMAs that wrote it,
 //     with that step's 16 dQ MFMAs in between (before the loop: explicit s_nop);
-//   * accumulators start from the instruction's zero operand, never from a vector write, and a
-//     result that is not also the addend is an early-clobber operand.
+//   * score accumulators start from the instruction's zero operand or from a tuple set up before the
+//     loop, never from a fresh vector write, and a result that is not also the addend is an
+//     early-clobber operand (the instruction writes while it still reads).
 // tests/test_attention_asm.py checks the compiled kernel for any reader that comes too early.
 // Fragments come from LDS through ordinary loads, whose waits the compiler does insert.
 // ---------------------------------------------------------------------------------------------
