@@ -1506,11 +1506,15 @@ __device__ __forceinline__ void dq_step(DqScores& nxt, const DqScores& cur, f32x
   }
 }
 
+// The kernel also takes over the pre-pass of the backward: each wave forms delta = sum_d dO . O of its 64
+// rows from the dO fragments it holds anyway, uses it, and writes it (and -lse in the log2 domain) for
+// the dK/dV kernel, which the host launches behind this one.
 __global__ __launch_bounds__(256, 1) void attn_bwd_dq_w64_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k, const bf16* __restrict__ v,
-    const bf16* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16* __restrict__ dq, int s, int nq, int nkv, float scale, float scale_log2, QLayout ql,
-    KLayout kl, KLayout vl, QLayout dol, QLayout dql) {
+    const bf16* __restrict__ dout, const bf16* __restrict__ o, const float* __restrict__ lse,
+    float* __restrict__ delta_out, float* __restrict__ neg_lse2_out, bf16* __restrict__ dq, int s, int nq,
+    int nkv, float scale, float scale_log2, QLayout ql, KLayout kl, KLayout vl, QLayout dol, QLayout ol,
+    QLayout dql) {
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];
   constexpr uint32_t STAGE = 2 * BT_BYTES;  // K tile | V tile
   constexpr int ROWS = 256;                 // queries per workgroup: 64 per wave
@@ -1540,16 +1544,30 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dq_w64_kernel(
     const int qrow = qw0 + 32 * qb + (lane & 31);
     const bf16* qp = q + ql.at(bi, head, per) + (int64_t)qrow * ql.s_;
     const bf16* dop = dout + dol.at(bi, head, per) + (int64_t)qrow * dol.s_;
+    const bf16* op = o + ol.at(bi, head, per) + (int64_t)qrow * ol.s_;
+    // delta from a second read of the dO row: the fragments kept for the MFMAs must stay values that
+    // only the MFMAs read, or the compiler keeps them in VGPRs and copies them into accumulation
+    // registers in front of every MFMA
+    const bf16* dop2 = dop;
+    asm volatile("" : "+v"(dop2));
+    float dsum = 0.f;  // this lane's half of the row (channels 16 kk + 8 h ..)
 #pragma unroll
     for (int kk = 0; kk < HD / 16; ++kk) {
       qf[qb][kk] = ldg8(qp + kk * 16 + h * 8);
       dof[qb][kk] = ldg8(dop + kk * 16 + h * 8);
+      const bf16x8 dov = ldg8(dop2 + kk * 16 + h * 8), of = ldg8(op + kk * 16 + h * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dsum += (float)dov[e] * (float)of[e];
     }
+    dsum += __shfl_xor(dsum, 32, KR_WAVE);
     const int64_t stat = ((int64_t)bi * nq + head) * s + qrow;
     neg_lse[qb] = -lse[stat] * kLog2e;
-    const float d = -delta[stat];
+    if (h == 0) {
+      delta_out[stat] = dsum;
+      neg_lse2_out[stat] = neg_lse[qb];
+    }
 #pragma unroll
-    for (int e = 0; e < 16; ++e) neg_delta[qb][e] = d;
+    for (int e = 0; e < 16; ++e) neg_delta[qb][e] = -dsum;
   }
 
   f32x16 dqacc[2][HD / 32];
@@ -2177,10 +2195,19 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   if (attr_status != hipSuccess) return KR_ELAUNCH;
 
   const int per = nq / nkv;
-  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
-                     (const bf16*)dout, (const bf16*)o, lse, delta, neg_lse2, s, nq, per, rows, dol, ol);
-  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const float scale_log2 = scale * kLog2e;
+  const int dq_blocks = (s / BQ) * nq * b;
+  if (forms.shared_dq) {
+    // 256-query tiles (one for every compute unit, or other streams beside): one wave per SIMD, 64 rows each.
+    // It comes first: it also computes delta and the log2-domain copy of lse that the dK/dV kernel reads.
+    hipLaunchKernelGGL(attn_bwd_dq_w64_kernel, dim3(dq_blocks / 2), dim3(256), lds_dq_w64, st,
+                       (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, (const bf16*)o, lse,
+                       delta, neg_lse2, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol, ol, dql);
+  } else {
+    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, st,
+                       (const bf16*)dout, (const bf16*)o, lse, delta, neg_lse2, s, nq, per, rows, dol, ol);
+  }
+  if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
   const dim3 grid_kv((s / 128) * (nq / hpw) * b * qsplit);
 #define KR_DKDV_LAUNCH(P)                                                                           \
   hipLaunchKernelGGL((attn_bwd_dkdv_kernel<P>), grid_kv, dim3(512), lds_dkdv, st, (const bf16*)q,   \
@@ -2199,14 +2226,8 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   }
 #undef KR_DKDV_LAUNCH
   if (hipGetLastError() != hipSuccess) return KR_ELAUNCH;
-  const int dq_blocks = (s / BQ) * nq * b;
-  if (forms.shared_dq) {
-    // 256-query tiles (one for every compute unit, or other streams beside): one wave per SIMD, 64 rows each
-    hipLaunchKernelGGL(attn_bwd_dq_w64_kernel, dim3(dq_blocks / 2), dim3(256), lds_dq_w64, st,
-                       (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
-                       (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,
-                       dql);
-  } else if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
+  if (forms.shared_dq) return kr_launch_status();  // its dQ kernel ran in front of the dK/dV kernel
+  if (dq_blocks <= 4 * 256) {  // few workgroups: the longest causal rows set the time
     hipLaunchKernelGGL((attn_bwd_dq_kernel<2>), dim3(dq_blocks), dim3(512), 2 * lds_dq, st,
                        (const bf16*)q, (const bf16*)k, (const bf16*)v, (const bf16*)dout, lse,
                        (const float*)delta, (bf16*)dq, s, nq, nkv, scale, scale_log2, ql, kl, vl, dol,

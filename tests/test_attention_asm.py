@@ -15,6 +15,7 @@ import pytest
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "kareus_amd", "csrc")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 WAIT_SLOTS = 12
+OPERAND_SLOTS = 4
 
 
 def _regs(token, kind):
@@ -40,11 +41,12 @@ def _kernel_body(text, kernel):
 
 def early_readers(lines, need=WAIT_SLOTS):
     """(number of inline-assembly MFMAs, [(line, text, distance)] of instructions that read a VGPR less than
-    `need` issue slots after an inline-assembly MFMA wrote it).  Every instruction counts as one slot (they
-    take at least that), `s_nop n` as n + 1.  An MFMA accumulating onto its own earlier result is the
+    `need` issue slots after an inline-assembly MFMA wrote it, and of inline-assembly MFMAs that take an operand
+    a vector instruction wrote fewer than OPERAND_SLOTS slots before).  Every instruction counts as one slot
+    (they take at least that), `s_nop n` as n + 1.  An MFMA accumulating onto its own earlier result is the
     hardware's business and is not a reader here."""
     stores = ("ds_write", "global_store", "buffer_store", "scratch_store")
-    in_asm, slot, written, bad, n_asm = False, 0, {}, [], 0
+    in_asm, slot, written, bad, n_asm, fresh = False, 0, {}, [], 0, {}
     for i, line in enumerate(lines):
         t = line.strip()
         if t.startswith(";;#ASMSTART"):
@@ -64,9 +66,20 @@ def early_readers(lines, need=WAIT_SLOTS):
             continue
         if in_asm and op.startswith("v_mfma"):
             n_asm += 1
+            # its operands must not have been written by a vector instruction just before it either: the
+            # compiler would separate such a pair if it knew what the assembly is
+            for a in args[1:]:
+                for kind in "va":
+                    for r in _regs(a, kind):
+                        if slot - fresh.get((kind, r), -10 ** 9) < OPERAND_SLOTS:
+                            bad.append((i, t, slot - fresh[(kind, r)]))
             for r in _regs(args[0], "v"):
                 written[r] = slot
             continue
+        if op.startswith("v_") and args:
+            for kind in "va":
+                for r in _regs(args[0], kind):
+                    fresh[(kind, r)] = slot
         for a in (args if op.startswith(stores) else args[1:]):
             for r in _regs(a, "v"):
                 if r in written and slot - written[r] < need:
@@ -87,6 +100,8 @@ def test_checker_sees_an_early_reader_and_accepts_a_late_one():
     assert early_readers(late) == (1, [])
     assert early_readers(chained) == (2, [])
     assert len(early_readers(spilled)[1]) == 4
+    copied = ["\tv_accvgpr_write_b32 a0, v9"] + mfma
+    assert early_readers(copied) == (1, [(2, "v_mfma_f32_32x32x16_bf16 v[0:15], v[20:23], a[0:3], 0", 1)])
 
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc is not installed")
