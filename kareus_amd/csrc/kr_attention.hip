@@ -186,8 +186,9 @@ inline bool attn_strides_ok(const int64_t (&seq)[N], std::initializer_list<int64
 }
 
 // =============================================================================================
-// Backward.  Launches: delta pre-pass, dK/dV pass, (group reduction), dQ pass.  No atomics,
-// deterministic.
+// Backward.  Launches: delta pre-pass, dK/dV pass, (group reduction), dQ pass — or, with 256-query
+// tiles, the one-wave dQ kernel first (it computes delta itself), then dK/dV and the group
+// reduction.  No atomics, deterministic.
 //   1. delta[b, h, i] = sum_d dO[i, d] * O[i, d]                      (HBM-bound pre-pass)
 //   2. dK, dV: a workgroup owns 128 keys of one (batch, QUERY head) — 32 per pair of waves,
 //      their K and V fragments in the registers of the pair's score wave, dK and dV in those of
