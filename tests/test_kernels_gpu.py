@@ -292,6 +292,11 @@ def test_attention_at_sequence_8192(be):
     assert rel(o, ro) <= TOL and rel(lse, rlse) <= 1e-4
     ro.backward(do.float().cpu())
     assert rel(dq.flatten(2, 3), qf.grad) <= TOL and rel(dk, kf.grad) <= TOL and rel(dv, vf.grad) <= TOL
+    # the whole forms (256-query workgroups: the query gradient with one wave per SIMD walks 128 key tiles here)
+    o2, lse2 = be.attn_fwd(q, k, v, hd ** -0.5, beside_other_streams=True)
+    assert rel(o2, ro) <= TOL and rel(lse2, rlse) <= 1e-4
+    dq2, dk2, dv2 = be.attn_bwd(do, q, k, v, o2, lse2, hd ** -0.5, beside_other_streams=True)
+    assert rel(dq2.flatten(2, 3), qf.grad) <= TOL and rel(dk2, kf.grad) <= TOL and rel(dv2, vf.grad) <= TOL
 
 
 def test_attention_does_not_depend_on_the_launch_size(be):
