@@ -610,6 +610,11 @@ def hbm_kernels(w, nnb, device, launches=50):
         qk = torch.randn(s_len, t // s_len, heads, hd, device=device, dtype=bf)
         freqs = rotary_frequencies(s_len, hd, 500000.0, device=device)
         report("rope_kernel (q and k heads)", t, 2 * t * heads * hd * 2, lambda: be.rope_fwd(qk, freqs))
+        # hidden dropout (not part of the benchmark workloads, p = 0 there): two bf16 operands read, the
+        # sum and a byte mask written; backward one bf16 operand and the mask read, one result written
+        _, mask = be.dropout_add(x, y, 0.1)
+        report("dropout_add_kernel (p = 0.1)", t, t * h * (3 * 2 + 1), lambda: be.dropout_add(x, y, 0.1))
+        report("dropout_bwd_kernel", t, t * h * (2 * 2 + 1), lambda: be.dropout_bwd(y, mask, 1 / 0.9))
     return rows_out
 
 

@@ -248,6 +248,26 @@ int kr_add(const void* a, const void* b, void* out, int64_t n, void* stream);
 int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
                 int64_t rows, int cols, void* stream);
 
+/* ---- Hidden dropout in front of the residual add ---------------------------------------
+ * out = residual + dropout(x) with probability p in [0, 1): replaces the Inductor kernels of
+ * fused_bias_dropout_add_forward / _backward without bias
+ * (kareus/megatron/core/extensions/ops/bias_dropout_add.py:15-45: native_dropout, then the add;
+ * native_dropout_backward(grad, mask, 1 / (1 - p))).
+ * kr_dropout_add: mask [rows, cols] bytes, dense (1 = kept), written for the backward;
+ *   out = bf16(residual + bf16(x * mask / (1 - p))) — the product is rounded before the add, as the
+ *   reference's is.  The mask comes from Philox-4x32-10 keyed by `seed`, counter `offset` + the
+ *   index of the 8-element vector: the same (seed, offset) gives the same mask whatever the launch,
+ *   and a caller that advances `offset` by rows * cols / 8 per call never reuses a counter.  It is
+ *   not the mask PyTorch would draw from the same seed.
+ * kr_dropout_bwd: dx = bf16(dy * mask * scale).
+ * Matrices [rows, cols] with row strides in elements (multiples of 8, >= cols; cols a multiple of
+ * 8), so that a strided nanobatch slice is used where it lies.  out may alias residual.        */
+int kr_dropout_add(const void* x, int64_t ldx, const void* residual, int64_t ldr, void* out, int64_t ldo,
+                   void* mask, int64_t rows, int cols, float p, uint64_t seed, uint64_t offset,
+                   void* stream);
+int kr_dropout_bwd(const void* dy, int64_t lddy, const void* mask, void* dx, int64_t lddx, int64_t rows,
+                   int cols, float scale, void* stream);
+
 /* ---- Causal grouped-query attention ----------------------------------------------------
  * Replaces flash_attn_2_cuda.fwd / bwd as called from
  * kareus/flash_attn/flash_attn_interface.py:66-80, 174-194.

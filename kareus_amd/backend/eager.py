@@ -156,6 +156,23 @@ class EagerBackend:
             raise RuntimeError(f"add: out has shape {tuple(out.shape)}, operands {tuple(a.shape)}")
         return torch.add(a, b, out=out)
 
+    # residual + dropout(x) and the byte mask (kareus/megatron/core/extensions/ops/bias_dropout_add.py:15-45)
+    def dropout_add(self, x: Tensor, residual: Tensor, p: float, out: Tensor = None):
+        seed = int(torch.randint(0, 1 << 62, (1,), dtype=torch.int64).item())   # as the hip backend draws it
+        gen = torch.Generator(device=x.device).manual_seed(seed)
+        keep = torch.rand(x.shape, generator=gen, device=x.device) >= p
+        dropped = (x.float() * keep / (1.0 - p)).to(x.dtype)
+        total = (residual.float() + dropped.float()).to(x.dtype)
+        if out is not None:
+            if out.shape != x.shape:
+                raise RuntimeError(f"dropout_add: out has shape {tuple(out.shape)}, operands {tuple(x.shape)}")
+            out.copy_(total)
+            total = out
+        return total, keep.to(torch.uint8)
+
+    def dropout_bwd(self, dy: Tensor, mask: Tensor, scale: float) -> Tensor:
+        return (dy.float() * mask * scale).to(dy.dtype)
+
     # Causal GQA attention on [s, b, heads, hd] tensors; query head i reads KV head
     # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32
     # (kareus/flash_attn/flash_attn_interface.py:473-493).

@@ -55,6 +55,9 @@ _SIGNATURES = {
     "kr_swiglu_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_void_p]),
     "kr_add": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_i64, _c_void_p]),
     "kr_add_rows": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_i64, _c_int, _c_void_p]),
+    "kr_dropout_add": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_int,
+                                _c_float, ctypes.c_uint64, ctypes.c_uint64, _c_void_p]),
+    "kr_dropout_bwd": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_void_p, _c_i64, _c_i64, _c_int, _c_float, _c_void_p]),
     "kr_embedding_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_embedding_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_cross_entropy_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p]),
@@ -584,6 +587,52 @@ class HipBackend:
         self._check(self.lib.kr_add_rows(a2.data_ptr(), a2.stride(0), b2.data_ptr(), b2.stride(0),
                                          o2.data_ptr(), o2.stride(0), rows, cols, self._stream()), "kr_add_rows")
         return out
+
+    def dropout_add(self, x: Tensor, residual: Tensor, p: float, out: Tensor = None) -> Tuple[Tensor, Tensor]:
+        """``residual + dropout(x, p)`` and the byte mask of kept elements (same shape, dense).  The
+        mask is keyed by a seed drawn from PyTorch's CPU generator, so ``torch.manual_seed`` fixes it
+        and a restored CPU generator state (activation recomputation) reproduces it."""
+        self._dev(x, residual)
+        self._bf16(x, residual)
+        if x.shape != residual.shape:
+            raise RuntimeError(f"dropout_add: shapes differ, {tuple(x.shape)} vs {tuple(residual.shape)}")
+        if not 0.0 <= p < 1.0:
+            raise RuntimeError(f"dropout_add: probability {p} is outside [0, 1)")
+        x2, r2 = self._rows(self._leading_rows(x)), self._rows(self._leading_rows(residual))
+        if out is None:
+            out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        else:
+            self._dev(out)
+            self._bf16(out)
+            if out.shape != x.shape:
+                raise RuntimeError(f"dropout_add: out has shape {tuple(out.shape)}, operands {tuple(x.shape)}")
+        try:
+            o2 = out.view(x2.shape)
+        except RuntimeError:
+            o2 = None
+        if o2 is None or o2.stride(1) != 1 or o2.stride(0) % 8 or o2.stride(0) < o2.shape[1]:
+            raise RuntimeError("dropout_add: out cannot be addressed with a single row stride")
+        rows, cols = x2.shape
+        mask = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+        seed = int(torch.randint(0, 1 << 62, (1,), dtype=torch.int64).item())
+        self._check(self.lib.kr_dropout_add(x2.data_ptr(), x2.stride(0), r2.data_ptr(), r2.stride(0), o2.data_ptr(),
+                                            o2.stride(0), mask.data_ptr(), rows, cols, float(p), seed, 0,
+                                            self._stream()), "kr_dropout_add")
+        return out, mask
+
+    def dropout_bwd(self, dy: Tensor, mask: Tensor, scale: float) -> Tensor:
+        """``dy * mask * scale``: native_dropout_backward."""
+        self._dev(dy)
+        self._bf16(dy)
+        if (not mask.is_cuda or mask.dtype != torch.uint8 or mask.shape != dy.shape
+                or not mask.is_contiguous()):
+            raise RuntimeError("dropout_bwd: the mask must be the dense byte mask the forward wrote")
+        d2 = self._rows(self._leading_rows(dy))
+        dx = torch.empty(dy.shape, dtype=dy.dtype, device=dy.device)
+        rows, cols = d2.shape
+        self._check(self.lib.kr_dropout_bwd(d2.data_ptr(), d2.stride(0), mask.data_ptr(), dx.data_ptr(), cols, rows, cols,
+                                            float(scale), self._stream()), "kr_dropout_bwd")
+        return dx
 
     @staticmethod
     def _leading_rows(t: Tensor) -> Tensor:

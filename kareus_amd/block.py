@@ -213,9 +213,10 @@ class DecoderLayer(torch.nn.Module):
         fuse = bool(getattr(c, "fuse_forward_epilogues", False))
         self.linear_fc1.fuse_activation = fuse    # SwiGLU forward in fc1's epilogue
         self.linear_fc2.fuse_activation = fuse    # SwiGLU backward in the epilogue of fc2's input gradient
+        # (with hidden dropout the residual is added behind the dropout, by the op that follows)
         for row_parallel in (self.linear_proj, self.linear_fc2):
-            row_parallel.fuse_residual = fuse
-            row_parallel.forward_accepts_out_sink = fuse
+            row_parallel.fuse_residual = fuse and c.hidden_dropout == 0.0
+            row_parallel.forward_accepts_out_sink = fuse and c.hidden_dropout == 0.0
 
     def get_all_operators(self) -> List:
         return [

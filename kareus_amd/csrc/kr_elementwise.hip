@@ -41,6 +41,74 @@ __global__ __launch_bounds__(kThreads) void add_rows_kernel(const bf16* a, int64
   }
 }
 
+// ---- hidden dropout in front of the residual add ------------------------------------------------
+// Philox-4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"): a counter-based
+// generator, so element i of a call gets the same bits whatever the launch shape.  One call of the
+// generator (128 bits) serves 8 elements, 16 bits each: an element is kept when its 16 bits are at
+// or above p * 65536.
+__device__ __forceinline__ void philox4x32_10(uint32_t (&ctr)[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * ctr[0], p1 = (uint64_t)0xCD9E8D57u * ctr[2];
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ ctr[1] ^ k0, n2 = (uint32_t)(p0 >> 32) ^ ctr[3] ^ k1;
+    ctr[1] = (uint32_t)p1;
+    ctr[3] = (uint32_t)p0;
+    ctr[0] = n0;
+    ctr[2] = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// out = residual + bf16(x * mask / (1 - p)); mask [rows, cols] bytes (1 = kept), dense.  The product
+// is rounded to bf16 before the add, as the reference's dropout output is.
+__global__ __launch_bounds__(kThreads) void dropout_add_kernel(const bf16* x, int64_t ldx, const bf16* res,
+                                                               int64_t ldr, bf16* out, int64_t ldo,
+                                                               uint8_t* __restrict__ mask, int64_t rows, int cols,
+                                                               uint32_t threshold, float scale, uint64_t seed,
+                                                               uint64_t offset) {
+  const int nv = cols / 8;
+  const int64_t total = rows * nv, stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / nv;
+    const int c = (int)(i - r * nv) * 8;
+    const uint64_t index = offset + (uint64_t)i;  // one generator call per 8 elements
+    uint32_t ctr[4] = {(uint32_t)index, (uint32_t)(index >> 32), 0u, 0u};
+    philox4x32_10(ctr, (uint32_t)seed, (uint32_t)(seed >> 32));
+    const bf16x8 xv = ldg8(x + r * ldx + c), rv = ldg8(res + r * ldr + c);
+    bf16x8 o;
+    uint64_t m = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t bits = (ctr[e >> 1] >> (16 * (e & 1))) & 0xffffu;
+      const bool keep = bits >= threshold;
+      const bf16 d = (bf16)(keep ? (float)xv[e] * scale : 0.f);
+      o[e] = (bf16)((float)rv[e] + (float)d);
+      m |= (uint64_t)(keep ? 1 : 0) << (8 * e);
+    }
+    stg8(out + r * ldo + c, o);
+    *reinterpret_cast<uint64_t*>(mask + r * cols + c) = m;
+  }
+}
+
+// dx = bf16(dy * mask * scale)
+__global__ __launch_bounds__(kThreads) void dropout_bwd_kernel(const bf16* dy, int64_t lddy,
+                                                               const uint8_t* __restrict__ mask, bf16* dx,
+                                                               int64_t lddx, int64_t rows, int cols, float scale) {
+  const int nv = cols / 8;
+  const int64_t total = rows * nv, stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / nv;
+    const int c = (int)(i - r * nv) * 8;
+    const bf16x8 g = ldg8(dy + r * lddy + c);
+    const uint64_t m = *reinterpret_cast<const uint64_t*>(mask + r * cols + c);
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)(((m >> (8 * e)) & 1) ? (float)g[e] * scale : 0.f);
+    stg8(dx + r * lddx + c, o);
+  }
+}
+
 __device__ __forceinline__ float sigmoidf_(float x) { return kr_sigmoidf(x); }
 
 // x [rows, 2F] -> y [rows, F]; one thread per 8 output columns.
@@ -162,6 +230,34 @@ extern "C" int kr_add_rows(const void* a, int64_t lda, const void* b, int64_t ld
   hipLaunchKernelGGL(add_rows_kernel, dim3(grid_for(rows * (cols / 8), kThreads)), dim3(kThreads), 0,
                      (hipStream_t)stream, (const bf16*)a, lda, (const bf16*)b, ldb, (bf16*)out, ldo,
                      rows, cols);
+  return kr_launch_status();
+}
+
+extern "C" int kr_dropout_add(const void* x, int64_t ldx, const void* residual, int64_t ldr, void* out,
+                              int64_t ldo, void* mask, int64_t rows, int cols, float p, uint64_t seed,
+                              uint64_t offset, void* stream) {
+  if (!x || !residual || !out || !mask || rows <= 0 || cols <= 0 || ldx < cols || ldr < cols || ldo < cols)
+    return KR_EINVAL;
+  if (!(p >= 0.f) || !(p < 1.f)) return KR_EINVAL;
+  if (cols % 8 || ldx % 8 || ldr % 8 || ldo % 8) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(x) || !kr_aligned16(residual) || !kr_aligned16(out) ||
+      (reinterpret_cast<uintptr_t>(mask) & 7u))
+    return KR_EINVAL;
+  const uint32_t threshold = (uint32_t)(p * 65536.0f + 0.5f);  // kept: 16 random bits >= threshold
+  hipLaunchKernelGGL(dropout_add_kernel, dim3(grid_for(rows * (cols / 8), kThreads)), dim3(kThreads), 0,
+                     (hipStream_t)stream, (const bf16*)x, ldx, (const bf16*)residual, ldr, (bf16*)out, ldo,
+                     (uint8_t*)mask, rows, cols, threshold, 1.0f / (1.0f - p), seed, offset);
+  return kr_launch_status();
+}
+
+extern "C" int kr_dropout_bwd(const void* dy, int64_t lddy, const void* mask, void* dx, int64_t lddx,
+                              int64_t rows, int cols, float scale, void* stream) {
+  if (!dy || !mask || !dx || rows <= 0 || cols <= 0 || lddy < cols || lddx < cols) return KR_EINVAL;
+  if (cols % 8 || lddy % 8 || lddx % 8) return KR_EUNSUPPORTED;
+  if (!kr_aligned16(dy) || !kr_aligned16(dx) || (reinterpret_cast<uintptr_t>(mask) & 7u)) return KR_EINVAL;
+  hipLaunchKernelGGL(dropout_bwd_kernel, dim3(grid_for(rows * (cols / 8), kThreads)), dim3(kThreads), 0,
+                     (hipStream_t)stream, (const bf16*)dy, lddy, (const uint8_t*)mask, (bf16*)dx, lddx, rows,
+                     cols, scale);
   return kr_launch_status();
 }
 

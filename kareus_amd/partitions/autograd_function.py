@@ -188,6 +188,11 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
                         c.output_sinks[producer] = sink
 
         schedule = scheduler.current_schedule if scheduler is not None else None
+        if checkpoint_activations:
+            # the recomputation in backward has to draw the same dropout masks
+            # (kareus/megatron/core/partitions/autograd_function.py:143-146)
+            func_ctx.fwd_cpu_rng_state = torch.get_rng_state()
+            func_ctx.fwd_cuda_rng_state = torch.cuda.get_rng_state() if torch.cuda.is_available() else None
         _fork(streams)
         _run_forward(fwd_parts, ctxs, schedule, is_grad_enabled)
         _join(streams)
@@ -247,7 +252,14 @@ class TransformerBlockAutogradFunction(torch.autograd.Function):
             hs = func_ctx.saved_tensors
             ctxs = [NanoBatchContext(batch_idx=i, stream=streams[i]) for i in range(n)]
             _seed_forward(ctxs, hs, rotary, mask, seed)
-            _run_forward(func_ctx.forward_partitions, ctxs, schedule, func_ctx.is_grad_enabled)
+            # with the generators as they were before the forward pass, and put back afterwards
+            # (kareus/megatron/core/partitions/autograd_function.py:263-266)
+            devices = [torch.cuda.current_device()] if func_ctx.fwd_cuda_rng_state is not None else []
+            with torch.random.fork_rng(devices=devices, enabled=True):
+                torch.set_rng_state(func_ctx.fwd_cpu_rng_state)
+                if func_ctx.fwd_cuda_rng_state is not None:
+                    torch.cuda.set_rng_state(func_ctx.fwd_cuda_rng_state)
+                _run_forward(func_ctx.forward_partitions, ctxs, schedule, func_ctx.is_grad_enabled)
             for c in ctxs:
                 c.finalize_recomputed_contexts()
         else:

@@ -19,7 +19,8 @@ reference reaches through third-party CUDA libraries, function by function:
                  dot_product_attention/backends.py:242-251, 304-347
   swiglu         kareus/megatron/core/extensions/ops/bias_swiglu.py:14-20; backward formula
                  :34-44 restated in ``swiglu_bwd_formula``
-  residual adds  kareus/megatron/core/extensions/ops/bias_dropout_add.py:24-45 with p = 0, no bias
+  residual adds  kareus/megatron/core/extensions/ops/bias_dropout_add.py:24-45, no bias; hidden dropout
+                 with the mask given (p = 0 in the benchmark workloads)
   layer order    kareus/megatron/core/transformer/transformer_layer.py:148-174
   embedding      3rdparty/Megatron-LM/megatron/core/tensor_parallel/layers.py:245-263 (rows of
                  one vocabulary shard, zeros for ids of other shards) and the [b s h] -> [s b h]
@@ -161,16 +162,30 @@ def init_layer_params(dims: LayerDims, generator: torch.Generator, std: float = 
     return p
 
 
-def layer_forward(x: Tensor, p: Dict[str, Tensor], dims: LayerDims, freqs: Tensor) -> Tensor:
-    """x [s, b, h] -> [s, b, h]; pre-norm attention block then pre-norm SwiGLU MLP block."""
+def dropout_with_mask(x: Tensor, mask: Tensor, prob: float) -> Tensor:
+    """native_dropout's output for a given mask of kept elements (0 / 1, same shape):
+    x * mask / (1 - p) (kareus/megatron/core/extensions/ops/bias_dropout_add.py:24-32)."""
+    return x * mask.to(x.dtype) / (1.0 - prob)
+
+
+def layer_forward(x: Tensor, p: Dict[str, Tensor], dims: LayerDims, freqs: Tensor, dropout=None) -> Tensor:
+    """x [s, b, h] -> [s, b, h]; pre-norm attention block then pre-norm SwiGLU MLP block.
+    dropout: None, or (probability, mask behind the out-projection, mask behind fc2) for hidden
+    dropout in front of the two residual adds, with the masks given."""
     s, b, _ = x.shape
     h1 = rmsnorm(x, p["ln1"], dims.eps)
     q, k, v = split_qkv(linear(h1, p["w_qkv"]), dims.nq, dims.nkv, dims.hd)
     q, k = rope(q, freqs), rope(k, freqs)
     a = causal_gqa_attention(q, k, v).reshape(s, b, dims.nq * dims.hd)
-    x = x + linear(a, p["w_proj"])
+    attn_out = linear(a, p["w_proj"])
+    if dropout is not None:
+        attn_out = dropout_with_mask(attn_out, dropout[1], dropout[0])
+    x = x + attn_out
     h2 = rmsnorm(x, p["ln2"], dims.eps)
-    return x + linear(swiglu(linear(h2, p["w_fc1"])), p["w_fc2"])
+    mlp_out = linear(swiglu(linear(h2, p["w_fc1"])), p["w_fc2"])
+    if dropout is not None:
+        mlp_out = dropout_with_mask(mlp_out, dropout[2], dropout[0])
+    return x + mlp_out
 
 
 def stack_forward(x: Tensor, layers: List[Dict[str, Tensor]], dims: LayerDims, freqs: Tensor) -> Tensor:

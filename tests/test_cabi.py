@@ -42,6 +42,10 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_rmsnorm_bwd(16, 16, 16, 16, 16, 16, 16, 4, 64, 64, 68, None) == -2  # stride not x8
     assert lib.kr_add_rows(16, 64, 16, 64, 16, 32, 4, 64, None) == -1             # output stride < width
     assert lib.kr_add_rows(16, 64, 16, 64, 16, 64, 4, 60, None) == -2             # width not x8
+    assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 8, 4, 64, 1.0, 1, 0, None) == -1   # p outside [0, 1)
+    assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 12, 4, 64, 0.1, 1, 0, None) == -1  # mask not 8-byte aligned
+    assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 8, 4, 60, 0.1, 1, 0, None) == -2   # width not x8
+    assert lib.kr_dropout_bwd(16, 32, 8, 16, 64, 4, 64, 1.25, None) == -1                # gradient stride < width
     assert lib.kr_gemm_workspace_bytes_shared(2, 1536, 4096, 4096, 0.3) <= lib.kr_gemm_workspace_bytes(2, 1536, 4096, 4096)
     assert lib.kr_gemm_bf16(0, 8, 8, 7, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -2
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1

@@ -228,6 +228,73 @@ def test_forward_epilogue_fusions_change_nothing(nnb, recompute, monkeypatch):
     assert calls["pairs"] == (0 if nnb > 1 else 2 * (2 if recompute else 1))   # (one nanobatch: no launch points)
 
 
+def _params_of(model):
+    return [{name: getattr(layer, attr).weight.detach().clone() for attr, name in PARAMS} for layer in model.layers]
+
+
+@pytest.mark.parametrize("recompute", [False, True])
+def test_hidden_dropout_matches_oracle_given_the_masks(recompute):
+    """Hidden dropout in front of the two residual adds (bias_dropout_add.py:24-45): with the masks the
+    operators drew handed to the oracle, output and every gradient agree; with recomputation the backward
+    pass draws the same masks again (the generator states are saved and replayed,
+    autograd_function.py:143-146, 263-266)."""
+    prob, dims = 0.25, R.LayerDims(512, 8, 8, 64, 1376)
+    cfg = LayerConfig(**C1, num_layers=1, num_nanobatches=1, params_dtype=torch.float32, backend="eager",
+                      hidden_dropout=prob, checkpoint_activations=recompute)
+    model = LayerStack(cfg, seed=1234)
+    gd = torch.Generator().manual_seed(5)
+    x, go = torch.randn(64, 2, 512, generator=gd), torch.randn(64, 2, 512, generator=gd)
+    torch.manual_seed(77)
+    y, dx = _run(model, x, go)
+    layer = model.layers[0]
+    masks = (prob, layer.self_attn_bda.last_mask.clone(), layer.mlp_bda.last_mask.clone())
+    for m in masks[1:]:
+        assert m.shape == x.shape and 0.70 < m.float().mean() < 0.80      # about 1 - p of the elements kept
+    assert not torch.equal(masks[1], masks[2])
+    xx = x.clone().requires_grad_(True)
+    leaves = {k: v.requires_grad_(True) for k, v in _params_of(model)[0].items()}
+    freqs = R.rope_table(64, dims.hd, dims.rope_base)
+    ry = R.layer_forward(xx, leaves, dims, freqs, dropout=masks)
+    ry.backward(go)
+    tol = 2e-4
+    assert (y - ry.detach()).abs().max() <= tol * ry.abs().max()
+    assert (dx - xx.grad).abs().max() <= tol * xx.grad.abs().max()
+    for attr, name in PARAMS:
+        g, rg = getattr(layer, attr).weight.grad, leaves[name].grad
+        assert (g - rg).abs().max() <= tol * rg.abs().max(), name
+    # without dropout the layer gives something else; the same seed gives the same step again
+    assert (y - R.layer_forward(x, _params_of(model)[0], dims, freqs)).abs().max() > 1e-2
+    for layer_param in model.parameters():
+        layer_param.grad = None
+    torch.manual_seed(77)
+    y2, dx2 = _run(model, x, go)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+
+
+def test_hidden_dropout_with_nanobatches_and_in_evaluation():
+    """Every nanobatch draws its own mask (so the result depends on the nanobatch count, as in the reference,
+    where each nanobatch's native_dropout call advances the generator); recomputation changes nothing; a layer
+    that is not training applies no dropout."""
+    base = dict(**C1, num_layers=1, params_dtype=torch.float32, backend="eager", hidden_dropout=0.3)
+    gd = torch.Generator().manual_seed(6)
+    x, go = torch.randn(32, 4, 512, generator=gd), torch.randn(32, 4, 512, generator=gd)
+    results = []
+    for recompute in (False, True):
+        model = LayerStack(LayerConfig(**base, num_nanobatches=2, checkpoint_activations=recompute), seed=1234)
+        torch.manual_seed(3)
+        y, dx = _run(model, x, go)
+        results.append((y, dx, [p.grad.clone() for p in model.parameters()]))
+    (y0, dx0, g0), (y1, dx1, g1) = results
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and all(torch.equal(a, b) for a, b in zip(g0, g1))
+    model = LayerStack(LayerConfig(**base, num_nanobatches=2), seed=1234)
+    for layer in model.layers:
+        layer.self_attn_bda.training = layer.mlp_bda.training = False
+    plain = LayerStack(LayerConfig(**{**base, "hidden_dropout": 0.0}, num_nanobatches=2), seed=1234)
+    ya, dxa = _run(model, x, go)
+    yb, dxb = _run(plain, x, go)
+    assert torch.equal(ya, yb) and torch.equal(dxa, dxb)
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
@@ -296,7 +363,9 @@ def test_host_error_paths():
     with pytest.raises(RuntimeError, match="executed by the partition engine"):
         m.layers[0](torch.randn(1))
     with pytest.raises(NotImplementedError):
-        LayerStack(LayerConfig(**C1, hidden_dropout=0.1, params_dtype=torch.float32, backend="eager"))
+        LayerStack(LayerConfig(**C1, attention_dropout=0.1, params_dtype=torch.float32, backend="eager"))
+    with pytest.raises(ValueError, match="outside"):
+        LayerStack(LayerConfig(**C1, hidden_dropout=1.5, params_dtype=torch.float32, backend="eager"))
     with pytest.raises(NotImplementedError):
         LayerStack(LayerConfig(**C1, add_bias_linear=True, params_dtype=torch.float32, backend="eager"))
     with pytest.raises(NotImplementedError):

@@ -33,6 +33,50 @@ def rnd(*shape, scale=1.0, seed=0):
 
 
 # ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("shape,p", [((64, 2, 512), 0.1), ((257, 3, 1024), 0.5), ((16, 8), 0.0), ((1000, 4096), 0.25)])
+def test_dropout_add_and_its_backward(be, shape, p):
+    """out = residual + dropout(x) (bias_dropout_add.py:15-45): with the mask the kernel wrote, the reference's
+    arithmetic gives the same bits (dropout output rounded to bf16, then the add); about 1 - p of the elements
+    are kept; the mask follows from PyTorch's CPU generator alone; the backward is dy * mask / (1 - p)."""
+    x, r = rnd(*shape, seed=3), rnd(*shape, seed=4)
+    torch.manual_seed(11)
+    out, mask = be.dropout_add(x, r, p)
+    assert mask.dtype == torch.uint8 and mask.shape == x.shape and int(mask.max()) <= 1
+    keep = mask.float().mean().item()
+    n = mask.numel()
+    assert abs(keep - (1 - p)) <= 5 * (p * (1 - p) / n) ** 0.5 + 1e-9
+    want = (r.float() + (x.float() * mask / (1 - p)).to(torch.bfloat16).float()).to(torch.bfloat16)
+    assert torch.equal(out, want)
+    torch.manual_seed(11)
+    out2, mask2 = be.dropout_add(x, r, p)
+    assert torch.equal(mask, mask2) and torch.equal(out, out2)
+    if p > 0:
+        torch.manual_seed(12)
+        assert not torch.equal(be.dropout_add(x, r, p)[1], mask)
+        # no structure along rows or between neighbours: the kept fraction of every column and of the
+        # products of neighbouring mask bits is what independent draws give
+        m2 = mask.view(-1, mask.shape[-1]).float()
+        if m2.shape[0] >= 64:
+            col = m2.mean(0)
+            assert (col - (1 - p)).abs().max() <= 6 * (p * (1 - p) / m2.shape[0]) ** 0.5
+        pair = (m2[:, 1:] * m2[:, :-1]).mean().item()
+        assert abs(pair - (1 - p) ** 2) <= 0.02
+    dy = rnd(*shape, seed=5)
+    dx = be.dropout_bwd(dy, mask, 1 / (1 - p))
+    assert torch.equal(dx, (dy.float() * mask / (1 - p)).to(torch.bfloat16))
+    # a strided nanobatch slice as operand and as output
+    if len(shape) == 3 and shape[1] >= 2:
+        big_x, big_r, big_o = rnd(shape[0], 2 * shape[1], shape[2], seed=6), rnd(shape[0], 2 * shape[1], shape[2], seed=7), \
+            torch.zeros(shape[0], 2 * shape[1], shape[2], device=DEV, dtype=torch.bfloat16)
+        xs, rs, os_ = big_x[:, :shape[1]], big_r[:, shape[1]:], big_o[:, shape[1]:]
+        torch.manual_seed(13)
+        o3, m3 = be.dropout_add(xs, rs, p, out=os_)
+        torch.manual_seed(13)
+        o4, m4 = be.dropout_add(xs.contiguous(), rs.contiguous(), p)
+        assert o3.data_ptr() == os_.data_ptr() and torch.equal(os_, o4) and torch.equal(m3, m4)
+        assert not big_o[:, :shape[1]].any()
+
+
 @pytest.mark.parametrize("n", [8, 1000 * 512, 4096 * 4096, 13 * 8 + 5])
 def test_add_is_exact(be, n):
     a, b = rnd(n, seed=1), rnd(n, seed=2)

@@ -77,6 +77,42 @@ def test_layer_matches_oracle(dims, s, b, layers, nnb):
     assert max(w[0] for w in worst) <= TOL
 
 
+@pytest.mark.parametrize("dims,s,b", [(R.LayerDims(1024, 8, 2, 128, 896), 384, 4), (R.LayerDims(512, 8, 8, 64, 1376), 256, 2)])
+def test_layer_with_hidden_dropout_matches_oracle_given_the_masks(dims, s, b):
+    """Hidden dropout in front of the two residual adds (bias_dropout_add.py:24-45; the reference's training
+    configuration uses 0.1): the masks the two operators drew go to the oracle, everything else as in
+    test_layer_matches_oracle.  With recomputation the backward pass draws the same masks again (generator
+    states saved and replayed, autograd_function.py:143-146, 263-266) and the step is bit-identical; with two
+    nanobatches, each drawing its own masks, the same seed still gives the same step."""
+    prob = 0.1
+    x, go = _inputs(s, b, dims.hidden)
+    model = _build(dims, 1, 1, hidden_dropout=prob)
+    torch.manual_seed(21)
+    y, dx, grads = _run(model, x, go)
+    layer = model.layers[0]
+    m1, m2 = layer.self_attn_bda.last_mask.float().cpu(), layer.mlp_bda.last_mask.float().cpu()
+    assert m1.shape == (s, b, dims.hidden) and 0.88 < m1.mean() < 0.92 and 0.88 < m2.mean() < 0.92
+    params = {n: getattr(layer, a).weight.detach().float().cpu().requires_grad_(True) for a, n in PARAMS}
+    xx = x.bfloat16().float().requires_grad_(True)
+    ry = R.layer_forward(xx, params, dims, R.rope_table(s, dims.hd, dims.rope_base), dropout=(prob, m1, m2))
+    ry.backward(go.bfloat16().float())
+    worst = [_rel(y, ry.detach()), _rel(dx, xx.grad)] + [_rel(grads[0][pi], params[n].grad) for pi, (_, n) in enumerate(PARAMS)]
+    print(f"hidden dropout {prob}: max-rel={max(w[0] for w in worst):.3e}")
+    assert max(w[0] for w in worst) <= TOL
+    recomputing = _build(dims, 1, 1, hidden_dropout=prob, checkpoint_activations=True)
+    torch.manual_seed(21)
+    y2, dx2, grads2 = _run(recomputing, x, go)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+    assert all(torch.equal(a, c) for a, c in zip(grads[0], grads2[0]))
+    two = _build(dims, 1, 2, hidden_dropout=prob)
+    torch.manual_seed(22)
+    ya, dxa, ga = _run(two, x, go)
+    torch.manual_seed(22)
+    yb, dxb, gb = _run(two, x, go)
+    assert torch.equal(ya, yb) and torch.equal(dxa, dxb) and all(torch.equal(a, c) for a, c in zip(ga[0], gb[0]))
+    assert not torch.equal(ya, y)
+
+
 def test_streams_recompute_and_schedule_do_not_change_results(fixtures_dir):
     dims = R.LayerDims(1024, 8, 2, 128, 896)
     x, go = _inputs(256, 4, dims.hidden)
