@@ -258,3 +258,18 @@ def test_layer_composition_equals_a_layer_of_library_routines():
                           _library_layer(_library_layer(x, p, dims), p2, dims), atol=1e-11)
     # the check has teeth: without the rotary embedding the library layer is somewhere else
     assert (_library_layer(x, p, dims, skip_rope=True) - y).abs().max() > 1e-3
+
+
+def test_dropout_with_mask_is_native_dropout_given_its_mask():
+    """The oracle's hidden dropout takes the mask as an input; for the mask the library routine drew, it is that
+    routine's output, and its gradient is native_dropout_backward (bias_dropout_add.py:24-32, 40-43)."""
+    torch.manual_seed(0)
+    x = torch.randn(64, 96, dtype=torch.float64, requires_grad=True)
+    out, mask = torch.ops.aten.native_dropout(x, 0.3, True)
+    mine = R.dropout_with_mask(x, mask, 0.3)
+    assert torch.allclose(mine, out, rtol=1e-15, atol=0) and 0.6 < mask.double().mean() < 0.8
+    g = torch.randn(64, 96, dtype=torch.float64)
+    (dx,) = torch.autograd.grad(mine, x, g)
+    assert torch.allclose(dx, torch.ops.aten.native_dropout_backward(g, mask, 1 / 0.7), rtol=1e-15, atol=0)
+    assert torch.equal(R.dropout_with_mask(x, torch.ones_like(mask), 0.0), x)
+
