@@ -35,7 +35,8 @@ The external pieces (flash-attention 2, Apex fused RoPE, cuBLASLt, Inductor outp
 in the reference tree and the reference holds no golden tensors for this path, so every
 function here is pinned by mathematics instead (tests/test_oracle.py): closed forms,
 invariants, brute-force loops on tiny inputs and PyTorch library routines
-(``F.scaled_dot_product_attention``, ``F.rms_norm``, ``F.silu``, ``torch.logsumexp``).
+(``F.scaled_dot_product_attention``, ``F.rms_norm``, ``F.silu``, ``torch.logsumexp``,
+``native_dropout`` for the dropout with a given mask).
 
 Everything runs in the dtype of its inputs (fp32 or fp64); bf16 comparisons first round the
 inputs to bf16 and then call this in fp32.
