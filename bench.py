@@ -615,6 +615,19 @@ def hbm_kernels(w, nnb, device, launches=50):
         _, mask = be.dropout_add(x, y, 0.1)
         report("dropout_add_kernel (p = 0.1)", t, t * h * (3 * 2 + 1), lambda: be.dropout_add(x, y, 0.1))
         report("dropout_bwd_kernel", t, t * h * (2 * 2 + 1), lambda: be.dropout_bwd(y, mask, 1 / 0.9))
+        # q / k layernorm of the QKV split (Qwen3-style layers; not part of the benchmark workloads): the
+        # fused buffer read and written once forward; backward the gradient and the saved input of the
+        # query and key heads read, their gradient rewritten in place
+        per = w["nq"] // w["nkv"]
+        if hd in (64, 128, 256):
+            fused = torch.randn(s_len, t // s_len, w["nkv"], per + 2, hd, device=device, dtype=bf)
+            dfused = torch.randn_like(fused)
+            gq, gk = torch.ones(hd, device=device, dtype=bf), torch.ones(hd, device=device, dtype=bf)
+            _, rs = be.qk_norm_fwd(fused, gq, gk, 1e-5)
+            report("qk_norm_fwd_kernel", t, 2 * fused.numel() * 2 + rs.numel() * 4,
+                   lambda: be.qk_norm_fwd(fused, gq, gk, 1e-5))
+            report("qk_norm_bwd_kernel + qk_norm_dgamma_kernel", t, 3 * t * heads * hd * 2 + rs.numel() * 4,
+                   lambda: be.qk_norm_bwd(dfused, fused, rs, gq, gk))
     return rows_out
 
 

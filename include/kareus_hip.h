@@ -210,6 +210,30 @@ int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const float* rstd,
                                int64_t dy_ld, int64_t x_ld, int64_t dres_ld, int64_t dx_ld,
                                void* stream);
 
+/* ---- Query / key layernorm of the QKV split -----------------------------------------------
+ * RMSNorm over the head dimension of every query head (weights gamma_q [hd]) and every key head
+ * (gamma_k [hd]) of a fused QKV projection output: replaces the q_layernorm / k_layernorm calls of
+ * QKVPostProcessOp (kareus/megatron/core/extensions/ops/qkv_postprocess.py:110-118 forward,
+ * :147-160 backward; each is an RMSNorm as in kareus/transformer_engine/pytorch/ops/basic/
+ * rmsnorm.py:165-273 with the head dimension as its width).
+ * mixed, out, dmixed: [tokens, ng, per + 2, hd] bf16, dense: per query heads, one key head and one
+ * value head per group.  rstd: [tokens, ng, per + 1] fp32, 1 / rms of every normalised head.
+ * kr_qk_norm_fwd: out = the buffer with its query and key heads normalised (y = bf16(x * rstd *
+ *   gamma)) and its value heads copied, so that out is again a fused buffer.  out must not alias
+ *   mixed (the backward needs the input).
+ * kr_qk_norm_bwd: rewrites the query and key heads of dmixed (the gradient w.r.t. out) in place
+ *   with the gradient w.r.t. mixed, dx = rstd * (dy*gamma - xhat * mean(dy*gamma*xhat)), leaves the
+ *   value heads alone, and writes dgamma_q, dgamma_k [hd] bf16 (sums of dy * xhat over all heads of
+ *   the kind, in fp32, in a fixed order).  workspace: kr_qk_norm_bwd_workspace_bytes() bytes of
+ *   device memory, 16-byte aligned.
+ * hd must be 64, 128 or 256 (KR_EUNSUPPORTED otherwise; the workspace query then returns 0).     */
+size_t kr_qk_norm_bwd_workspace_bytes(int64_t tokens, int ng, int per, int hd);
+int kr_qk_norm_fwd(const void* mixed, const void* gamma_q, const void* gamma_k, void* out, float* rstd,
+                   int64_t tokens, int ng, int per, int hd, float eps, void* stream);
+int kr_qk_norm_bwd(void* dmixed, const void* mixed, const float* rstd, const void* gamma_q,
+                   const void* gamma_k, void* dgamma_q, void* dgamma_k, void* workspace,
+                   int64_t tokens, int ng, int per, int hd, void* stream);
+
 /* ---- Rotary position embedding ---------------------------------------------------------
  * Replaces fused_rotary_positional_embedding.forward / backward (Apex), called from
  * kareus/apex/transformer/functional/fused_rope.py:27-35, 41-46.

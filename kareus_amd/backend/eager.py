@@ -173,6 +173,30 @@ class EagerBackend:
     def dropout_bwd(self, dy: Tensor, mask: Tensor, scale: float) -> Tensor:
         return (dy.float() * mask * scale).to(dy.dtype)
 
+    # RMSNorm over the head dimension of the query and key heads of a fused QKV buffer
+    # [s, b, groups, per + 2, hd]; value heads carried along (qkv_postprocess.py:115-118, 150-157).
+    @staticmethod
+    def _qk_weights(gamma_q: Tensor, gamma_k: Tensor, per: int) -> Tensor:
+        return torch.cat([gamma_q.float().expand(per, -1), gamma_k.float()[None]], dim=0)  # [per + 1, hd]
+
+    def qk_norm_fwd(self, mixed5: Tensor, gamma_q: Tensor, gamma_k: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+        per = mixed5.shape[3] - 2
+        x = mixed5[..., :per + 1, :].float()
+        rstd = torch.rsqrt(x.pow(2).mean(-1) + eps)
+        y = (x * rstd[..., None] * self._qk_weights(gamma_q, gamma_k, per)).to(mixed5.dtype)
+        return torch.cat([y, mixed5[..., per + 1:, :]], dim=3), rstd
+
+    def qk_norm_bwd(self, dmixed5: Tensor, mixed5: Tensor, rstd: Tensor, gamma_q: Tensor,
+                    gamma_k: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        per = mixed5.shape[3] - 2
+        xhat = mixed5[..., :per + 1, :].float() * rstd[..., None]
+        dy = dmixed5[..., :per + 1, :].float()
+        dyg = dy * self._qk_weights(gamma_q, gamma_k, per)
+        dx = rstd[..., None] * (dyg - xhat * (dyg * xhat).mean(-1, keepdim=True))
+        dgam = (dy * xhat).sum(dim=(0, 1, 2))                      # [per + 1, hd]
+        out = torch.cat([dx.to(dmixed5.dtype), dmixed5[..., per + 1:, :]], dim=3)
+        return out, dgam[:per].sum(0).to(gamma_q.dtype), dgam[per].to(gamma_k.dtype)
+
     # Causal GQA attention on [s, b, heads, hd] tensors; query head i reads KV head
     # i // (nq / nkv); lse = logsumexp of the scaled, masked scores, [b, nq, s] fp32
     # (kareus/flash_attn/flash_attn_interface.py:473-493).

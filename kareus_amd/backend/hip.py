@@ -58,6 +58,9 @@ _SIGNATURES = {
     "kr_dropout_add": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_void_p, _c_i64, _c_int,
                                 _c_float, ctypes.c_uint64, ctypes.c_uint64, _c_void_p]),
     "kr_dropout_bwd": (_c_int, [_c_void_p, _c_i64, _c_void_p, _c_void_p, _c_i64, _c_i64, _c_int, _c_float, _c_void_p]),
+    "kr_qk_norm_bwd_workspace_bytes": (_c_size_t, [_c_i64, _c_int, _c_int, _c_int]),
+    "kr_qk_norm_fwd": (_c_int, [_c_void_p] * 5 + [_c_i64, _c_int, _c_int, _c_int, _c_float, _c_void_p]),
+    "kr_qk_norm_bwd": (_c_int, [_c_void_p] * 8 + [_c_i64, _c_int, _c_int, _c_int, _c_void_p]),
     "kr_embedding_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_embedding_bwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_i64, _c_i64, _c_void_p]),
     "kr_cross_entropy_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_i64, _c_int, _c_i64, _c_void_p]),
@@ -633,6 +636,55 @@ class HipBackend:
         self._check(self.lib.kr_dropout_bwd(d2.data_ptr(), d2.stride(0), mask.data_ptr(), dx.data_ptr(), cols, rows, cols,
                                             float(scale), self._stream()), "kr_dropout_bwd")
         return dx
+
+    # -- query / key layernorm of the QKV split ----------------------------------------------
+    def _fused5(self, name: str, t: Tensor) -> Tuple[int, int, int, int]:
+        self._dev(t)
+        self._bf16(t)
+        if t.dim() != 5 or not t.is_contiguous() or t.shape[3] < 3:
+            raise RuntimeError(f"{name}: needs a dense fused buffer [s, b, groups, per + 2, hd], got "
+                               f"{tuple(t.shape)} with strides {t.stride()}")
+        s, b, ng, slots, hd = t.shape
+        return s * b, ng, slots - 2, hd
+
+    def _qk_gammas(self, name: str, hd: int, gamma_q: Tensor, gamma_k: Tensor) -> None:
+        self._dev(gamma_q, gamma_k)
+        self._bf16(gamma_q, gamma_k)
+        for g in (gamma_q, gamma_k):
+            if g.shape != (hd,) or not g.is_contiguous():
+                raise RuntimeError(f"{name}: a weight vector has shape {tuple(g.shape)}, the head dimension is {hd}")
+
+    def qk_norm_fwd(self, mixed5: Tensor, gamma_q: Tensor, gamma_k: Tensor, eps: float) -> Tuple[Tensor, Tensor]:
+        """RMSNorm over the head dimension of the query and key heads of a fused QKV buffer
+        ``[s, b, groups, per + 2, hd]``; the value heads are copied.  Returns the new fused buffer and
+        ``rstd [s, b, groups, per + 1]`` (qkv_postprocess.py:115-118)."""
+        tokens, ng, per, hd = self._fused5("qk_norm_fwd", mixed5)
+        self._qk_gammas("qk_norm_fwd", hd, gamma_q, gamma_k)
+        out = torch.empty_like(mixed5)
+        rstd = torch.empty(mixed5.shape[:3] + (per + 1,), dtype=torch.float32, device=mixed5.device)
+        self._check(self.lib.kr_qk_norm_fwd(mixed5.data_ptr(), gamma_q.data_ptr(), gamma_k.data_ptr(), out.data_ptr(),
+                                            rstd.data_ptr(), tokens, ng, per, hd, float(eps), self._stream()),
+                    "kr_qk_norm_fwd")
+        return out, rstd
+
+    def qk_norm_bwd(self, dmixed5: Tensor, mixed5: Tensor, rstd: Tensor, gamma_q: Tensor,
+                    gamma_k: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        """The backward of :meth:`qk_norm_fwd`, in place on the query and key heads of ``dmixed5``
+        (qkv_postprocess.py:150-157).  Returns ``(dmixed5, dgamma_q, dgamma_k)``."""
+        tokens, ng, per, hd = self._fused5("qk_norm_bwd", dmixed5)
+        if self._fused5("qk_norm_bwd", mixed5) != (tokens, ng, per, hd):
+            raise RuntimeError(f"qk_norm_bwd: gradient {tuple(dmixed5.shape)} and input {tuple(mixed5.shape)} differ")
+        self._qk_gammas("qk_norm_bwd", hd, gamma_q, gamma_k)
+        self._dev(rstd)
+        if rstd.dtype != torch.float32 or rstd.shape != mixed5.shape[:3] + (per + 1,) or not rstd.is_contiguous():
+            raise RuntimeError("qk_norm_bwd: rstd is not the fp32 [s, b, groups, per + 1] tensor of the forward")
+        dgq, dgk = torch.empty_like(gamma_q), torch.empty_like(gamma_k)
+        nbytes = self.lib.kr_qk_norm_bwd_workspace_bytes(tokens, ng, per, hd)
+        ws = self._workspace(max(nbytes, 16), mixed5.device)
+        self._check(self.lib.kr_qk_norm_bwd(dmixed5.data_ptr(), mixed5.data_ptr(), rstd.data_ptr(), gamma_q.data_ptr(),
+                                            gamma_k.data_ptr(), dgq.data_ptr(), dgk.data_ptr(), ws.data_ptr(),
+                                            tokens, ng, per, hd, self._stream()), "kr_qk_norm_bwd")
+        return dmixed5, dgq, dgk
 
     @staticmethod
     def _leading_rows(t: Tensor) -> Tensor:

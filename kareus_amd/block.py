@@ -25,6 +25,7 @@ from .operators import (
     NoOpAllReduce,
     PartitionableRMSNorm,
     QKVPostProcessOp,
+    RMSNorm,
     ResidualForkOp,
     RotaryEmbeddingOp,
     TEColumnParallelLinearOp,
@@ -90,6 +91,9 @@ class LayerConfig:
     hidden_dropout: float = 0.0
     attention_dropout: float = 0.0
     add_bias_linear: bool = False
+    # an RMSNorm over the head dimension of every query head and of every key head, between the QKV split
+    # and the rotary embedding (Qwen3-style models)
+    qk_layernorm: bool = False
     # Filled in by the driver / the training loop:
     kareus_scheduler: Optional[Any] = None
     nanobatch_streams: Optional[List[Any]] = field(default=None, repr=False)
@@ -197,7 +201,10 @@ class DecoderLayer(torch.nn.Module):
         self.attn_residual_fork = ResidualForkOp(backend=be)
         self.input_layernorm = PartitionableRMSNorm(c.hidden_size, c.layernorm_epsilon, device=device, dtype=dt, backend=be)
         self.linear_qkv = TEColumnParallelLinearOp(c.hidden_size, c.qkv_width, skip_bias_add=False, **lin)
-        self.qkv_postprocess = QKVPostProcessOp(c.num_query_groups, c.num_attention_heads, c.kv_channels)
+        head_norm = (lambda: RMSNorm(c.kv_channels, c.layernorm_epsilon, device=device, dtype=dt, backend=be)
+                     ) if c.qk_layernorm else (lambda: None)
+        self.qkv_postprocess = QKVPostProcessOp(c.num_query_groups, c.num_attention_heads, c.kv_channels,
+                                                q_layernorm=head_norm(), k_layernorm=head_norm(), backend=be)
         self.rotary = RotaryEmbeddingOp(config=c, backend=be)
         self.core_attention = TEDotProductAttentionOp(config=c, layer_number=layer_number, backend=be,
                                                       attention_dropout=c.attention_dropout)

@@ -14,6 +14,13 @@ outputs remember the fused buffer they are views of (``_kr_fused5``), which lets
 the rotary operator rotate q and k in place with one launch, and lets ``merge``
 return the attention backward's fused gradient buffer as is.  Pass
 ``grouped_query_view=False`` to get the reference's dense 4-D query instead.
+
+With ``q_layernorm`` and ``k_layernorm`` (Qwen3-style models: an RMSNorm over the head
+dimension of every query head and one over every key head, qkv_postprocess.py:115-118,
+backward :150-157) one kernel writes a second fused buffer with the query and key heads
+normalised and the value heads copied, and the three outputs are views of that buffer, so
+everything downstream works as without the norms; the backward rewrites the query and key
+heads of the merged gradient in place and returns the two weight gradients, query first.
 """
 
 from __future__ import annotations
@@ -22,6 +29,7 @@ from typing import List
 
 import torch
 
+from ..backend import get_backend
 from ..partitions.op_context import BasicOperation
 from ..partitions.tensor_graph import Channel, PartitionableOperator
 
@@ -31,10 +39,22 @@ class QKVPostProcessOp(BasicOperation, PartitionableOperator):
 
     def __init__(self, num_query_groups_per_partition: int, num_attention_heads_per_partition: int,
                  hidden_size_per_attention_head: int, q_layernorm=None, k_layernorm=None,
-                 grouped_query_view: bool = True) -> None:
+                 grouped_query_view: bool = True, backend="hip") -> None:
         super().__init__()
-        if q_layernorm is not None or k_layernorm is not None:
-            raise NotImplementedError("q/k layernorm is not used by the Llama-style layer")
+        if (q_layernorm is None) != (k_layernorm is None):
+            raise NotImplementedError("q_layernorm and k_layernorm come as a pair (qk_layernorm) or not at all")
+        for norm in (q_layernorm, k_layernorm):
+            if norm is None:
+                continue
+            weight = getattr(norm, "weight", None)
+            if weight is None or tuple(weight.shape) != (hidden_size_per_attention_head,) or not hasattr(norm, "eps"):
+                raise ValueError("q/k layernorm must be an RMSNorm over the head dimension "
+                                 f"({hidden_size_per_attention_head} channels) with a weight and an eps")
+        if q_layernorm is not None and float(q_layernorm.eps) != float(k_layernorm.eps):
+            raise ValueError("q_layernorm and k_layernorm must share one epsilon")
+        self.q_layernorm = q_layernorm   # (registered in this order: the weight gradients come back query first)
+        self.k_layernorm = k_layernorm
+        self._backend_name = backend
         if num_attention_heads_per_partition % num_query_groups_per_partition:
             raise ValueError("query heads must be a multiple of KV groups")
         self.ng = num_query_groups_per_partition
@@ -71,9 +91,32 @@ class QKVPostProcessOp(BasicOperation, PartitionableOperator):
 
     def fuser_forward(self, basic_op_ctxs, input_, *, basic_op_extra_inputs, basic_op_prev_ops,
                       basic_op_next_ops, basic_op_kwargs):
-        q, k, v = self.split(input_)
+        if self.q_layernorm is None:
+            q, k, v = self.split(input_)
+            return q, [(k, v)]
+        ng, hd, per = self.ng, self.hd, self.nq // self.ng
+        if input_.shape[-1] != ng * (per + 2) * hd:
+            raise ValueError(f"fused QKV width {input_.shape[-1]} != ng*(nq/ng+2)*hd = {ng * (per + 2) * hd}")
+        mixed = input_.contiguous()
+        be = get_backend(self._backend_name)
+        # (the leading dimensions, [s, b] in the layer, are all tokens to the norm)
+        normed5, rstd = be.qk_norm_fwd(mixed.view(-1, 1, ng, per + 2, hd), self.q_layernorm.weight.detach(),
+                                       self.k_layernorm.weight.detach(), float(self.q_layernorm.eps))
+        ctx = basic_op_ctxs[0]
+        if ctx.requires_grad:
+            ctx.save_for_backward(mixed, rstd)
+        q, k, v = self.split(normed5.view(mixed.shape))
         return q, [(k, v)]
 
     def fuser_backward(self, basic_op_ctxs, grad_output, *, basic_op_grad_extra_outputs):
         gk, gv = basic_op_grad_extra_outputs[0]
-        return self.merge(grad_output, gk, gv), [()], [()]
+        merged = self.merge(grad_output, gk, gv)
+        if self.q_layernorm is None:
+            return merged, [()], [()]
+        mixed, rstd = basic_op_ctxs[0].saved_tensors
+        ng, hd, per = self.ng, self.hd, self.nq // self.ng
+        merged = merged.contiguous()
+        be = get_backend(self._backend_name)
+        dmixed5, dgq, dgk = be.qk_norm_bwd(merged.view(-1, 1, ng, per + 2, hd), mixed.view(-1, 1, ng, per + 2, hd), rstd,
+                                           self.q_layernorm.weight.detach(), self.k_layernorm.weight.detach())
+        return dmixed5.view(mixed.shape), [(dgq, dgk)], [()]

@@ -10,6 +10,10 @@ reference reaches through third-party CUDA libraries, function by function:
                  stated separately in ``rmsnorm_bwd_formula`` so tests can cross-check the two
   linear         kareus/transformer_engine/pytorch/ops/basic/basic_linear.py:571-582 (y = x W^T)
   split_qkv      kareus/megatron/core/extensions/ops/qkv_postprocess.py:84-109
+  q / k norm     kareus/megatron/core/extensions/ops/qkv_postprocess.py:115-118: ``rmsnorm`` over the
+                 head dimension of every query head and every key head (optional; pinned by
+                 its invariances: the layer's output does not change when one head's query
+                 or key rows of the QKV weight are scaled, and does when value rows are)
   rope           kareus/megatron/core/models/common/embedding/rope_utils.py:147-182 with the
                  table of 3rdparty/Megatron-LM/megatron/core/models/common/embeddings/
                  rotary_pos_embedding.py:76-78,129,161,167
@@ -172,10 +176,14 @@ def dropout_with_mask(x: Tensor, mask: Tensor, prob: float) -> Tensor:
 def layer_forward(x: Tensor, p: Dict[str, Tensor], dims: LayerDims, freqs: Tensor, dropout=None) -> Tensor:
     """x [s, b, h] -> [s, b, h]; pre-norm attention block then pre-norm SwiGLU MLP block.
     dropout: None, or (probability, mask behind the out-projection, mask behind fc2) for hidden
-    dropout in front of the two residual adds, with the masks given."""
+    dropout in front of the two residual adds, with the masks given.
+    p["q_norm"], p["k_norm"] ([hd] each), when present: the q / k layernorm of the QKV split
+    (kareus/megatron/core/extensions/ops/qkv_postprocess.py:115-118)."""
     s, b, _ = x.shape
     h1 = rmsnorm(x, p["ln1"], dims.eps)
     q, k, v = split_qkv(linear(h1, p["w_qkv"]), dims.nq, dims.nkv, dims.hd)
+    if "q_norm" in p:  # Qwen3-style: RMSNorm over the head dimension of every query / key head, then rotary
+        q, k = rmsnorm(q, p["q_norm"], dims.eps), rmsnorm(k, p["k_norm"], dims.eps)
     q, k = rope(q, freqs), rope(k, freqs)
     a = causal_gqa_attention(q, k, v).reshape(s, b, dims.nq * dims.hd)
     attn_out = linear(a, p["w_proj"])

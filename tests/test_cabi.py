@@ -46,6 +46,15 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 12, 4, 64, 0.1, 1, 0, None) == -1  # mask not 8-byte aligned
     assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 8, 4, 60, 0.1, 1, 0, None) == -2   # width not x8
     assert lib.kr_dropout_bwd(16, 32, 8, 16, 64, 4, 64, 1.25, None) == -1                # gradient stride < width
+    assert lib.kr_qk_norm_fwd(16, 16, 16, 16, 16, 4, 2, 4, 96, 1e-5, None) == -2         # head dimension not 64/128/256
+    assert lib.kr_qk_norm_fwd(16, 16, 24, 16, 16, 4, 2, 4, 128, 1e-5, None) == -1        # misaligned weight
+    assert lib.kr_qk_norm_fwd(16, 16, 16, 16, 16, 4, 2, 0, 128, 1e-5, None) == -1        # no query head in a group
+    assert lib.kr_qk_norm_bwd(16, 16, 16, 16, 16, 16, 16, None, 4, 2, 4, 128, None) == -1  # no workspace
+    assert lib.kr_qk_norm_bwd_workspace_bytes(4, 2, 4, 96) == 0
+    # 8192 tokens x 2 groups x 6 heads of 128 channels: 16 rows per workgroup, capped at 1024 workgroups, each
+    # leaving 2 x 128 fp32 partial sums
+    assert lib.kr_qk_norm_bwd_workspace_bytes(8192, 2, 4, 128) == 1024 * 2 * 128 * 4
+    assert lib.kr_qk_norm_bwd_workspace_bytes(16, 1, 2, 64) == 2 * 2 * 64 * 4              # 64 rows, 32 a workgroup
     assert lib.kr_gemm_workspace_bytes_shared(2, 1536, 4096, 4096, 0.3) <= lib.kr_gemm_workspace_bytes(2, 1536, 4096, 4096)
     assert lib.kr_gemm_bf16(0, 8, 8, 7, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -2
     assert lib.kr_gemm_bf16(9, 8, 8, 8, 16, 8, 16, 8, 16, 8, 0, None, 0, None) == -1

@@ -295,6 +295,45 @@ def test_hidden_dropout_with_nanobatches_and_in_evaluation():
     assert torch.equal(ya, yb) and torch.equal(dxa, dxb)
 
 
+@pytest.mark.parametrize("nnb,recompute,grouped", [(1, False, True), (2, True, True), (2, False, False)])
+def test_query_and_key_norms_match_oracle(nnb, recompute, grouped):
+    """The q / k layernorm of the QKV split (Qwen3-style layers; qkv_postprocess.py:115-118 forward,
+    :150-157 backward, weight gradients query first): output, input gradient and every parameter's gradient,
+    the two head-norm weights included, against the oracle; the nanobatches' weight gradients add up."""
+    dims = R.LayerDims(hidden=64, nq=6, nkv=2, hd=16, ffn=40)
+    cfg = LayerConfig(hidden_size=64, num_attention_heads=6, num_query_groups=2, kv_channels=16, ffn_hidden_size=40,
+                      num_layers=2, num_nanobatches=nnb, params_dtype=torch.float32, backend="eager",
+                      qk_layernorm=True, checkpoint_activations=recompute)
+    model = LayerStack(cfg, seed=1234)
+    gd = torch.Generator().manual_seed(8)
+    for layer in model.layers:
+        layer.qkv_postprocess.grouped_query_view = grouped
+        for norm in (layer.qkv_postprocess.q_layernorm, layer.qkv_postprocess.k_layernorm):
+            with torch.no_grad():
+                norm.weight.copy_(1 + 0.3 * torch.randn(16, generator=gd))
+    names = [n for n, _ in model.named_parameters() if "qkv_postprocess" in n]
+    assert [n.split("qkv_postprocess.")[1] for n in names[:2]] == ["q_layernorm.weight", "k_layernorm.weight"]
+    x, go = torch.randn(24, 4, 64, generator=gd), torch.randn(24, 4, 64, generator=gd)
+    y, dx = _run(model, x, go)
+    params = []
+    for layer, plain in zip(model.layers, _params_of(model)):
+        post = layer.qkv_postprocess
+        params.append({**plain, "q_norm": post.q_layernorm.weight.detach().clone(),
+                       "k_norm": post.k_layernorm.weight.detach().clone()})
+    ry, rdx, rgrads = R.stack_forward_backward(x, params, dims, go)
+    tol = 2e-4
+    assert (y - ry).abs().max() <= tol * ry.abs().max()
+    assert (dx - rdx).abs().max() <= tol * rdx.abs().max()
+    for layer, rg in zip(model.layers, rgrads):
+        post = layer.qkv_postprocess
+        got = {name: getattr(layer, attr).weight.grad for attr, name in PARAMS}
+        got.update(q_norm=post.q_layernorm.weight.grad, k_norm=post.k_layernorm.weight.grad)
+        for name, g in got.items():
+            assert (g - rg[name]).abs().max() <= tol * rg[name].abs().max(), name
+    # the norms matter: the oracle without them is somewhere else
+    assert (R.stack_forward(x, _params_of(model), dims, R.rope_table(24, 16, dims.rope_base)) - ry).abs().max() > 1e-2
+
+
 def test_config1_exact_shape_two_layers():
     x, go, ref = _oracle(layers=2, s=256, b=2)
     cfg = LayerConfig(**C1, num_layers=2, num_nanobatches=2, params_dtype=torch.float32, backend="eager")
@@ -368,6 +407,10 @@ def test_host_error_paths():
         LayerStack(LayerConfig(**C1, hidden_dropout=1.5, params_dtype=torch.float32, backend="eager"))
     with pytest.raises(NotImplementedError):
         LayerStack(LayerConfig(**C1, add_bias_linear=True, params_dtype=torch.float32, backend="eager"))
+    with pytest.raises(NotImplementedError, match="come as a pair"):
+        QKVPostProcessOp(2, 6, 16, q_layernorm=torch.nn.LayerNorm(16))
+    with pytest.raises(ValueError, match="over the head dimension"):
+        QKVPostProcessOp(2, 6, 16, q_layernorm=torch.nn.LayerNorm(32), k_layernorm=torch.nn.LayerNorm(32))
     with pytest.raises(NotImplementedError):
         NoOpAllReduce(world_size=2)
     with pytest.raises(ValueError, match="unknown backend"):

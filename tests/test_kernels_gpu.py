@@ -77,6 +77,44 @@ def test_dropout_add_and_its_backward(be, shape, p):
         assert not big_o[:, :shape[1]].any()
 
 
+@pytest.mark.parametrize("s,b,ng,per,hd", [(64, 2, 2, 4, 128), (333, 1, 1, 1, 64), (50, 3, 3, 2, 256),
+                                           (4096, 2, 2, 4, 128)])
+def test_query_key_norm_and_its_backward(be, s, b, ng, per, hd):
+    """The q / k layernorm of the QKV split on the fused buffer (qkv_postprocess.py:115-118, 150-157): query and
+    key heads against the oracle's RMSNorm over the head dimension and its backward formula, value heads carried
+    along bit for bit, weight gradients summed over all heads of the kind.  (The last case has more rows than
+    the launch has row slots, so every workgroup walks several.)"""
+    eps = 1e-5
+    mixed = rnd(s, b, ng, per + 2, hd, seed=1)
+    gq = (1 + 0.3 * torch.randn(hd, generator=torch.Generator().manual_seed(2))).to(DEV, torch.bfloat16)
+    gk = (1 + 0.3 * torch.randn(hd, generator=torch.Generator().manual_seed(3))).to(DEV, torch.bfloat16)
+    before = mixed.clone()
+    out, rstd = be.qk_norm_fwd(mixed, gq, gk, eps)
+    assert torch.equal(mixed, before) and out.shape == mixed.shape and rstd.shape == (s, b, ng, per + 1)
+    xq, xk = mixed[..., :per, :].float(), mixed[..., per, :].float()
+    assert rel(out[..., :per, :], R.rmsnorm(xq, gq.float(), eps)) <= TOL
+    assert rel(out[..., per, :], R.rmsnorm(xk, gk.float(), eps)) <= TOL
+    assert torch.equal(out[..., per + 1, :], mixed[..., per + 1, :])
+    assert rel(rstd, torch.rsqrt(mixed[..., :per + 1, :].float().pow(2).mean(-1) + eps)) <= 1e-5
+    dy = rnd(s, b, ng, per + 2, hd, seed=4)
+    rdq, rdgq = R.rmsnorm_bwd_formula(dy[..., :per, :].float(), xq, gq.float(), eps)
+    rdk, rdgk = R.rmsnorm_bwd_formula(dy[..., per, :].float(), xk, gk.float(), eps)
+    dvalue = dy[..., per + 1, :].clone()
+    dx, dgq, dgk = be.qk_norm_bwd(dy, mixed, rstd, gq, gk)
+    assert dx.data_ptr() == dy.data_ptr()                                   # in place
+    assert rel(dx[..., :per, :], rdq) <= TOL and rel(dx[..., per, :], rdk) <= TOL
+    assert torch.equal(dx[..., per + 1, :], dvalue)
+    assert rel(dgq, rdgq) <= TOL and rel(dgk, rdgk) <= TOL
+    # the same call again gives the same bits (fixed summation order, no atomics)
+    dy2 = rnd(s, b, ng, per + 2, hd, seed=4)
+    dx2, dgq2, dgk2 = be.qk_norm_bwd(dy2, mixed, rstd, gq, gk)
+    assert torch.equal(dx2, dx) and torch.equal(dgq2, dgq) and torch.equal(dgk2, dgk)
+    with pytest.raises(RuntimeError, match="dense fused buffer"):
+        be.qk_norm_fwd(mixed[:, :, :, :per + 1], gq, gk, eps)
+    with pytest.raises(RuntimeError, match="head dimension"):
+        be.qk_norm_fwd(mixed, gq[: hd // 2], gk, eps)
+
+
 @pytest.mark.parametrize("n", [8, 1000 * 512, 4096 * 4096, 13 * 8 + 5])
 def test_add_is_exact(be, n):
     a, b = rnd(n, seed=1), rnd(n, seed=2)

@@ -113,6 +113,52 @@ def test_layer_with_hidden_dropout_matches_oracle_given_the_masks(dims, s, b):
     assert not torch.equal(ya, y)
 
 
+@pytest.mark.parametrize("dims,s,b,nnb", [
+    (R.LayerDims(2048, 4, 2, 128, 1536), 384, 4, 1),   # Qwen3-1.7B widths (16 q / 8 kv heads of 128) at TP=4
+    (R.LayerDims(2048, 4, 2, 128, 1536), 384, 4, 2),
+    (R.LayerDims(512, 8, 8, 64, 1376), 200, 2, 2),     # one query head per group, 64 channels, ragged length
+])
+def test_layer_with_query_and_key_norms_matches_oracle(dims, s, b, nnb):
+    """Qwen3-style layers (qk_layernorm): an RMSNorm over the head dimension of every query head and of every
+    key head between the QKV split and the rotary embedding (qkv_postprocess.py:115-118, 150-157).  Output, input
+    gradient and all gradients, the two head-norm weights' included, against the oracle; recomputation and the
+    nanobatch streams change no bit."""
+    x, go = _inputs(s, b, dims.hidden)
+    model = _build(dims, 2, nnb, qk_layernorm=True)
+    gen = torch.Generator().manual_seed(9)
+    heads = [("q_layernorm", "q_norm"), ("k_layernorm", "k_norm")]
+    for layer in model.layers:
+        for attr, _ in heads:
+            with torch.no_grad():
+                getattr(layer.qkv_postprocess, attr).weight.copy_(1 + 0.3 * torch.randn(dims.hd, generator=gen))
+
+    def run(m):
+        y, dx, grads = _run(m, x, go)
+        extra = [[getattr(layer.qkv_postprocess, a).weight.grad.clone() for a, _ in heads] for layer in m.layers]
+        return y, dx, grads, extra
+
+    y, dx, grads, extra = run(model)
+    params = [{**{n: getattr(layer, a).weight.detach().float().cpu() for a, n in PARAMS},
+               **{n: getattr(layer.qkv_postprocess, a).weight.detach().float().cpu() for a, n in heads}}
+              for layer in model.layers]
+    ry, rdx, rgrads = R.stack_forward_backward(x.bfloat16().float(), params, dims, go.bfloat16().float())
+    worst = [_rel(y, ry), _rel(dx, rdx)]
+    for li in range(2):
+        worst += [_rel(grads[li][pi], rgrads[li][name]) for pi, (_, name) in enumerate(PARAMS)]
+        worst += [_rel(extra[li][pi], rgrads[li][name]) for pi, (_, name) in enumerate(heads)]
+    print(f"qk_layernorm nnb={nnb} max-rel={max(w[0] for w in worst):.3e} max-abs={max(w[1] for w in worst):.3e}")
+    assert max(w[0] for w in worst) <= TOL
+    plain = [{n: t for n, t in p.items() if n not in ("q_norm", "k_norm")} for p in params]
+    without = R.stack_forward(x.bfloat16().float(), plain, dims, R.rope_table(s, dims.hd, dims.rope_base))
+    assert _rel(without, ry)[0] > 2 * TOL       # the norms matter at this tolerance
+    other = _build(dims, 2, nnb, qk_layernorm=True, checkpoint_activations=True, use_streams=False)
+    other.load_state_dict(model.state_dict())
+    y2, dx2, grads2, extra2 = run(other)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+    for la, lb in zip(grads + extra, grads2 + extra2):
+        assert all(torch.equal(a, c) for a, c in zip(la, lb))
+
+
 def test_streams_recompute_and_schedule_do_not_change_results(fixtures_dir):
     dims = R.LayerDims(1024, 8, 2, 128, 896)
     x, go = _inputs(256, 4, dims.hidden)

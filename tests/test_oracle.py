@@ -214,6 +214,8 @@ def _library_layer(x, p, dims, skip_rope=False):
     h1 = F.rms_norm(x, (h,), p["ln1"], dims.eps)
     mixed = F.linear(h1, p["w_qkv"]).view(s, b, dims.nkv, per + 2, hd)
     q, k, v = mixed[:, :, :, :per].reshape(s, b, dims.nq, hd), mixed[:, :, :, per], mixed[:, :, :, per + 1]
+    if "q_norm" in p:
+        q, k = F.rms_norm(q, (hd,), p["q_norm"], dims.eps), F.rms_norm(k, (hd,), p["k_norm"], dims.eps)
     if not skip_rope:
         # halves layout: channel i pairs with i + hd/2; rotating the pair by angle a_i is the
         # complex product (t_i + j t_{i+hd/2}) * exp(j a_i)
@@ -258,6 +260,44 @@ def test_layer_composition_equals_a_layer_of_library_routines():
                           _library_layer(_library_layer(x, p, dims), p2, dims), atol=1e-11)
     # the check has teeth: without the rotary embedding the library layer is somewhere else
     assert (_library_layer(x, p, dims, skip_rope=True) - y).abs().max() > 1e-3
+
+
+def test_layer_with_query_and_key_norms():
+    """The q / k layernorm of the QKV split (qkv_postprocess.py:115-118): an RMSNorm per head over the head
+    dimension, on queries and keys, in front of the rotary embedding, not on values.  Pinned by the library
+    routine in the library layer and by what the norm makes invariant: scaling the QKV weight rows of ONE query
+    head, or of one key head, leaves the layer's output alone (a norm over all heads together, or none, would
+    not), scaling a value head's rows does not."""
+    dims = R.LayerDims(hidden=48, nq=6, nkv=2, hd=16, ffn=40, eps=1e-12)
+    gen = torch.Generator().manual_seed(11)
+    p = R.init_layer_params(dims, gen, std=0.3, dtype=D)
+    p["q_norm"] = 1 + 0.3 * torch.randn(16, generator=gen, dtype=D)
+    p["k_norm"] = 1 + 0.3 * torch.randn(16, generator=gen, dtype=D)
+    x = torch.randn(12, 3, 48, generator=gen, dtype=D)
+    go = torch.randn(12, 3, 48, generator=gen, dtype=D)
+    y, dx, grads = R.stack_forward_backward(x, [p], dims, go)
+    xl = x.clone().requires_grad_(True)
+    pl = {k: t.clone().requires_grad_(True) for k, t in p.items()}
+    yl = _library_layer(xl, pl, dims)
+    yl.backward(go)
+    assert torch.allclose(yl, y, atol=1e-11) and torch.allclose(xl.grad, dx, atol=1e-10)
+    for name in p:
+        assert torch.allclose(pl[name].grad, grads[0][name], atol=1e-9), name
+    plain = {k: t for k, t in p.items() if k not in ("q_norm", "k_norm")}
+    f = R.rope_table(12, dims.hd, dims.rope_base, dtype=D)
+    assert (R.layer_forward(x, plain, dims, f) - y).abs().max() > 1e-3     # the norms do something
+    per, hd = dims.nq // dims.nkv, dims.hd
+
+    def scaled(slot, group=1, factor=3.0):
+        w = p["w_qkv"].clone().view(dims.nkv, per + 2, hd, dims.hidden)
+        w[group, slot] *= factor
+        return {**p, "w_qkv": w.view(-1, dims.hidden)}
+
+    for slot in (0, per - 1, per):                     # a query head, another, the group's key head
+        assert torch.allclose(R.layer_forward(x, scaled(slot), dims, f), y, atol=1e-9), slot
+        assert (R.layer_forward(x, {**plain, "w_qkv": scaled(slot)["w_qkv"]}, dims, f)
+                - R.layer_forward(x, plain, dims, f)).abs().max() > 1e-3
+    assert (R.layer_forward(x, scaled(per + 1), dims, f) - y).abs().max() > 1e-3   # values are not normalised
 
 
 def test_dropout_with_mask_is_native_dropout_given_its_mask():
