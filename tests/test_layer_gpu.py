@@ -388,6 +388,13 @@ def test_full_size_properties_config5():
     _size_independent_properties(C5, 4, 8192, 2, [1, 2], cut=6144)
 
 
+def test_full_size_properties_qwen3_shard_with_head_norms():
+    """The reference's Qwen3-1.7B configuration (h2048, 16q/8kv heads of 128, ffn 6144, qk_layernorm; seq 4096)
+    as a TP=4 shard at MBS 4, nanobatch counts 1, 2, 4."""
+    _size_independent_properties(R.LayerDims(2048, 4, 2, 128, 1536), 1, 4096, 4, [1, 2, 4], cut=3072,
+                                 qk_layernorm=True)
+
+
 def test_nanobatch_streams_do_not_share_a_hardware_queue():
     """Streams handed to the nanobatches must overlap for real: a short kernel on one finishes
     while a spinning kernel occupies the other."""
