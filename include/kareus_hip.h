@@ -220,7 +220,7 @@ int kr_rmsnorm_bwd_add_noalloc(const void* dy, const void* x, const float* rstd,
  * value head per group.  rstd: [tokens, ng, per + 1] fp32, 1 / rms of every normalised head.
  * kr_qk_norm_fwd: out = the buffer with its query and key heads normalised (y = bf16(x * rstd *
  *   gamma)) and its value heads copied, so that out is again a fused buffer.  out must not alias
- *   mixed (the backward needs the input).
+ *   mixed (the backward needs the input; out == mixed returns KR_EINVAL).
  * kr_qk_norm_bwd: rewrites the query and key heads of dmixed (the gradient w.r.t. out) in place
  *   with the gradient w.r.t. mixed, dx = rstd * (dy*gamma - xhat * mean(dy*gamma*xhat)), leaves the
  *   value heads alone, and writes dgamma_q, dgamma_k [hd] bf16 (sums of dy * xhat over all heads of

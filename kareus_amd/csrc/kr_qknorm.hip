@@ -156,7 +156,8 @@ extern "C" size_t kr_qk_norm_bwd_workspace_bytes(int64_t tokens, int ng, int per
 
 extern "C" int kr_qk_norm_fwd(const void* mixed, const void* gamma_q, const void* gamma_k, void* out, float* rstd,
                               int64_t tokens, int ng, int per, int hd, float eps, void* stream) {
-  if (!mixed || !gamma_q || !gamma_k || !out || !rstd || !qk_shape_ok(tokens, ng, per)) return KR_EINVAL;
+  if (!mixed || !gamma_q || !gamma_k || !out || !rstd || out == mixed || !qk_shape_ok(tokens, ng, per))
+    return KR_EINVAL;
   if (hd != 64 && hd != 128 && hd != 256) return KR_EUNSUPPORTED;
   if (!kr_aligned16(mixed) || !kr_aligned16(gamma_q) || !kr_aligned16(gamma_k) || !kr_aligned16(out))
     return KR_EINVAL;

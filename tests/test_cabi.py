@@ -46,9 +46,10 @@ def test_argument_checks_run_without_a_device():
     assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 12, 4, 64, 0.1, 1, 0, None) == -1  # mask not 8-byte aligned
     assert lib.kr_dropout_add(16, 64, 16, 64, 16, 64, 8, 4, 60, 0.1, 1, 0, None) == -2   # width not x8
     assert lib.kr_dropout_bwd(16, 32, 8, 16, 64, 4, 64, 1.25, None) == -1                # gradient stride < width
-    assert lib.kr_qk_norm_fwd(16, 16, 16, 16, 16, 4, 2, 4, 96, 1e-5, None) == -2         # head dimension not 64/128/256
-    assert lib.kr_qk_norm_fwd(16, 16, 24, 16, 16, 4, 2, 4, 128, 1e-5, None) == -1        # misaligned weight
-    assert lib.kr_qk_norm_fwd(16, 16, 16, 16, 16, 4, 2, 0, 128, 1e-5, None) == -1        # no query head in a group
+    assert lib.kr_qk_norm_fwd(16, 32, 48, 64, 80, 4, 2, 4, 96, 1e-5, None) == -2         # head dimension not 64/128/256
+    assert lib.kr_qk_norm_fwd(16, 32, 40, 64, 80, 4, 2, 4, 128, 1e-5, None) == -1        # misaligned weight
+    assert lib.kr_qk_norm_fwd(16, 32, 48, 64, 80, 4, 2, 0, 128, 1e-5, None) == -1        # no query head in a group
+    assert lib.kr_qk_norm_fwd(16, 32, 48, 16, 64, 4, 2, 4, 128, 1e-5, None) == -1        # output on top of the input
     assert lib.kr_qk_norm_bwd(16, 16, 16, 16, 16, 16, 16, None, 4, 2, 4, 128, None) == -1  # no workspace
     assert lib.kr_qk_norm_bwd_workspace_bytes(4, 2, 4, 96) == 0
     # 8192 tokens x 2 groups x 6 heads of 128 channels: 16 rows per workgroup, capped at 1024 workgroups, each
