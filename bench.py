@@ -60,6 +60,11 @@ WORKLOADS = {
                label="Llama-3.1-8B layer, TP=4 shard, MBS 4 x seq 4096, 4 nanobatches"),
     "c5": dict(h=4096, nq=32, nkv=8, hd=128, ffn=14336, layers=4, b=2, s=8192, nnb=2,
                label="4-layer full-width Llama-3.1-8B stack, MBS 2 x seq 8192, 2 nanobatches"),
+    # not one of the benchmark configurations: the reference's second training configuration as shipped
+    # (tests/artifact/conf/megatron_qwen3_1.7b_config.yaml: q / k head norms, hidden dropout 0.1)
+    "qwen3": dict(h=2048, nq=2, nkv=1, hd=128, ffn=768, layers=1, b=8, s=4096, nnb=2, qk_layernorm=True,
+                  hidden_dropout=0.1,
+                  label="Qwen3-1.7B layer, TP=8 shard, MBS 8 x seq 4096, 2 nanobatches, q/k head norms, hidden dropout 0.1"),
 }
 
 
@@ -79,7 +84,8 @@ def make_model(w, nnb, device, use_streams=True, schedule=None, all_on_one_strea
 
     cfg = LayerConfig(hidden_size=w["h"], num_attention_heads=w["nq"], num_query_groups=w["nkv"],
                       kv_channels=w["hd"], ffn_hidden_size=w["ffn"], num_layers=w["layers"],
-                      num_nanobatches=nnb, backend="hip", use_streams=use_streams)
+                      num_nanobatches=nnb, backend="hip", use_streams=use_streams,
+                      **{k: w[k] for k in ("qk_layernorm", "hidden_dropout") if k in w})
     cfg.kareus_scheduler = schedule
     if all_on_one_stream and nnb > 1:
         cfg.nanobatch_streams = [torch.cuda.current_stream()] * nnb
@@ -722,6 +728,8 @@ def cpu_baseline(w, budget_s=25.0):
     dims = ref.LayerDims(w["h"], w["nq"], w["nkv"], w["hd"], w["ffn"])
     gen = torch.Generator().manual_seed(1234)
     params = [ref.init_layer_params(dims, gen)]
+    if w.get("qk_layernorm"):
+        params[0].update(q_norm=torch.ones(w["hd"]), k_norm=torch.ones(w["hd"]))
     x = torch.randn(s, 1, w["h"], generator=gen)
     go = torch.randn(s, 1, w["h"], generator=gen)
     freqs = ref.rope_table(s, w["hd"], dims.rope_base)

@@ -180,12 +180,13 @@ class HipBackend:
         one stride, ``t`` itself when it is a [s, r, cols] tensor whose rows come in runs; None when only a
         copy would do."""
         cols = t.shape[-1]
-        try:
+        # (whether the leading dimensions merge into one is read off the strides: asking ``view`` and catching
+        # its error costs 10 us per nanobatch slice that does not)
+        lead = [(n, st) for n, st in zip(t.shape[:-1], t.stride()[:-1]) if n != 1]
+        if all(a[1] == b[0] * b[1] for a, b in zip(lead, lead[1:])) and t.numel():
             m = t.view(-1, cols)
             if self._operand(m) is not None:
                 return m
-        except RuntimeError:
-            pass
         if t.dim() == 3 and self._operand(t) is not None:
             return t
         return None
