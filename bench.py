@@ -245,18 +245,18 @@ def partition_timeline(w, device, steps=24, wgrad_launches_at_end=None):
 # reports null.  A constant read off a profile, not something measured in this run: the entry
 # names the profile it came from, and it is only reported while the GEMM source is the one the
 # counters were read with (first 16 hex digits of its SHA-256).
-TRAFFIC_GEMM_SOURCE = "737c82ec2f2b537c"
+TRAFFIC_GEMM_SOURCE = "1a6828d98a39b5eb"
 MEASURED_TRAFFIC = {
     # (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000) x 1024, means over the launches of `bench.py --roofline-only`
     # one nanobatch of four (4096 tokens), what the default run launches; the weight gradient is one launch over
     # the operand pieces of all four nanobatches
-    ("TN", 4096, 7168, 4096): {"bytes": (180573.0 * 2.000 + 86016.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 4096, 4096, 7168): {"bytes": (172289.5 * 2.000 + 32768.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NT", 7168, 4096, 16384, "pieces"): {"bytes": (813203.0 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 4096, 7168, 4096): {"bytes": (180551.6 * 2.000 + 90074.8) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 4096, 4096, 7168): {"bytes": (172289.5 * 2.000 + 32769.4) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NT", 7168, 4096, 16384, "pieces"): {"bytes": (772842.6 * 2.000 + 57344.8) * 1024, "source": "profiles/gemm_fc1_c4.md"},
     # the whole microbatch as one nanobatch (16384 tokens, --nanobatches 1)
-    ("NT", 7168, 4096, 16384): {"bytes": (895807.3 * 2.000 + 57344.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("TN", 16384, 7168, 4096): {"bytes": (723643.7 * 2.000 + 344064.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
-    ("NN", 16384, 4096, 7168): {"bytes": (688398.5 * 2.000 + 131072.0) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NT", 7168, 4096, 16384): {"bytes": (839136.2 * 2.000 + 57344.9) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("TN", 16384, 7168, 4096): {"bytes": (721271.9 * 2.000 + 344090.9) * 1024, "source": "profiles/gemm_fc1_c4.md"},
+    ("NN", 16384, 4096, 7168): {"bytes": (688467.1 * 2.000 + 131076.5) * 1024, "source": "profiles/gemm_fc1_c4.md"},
 }
 
 

@@ -59,6 +59,15 @@ constexpr int kGroupM = 4;
 
 // ---- LDS layouts (element offsets inside one operand tile) ----------------------------------
 // K-major tile [256 rows][64]: 128-byte rows, 16-byte chunk index XORed with (row>>1)&7.
+// Output stores carry the non-temporal hint: nothing in the launch reads an output tile again.  Measured on
+// the 8B shard's layer at 16384 tokens: the out-projection forward 7 % shorter, the fc1 forward with its
+// SwiGLU epilogue 3-6 %, fc2's forward 2 %, the one-nanobatch step 1 %.  The bytes a launch fetches from
+// memory are the same with and without the hint (FETCH_SIZE), so the time is won on the store path, not on
+// operand re-reads; the same hint on other kernels' stores or on the epilogues' residual loads changed nothing.
+__device__ __forceinline__ void stg8_out(bf16* p, bf16x8 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p));
+}
+
 __device__ __forceinline__ int kmajor_off(int row, int chunk) {
   return row * BK + ((chunk ^ ((row >> 1) & 7)) << 3);
 }
@@ -673,7 +682,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
             const int rr = 4 * q + quad;
             const bf16x8 v = *(KR_LDS const bf16x8*)(buf + rr * 256 + ((rch ^ rr) << 4));
             const int n = n_wave + nt * 16 + rr;
-            if (tcols_in && n < N) stg8(C + (int64_t)n * ldc + m_wave + 8 * rch, v);
+            if (tcols_in && n < N) stg8_out(C + (int64_t)n * ldc + m_wave + 8 * rch, v);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -726,11 +735,11 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
                 d2[e] = (bf16)du;
               }
               if (in) {
-                stg8(C + blk + nlo[q], d1);
-                stg8(C + blk + nlo[q] + N, d2);
+                stg8_out(C + blk + nlo[q], d1);
+                stg8_out(C + blk + nlo[q] + N, d2);
               }
             } else {
-              if (in) stg8(C + blk + nlo[q], v);
+              if (in) stg8_out(C + blk + nlo[q], v);
             }
           }
           if constexpr (swiglu) {
@@ -749,7 +758,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
 #pragma unroll
               for (int e = 0; e < 8; ++e) y[e] = (bf16)kr_swiglu_f((float)g[e], (float)u[e]);
               if (ncols_in && (rows_in || m_wave + mt * 16 + rr < M))
-                stg8(out2 + (int64_t)(m_wave + mt * 16 + rr) * ld_out2 + out_n0 + 8 * rch, y);
+                stg8_out(out2 + (int64_t)(m_wave + mt * 16 + rr) * ld_out2 + out_n0 + 8 * rch, y);
             }
           }
         } else {
@@ -768,7 +777,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const bf16* __restrict__
               bf16x4 o;
 #pragma unroll
               for (int e = 0; e < 4; ++e) o[e] = (bf16)(v[e] + (float)oldc[mt & 1][q][e]);
-              if (in) *reinterpret_cast<bf16x4*>(C + blk + lo[q]) = o;
+              if (in) __builtin_nontemporal_store(o, reinterpret_cast<bf16x4*>(C + blk + lo[q]));
             }
           }
           wave_sync();
