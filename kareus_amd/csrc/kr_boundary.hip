@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kThreads) void xent_fwd_kernel(const bf16* __restri
   const int nvec = vocab / 8;
   float m = -INFINITY, l = 0.f;
   for (int v = threadIdx.x; v < nvec; v += kThreads) {
-    const bf16x8 p = ldg8(x + v * 8);
+    const bf16x8 p = ldg8_stream(x + v * 8);
     float f[8], cm = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void xent_bwd_kernel(const bf16* logits,
   const float shift = lse[row] * kLog2e;
   const int nvec = vocab / 8;
   for (int v = threadIdx.x; v < nvec; v += kThreads) {
-    const bf16x8 p = ldg8(x + v * 8);
+    const bf16x8 p = ldg8_stream(x + v * 8);
     bf16x8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kThreads) void xent_bwd_kernel(const bf16* logits,
       if (v * 8 + e == lab) prob -= 1.f;
       o[e] = (bf16)(prob * g);
     }
-    stg8(dx + v * 8, o);
+    stg8_stream(dx + v * 8, o);
   }
 }
 

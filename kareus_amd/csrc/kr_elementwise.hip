@@ -13,10 +13,10 @@ __global__ __launch_bounds__(kThreads) void add_kernel(const bf16* a, const bf16
                                                        int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * kThreads;
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
-    bf16x8 x = ldg8(a + i * 8), y = ldg8(b + i * 8), r;
+    bf16x8 x = ldg8_stream(a + i * 8), y = ldg8_stream(b + i * 8), r;
 #pragma unroll
     for (int e = 0; e < 8; ++e) r[e] = (bf16)((float)x[e] + (float)y[e]);
-    stg8(out + i * 8, r);
+    stg8_stream(out + i * 8, r);
   }
   // tail (n not a multiple of 8)
   if (blockIdx.x == 0) {
@@ -34,10 +34,10 @@ __global__ __launch_bounds__(kThreads) void add_rows_kernel(const bf16* a, int64
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
     const int64_t r = i / nv;
     const int c = (int)(i - r * nv) * 8;
-    bf16x8 x = ldg8(a + r * lda + c), y = ldg8(b + r * ldb + c), o;
+    bf16x8 x = ldg8_stream(a + r * lda + c), y = ldg8_stream(b + r * ldb + c), o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)x[e] + (float)y[e]);
-    stg8(out + r * ldo + c, o);
+    stg8_stream(out + r * ldo + c, o);
   }
 }
 
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void dropout_add_kernel(const bf16* x, in
     const uint64_t index = offset + (uint64_t)i;  // one generator call per 8 elements
     uint32_t ctr[4] = {(uint32_t)index, (uint32_t)(index >> 32), 0u, 0u};
     philox4x32_10(ctr, (uint32_t)seed, (uint32_t)(seed >> 32));
-    const bf16x8 xv = ldg8(x + r * ldx + c), rv = ldg8(res + r * ldr + c);
+    const bf16x8 xv = ldg8_stream(x + r * ldx + c), rv = ldg8_stream(res + r * ldr + c);
     bf16x8 o;
     uint64_t m = 0;
 #pragma unroll
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void dropout_add_kernel(const bf16* x, in
       o[e] = (bf16)((float)rv[e] + (float)d);
       m |= (uint64_t)(keep ? 1 : 0) << (8 * e);
     }
-    stg8(out + r * ldo + c, o);
+    stg8_stream(out + r * ldo + c, o);
     *reinterpret_cast<uint64_t*>(mask + r * cols + c) = m;
   }
 }
@@ -100,12 +100,12 @@ __global__ __launch_bounds__(kThreads) void dropout_bwd_kernel(const bf16* dy, i
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
     const int64_t r = i / nv;
     const int c = (int)(i - r * nv) * 8;
-    const bf16x8 g = ldg8(dy + r * lddy + c);
+    const bf16x8 g = ldg8_stream(dy + r * lddy + c);
     const uint64_t m = *reinterpret_cast<const uint64_t*>(mask + r * cols + c);
     bf16x8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (bf16)(((m >> (8 * e)) & 1) ? (float)g[e] * scale : 0.f);
-    stg8(dx + r * lddx + c, o);
+    stg8_stream(dx + r * lddx + c, o);
   }
 }
 
@@ -122,13 +122,13 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const bf16* __rest
     const int64_t r = i / fv;
     const int c = (int)(i - r * fv) * 8;
     const bf16* xr = x + r * 2 * F;
-    bf16x8 g = ldg8(xr + c), u = ldg8(xr + F + c), o;
+    bf16x8 g = ldg8_stream(xr + c), u = ldg8_stream(xr + F + c), o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float x1 = (float)g[e], x2 = (float)u[e];
       o[e] = (bf16)kr_swiglu_f(x1, x2);
     }
-    stg8(y + r * F + c, o);
+    stg8_stream(y + r * F + c, o);
   }
 }
 
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16* __rest
     const int64_t r = i / fv;
     const int c = (int)(i - r * fv) * 8;
     const bf16* xr = x + r * 2 * F;
-    bf16x8 g = ldg8(xr + c), u = ldg8(xr + F + c), d = ldg8(dy + r * F + c), d1, d2;
+    bf16x8 g = ldg8_stream(xr + c), u = ldg8_stream(xr + F + c), d = ldg8_stream(dy + r * F + c), d1, d2;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float dg, du;
@@ -151,8 +151,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const bf16* __rest
       d1[e] = (bf16)dg;
       d2[e] = (bf16)du;
     }
-    stg8(dx + r * 2 * F + c, d1);
-    stg8(dx + r * 2 * F + F + c, d2);
+    stg8_stream(dx + r * 2 * F + c, d1);
+    stg8_stream(dx + r * 2 * F + F + c, d2);
   }
 }
 

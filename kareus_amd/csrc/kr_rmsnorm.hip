@@ -128,12 +128,12 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int v = v0 + c * 64;
-      xv[c] = (active && (FULL || v < nvec)) ? ldg8(xr + v * 8) : zero8();
-      dv[c] = (active && (FULL || v < nvec)) ? ldg8(dr + v * 8) : zero8();
+      xv[c] = (active && (FULL || v < nvec)) ? ldg8_stream(xr + v * 8) : zero8();
+      dv[c] = (active && (FULL || v < nvec)) ? ldg8_stream(dr + v * 8) : zero8();
     }
     if (ADD && FULL) {
 #pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) rv[c] = active ? ldg8(rr + (v0 + c * 64) * 8) : zero8();
+      for (int c = 0; c < NCHUNK; ++c) rv[c] = active ? ldg8_stream(rr + (v0 + c * 64) * 8) : zero8();
     }
     float dot = 0.f;
 #pragma unroll
@@ -159,14 +159,14 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(
       const int v = v0 + c * 64;
       if (active && (FULL || v < nvec)) {
         bf16x8 o, r;
-        if (ADD) r = FULL ? rv[c] : ldg8(rr + v * 8);
+        if (ADD) r = FULL ? rv[c] : ldg8_stream(rr + v * 8);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float xh = (float)xv[c][e] * rs;
           o[e] = (bf16)(rs * ((float)dv[c][e] * (float)g[c][e] - xh * dot));
           if (ADD) o[e] = (bf16)((float)o[e] + (float)r[e]);
         }
-        stg8(oxr + v * 8, o);
+        stg8_stream(oxr + v * 8, o);
       }
     }
   }
