@@ -117,6 +117,7 @@ def test_layer_with_hidden_dropout_matches_oracle_given_the_masks(dims, s, b):
     (R.LayerDims(2048, 4, 2, 128, 1536), 384, 4, 1),   # Qwen3-1.7B widths (16 q / 8 kv heads of 128) at TP=4
     (R.LayerDims(2048, 4, 2, 128, 1536), 384, 4, 2),
     (R.LayerDims(512, 8, 8, 64, 1376), 200, 2, 2),     # one query head per group, 64 channels, ragged length
+    (R.LayerDims(2048, 2, 1, 128, 768), 256, 8, 2),     # the TP=8 shard at MBS 8: nanobatches of four sequences, addressed in row runs
 ])
 def test_layer_with_query_and_key_norms_matches_oracle(dims, s, b, nnb):
     """Qwen3-style layers (qk_layernorm): an RMSNorm over the head dimension of every query head and of every
