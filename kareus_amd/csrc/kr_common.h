@@ -28,13 +28,13 @@ struct __attribute__((aligned(16))) Pack8 {
 __device__ __forceinline__ bf16x8 ldg8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ void stg8(bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
 // The same for data that streams through a kernel: operands it reads once and results it does not read
-// back, with the non-temporal hint.  Kernels that read two or three streams for each one they write move
-// 10-17 % more bytes per second with it at 16384 tokens of the 8B shard (residual add 5.2 -> 6.1 TB/s, RMSNorm
-// backward with the residual gradient 5.1 -> 6.0, SwiGLU 5.4 -> 6.1, dropout 5.2 -> 6.2); at 4096 tokens,
-// where a benchmark loop finds its operands in the memory-side cache, it makes no difference or costs a few
-// per cent.  Kernels that read one stream and write one got slower with it on either side (RMSNorm forward
-// 7-10 %, the per-head norm 39 %), as did loads that lanes or workgroups share (norm weights, rotary
-// angles): those keep the default policy.
+// back, with the non-temporal hint.  Results stored with it: every kernel that writes a tensor it did not read
+// (RMSNorm forward 42.9 -> 40.7 us at 16384 tokens of the 8B shard, 12.6 -> 10.6 us at 4096).  Operands loaded
+// with it: only where a kernel reads two or three streams for each one it writes (residual add 5.2 -> 6.1 TB/s,
+// RMSNorm backward with the residual gradient 5.1 -> 6.0, SwiGLU 5.4 -> 6.1, dropout 5.2 -> 6.2, 10-17 % less
+// time at 16384 tokens); kernels that read one stream got 7-39 % slower with the hint on their loads, kernels
+// that rewrite what they read (rotary, the per-head norm's backward) gained nothing either way, and loads that
+// lanes or workgroups share (norm weights, rotary angles) keep the default policy.
 __device__ __forceinline__ bf16x8 ldg8_stream(const bf16* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
 }

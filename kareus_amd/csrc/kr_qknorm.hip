@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_fwd_kernel(const bf16* __res
     const int j = (int)(r % (per + 2));
     const bf16x8 x = ldg8(mixed + r * HD + sub * 8);
     if (j == per + 1) {  // a value head: carried along
-      stg8(out + r * HD + sub * 8, x);
+      stg8_stream(out + r * HD + sub * 8, x);
       continue;          // (all lanes of a row take the same branch)
     }
     float ss = 0.f;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_fwd_kernel(const bf16* __res
     bf16x8 y;
 #pragma unroll
     for (int e = 0; e < 8; ++e) y[e] = (bf16)((float)x[e] * rs * (float)g[e]);
-    stg8(out + r * HD + sub * 8, y);
+    stg8_stream(out + r * HD + sub * 8, y);
     if (sub == 0) rstd[(r / (per + 2)) * (per + 1) + j] = rs;
   }
 }

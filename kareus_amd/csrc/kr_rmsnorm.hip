@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const bf16* __res
         bf16x8 o;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = (bf16)(((float)xv[c][e] * rs) * (float)g[c][e]);
-        stg8(yr + v * 8, o);
+        stg8_stream(yr + v * 8, o);
       }
     }
   }
