@@ -33,6 +33,7 @@ from .operators import (
     TERowParallelLinearOp,
     rotary_frequencies,
 )
+from .partitions.op_context import operator_parameters
 from .partitions.streams import stream_api
 from .partitions import (
     CommunicationType,
@@ -335,7 +336,7 @@ class LayerStack(torch.nn.Module):
         params: List[torch.nn.Parameter] = []
         for layer in self.layers:
             for op in layer.get_all_operators():
-                params.extend(op.parameters())
+                params.extend(operator_parameters(op))
         return params
 
     def rotary_pos_emb(self, seq_len: int, device=None) -> torch.Tensor:

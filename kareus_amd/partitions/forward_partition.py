@@ -13,6 +13,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 from .context_manager import NanoBatchContext
+from .op_context import operator_parameters
 from .partition_base import PartitionBase, _current_stream
 
 
@@ -57,7 +58,7 @@ class ForwardPartition(PartitionBase):
 
             needs_grad = self.is_grad_enabled and (
                 any(store.needs_grad(t) for t in in_ids)
-                or any(p.requires_grad for member in group for p in member.operator.parameters())
+                or any(p.requires_grad for member in group for p in operator_parameters(member.operator))
             )
             group_ctxs = []
             for member in group:
