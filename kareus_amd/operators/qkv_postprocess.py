@@ -46,6 +46,8 @@ class QKVPostProcessOp(BasicOperation, PartitionableOperator):
         for norm in (q_layernorm, k_layernorm):
             if norm is None:
                 continue
+            if getattr(norm, "bias", None) is not None or isinstance(norm, torch.nn.LayerNorm):
+                raise NotImplementedError("q/k layernorm: only an RMSNorm (no mean subtraction, no bias) is supported")
             weight = getattr(norm, "weight", None)
             if weight is None or tuple(weight.shape) != (hidden_size_per_attention_head,) or not hasattr(norm, "eps"):
                 raise ValueError("q/k layernorm must be an RMSNorm over the head dimension "

@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from kareus_amd import LayerConfig, LayerStack
-from kareus_amd.operators import NoOpAllReduce, QKVPostProcessOp
+from kareus_amd.operators import NoOpAllReduce, QKVPostProcessOp, RMSNorm
 from kareus_amd.partitions import NanoBatchContext, TensorStore, TransformerBlockAutogradFunction
 from kareus_amd.partitions.autograd_function import _flatten_grad_params
 from kareus_amd.partitions.partition_base import PartitionBase
@@ -409,8 +409,10 @@ def test_host_error_paths():
         LayerStack(LayerConfig(**C1, add_bias_linear=True, params_dtype=torch.float32, backend="eager"))
     with pytest.raises(NotImplementedError, match="come as a pair"):
         QKVPostProcessOp(2, 6, 16, q_layernorm=torch.nn.LayerNorm(16))
+    with pytest.raises(NotImplementedError, match="only an RMSNorm"):
+        QKVPostProcessOp(2, 6, 16, q_layernorm=torch.nn.LayerNorm(16), k_layernorm=torch.nn.LayerNorm(16))
     with pytest.raises(ValueError, match="over the head dimension"):
-        QKVPostProcessOp(2, 6, 16, q_layernorm=torch.nn.LayerNorm(32), k_layernorm=torch.nn.LayerNorm(32))
+        QKVPostProcessOp(2, 6, 16, q_layernorm=RMSNorm(32, backend="eager"), k_layernorm=RMSNorm(32, backend="eager"))
     with pytest.raises(NotImplementedError):
         NoOpAllReduce(world_size=2)
     with pytest.raises(ValueError, match="unknown backend"):
